@@ -1,0 +1,239 @@
+"""A plain, slow Mistral: whole sequences, no cache, one function for each part.
+
+Written from the formulas of the reference (paths are relative to the
+reference's root).  It shares no code with the engine: it takes a dict of
+tensors by their checkpoint names and a dict of the config.json keys, and
+works on the CPU in the dtype it is asked for (float64 by default, so that
+it can serve as ground truth for the engine's float32 path).
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+
+def embedding(table: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
+    """Row copy, no scaling.  src/model/modules/embedding.rs:15-21"""
+    return table[ids.long()]
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """x / sqrt(mean(x^2) + eps) * w; eps inside the root, weight used as it
+    is.  src/kernels/mod.rs:558-568"""
+    ss = (x * x).sum(dim=-1, keepdim=True)
+    rms = torch.sqrt(ss / x.shape[-1] + eps)
+    return (x / rms) * weight
+
+
+def linear(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """out[r] = sum_c W[r, c] x[c], no bias.  src/loader/parameters.rs:551-594"""
+    return x @ w.t()
+
+
+def rope_inv_freq(head_dim: int, theta: float, dtype=torch.float64) -> torch.Tensor:
+    """inv_freq[i] = 1 / theta^(i / (d/2)).  src/kernels/mod.rs:572-579"""
+    half = head_dim // 2
+    i = torch.arange(half, dtype=dtype)
+    return 1.0 / torch.pow(torch.tensor(theta, dtype=dtype), i / half)
+
+
+def rope(x: torch.Tensor, positions: torch.Tensor, theta: float) -> torch.Tensor:
+    """Half-split rotation of x[T, heads, d] by the angle pos * inv_freq:
+    x'_i = x_i c_i - x_{i+d/2} s_i ; x'_{i+d/2} = x_i s_i + x_{i+d/2} c_i.
+    src/kernels/mod.rs:582-608"""
+    d = x.shape[-1]
+    half = d // 2
+    inv = rope_inv_freq(d, theta, x.dtype)
+    ang = positions.to(x.dtype)[:, None] * inv[None, :]          # [T, d/2]
+    c = torch.cos(ang)[:, None, :]
+    s = torch.sin(ang)[:, None, :]
+    a, b = x[..., :half], x[..., half:]
+    return torch.cat([a * c - b * s, a * s + b * c], dim=-1)
+
+
+def visible(positions: torch.Tensor, window) -> torch.Tensor:
+    """mask[p, j]: key j visible to the query at p iff j <= p, and with a
+    window W, not (p >= W and j < p - W + 1).  Causality:
+    src/model/modules/attention.rs:90 ; window: src/model/models/gpt_oss.rs:168-175"""
+    p = positions[:, None]
+    j = positions[None, :]
+    m = j <= p
+    if window:
+        m &= ~((p >= window) & (j < p - window + 1))
+    return m
+
+
+def softmax(s: torch.Tensor) -> torch.Tensor:
+    """exp(s - max) / sum.  src/kernels/mod.rs:538-543"""
+    m = s.max(dim=-1, keepdim=True).values
+    e = torch.exp(s - m)
+    return e / e.sum(dim=-1, keepdim=True)
+
+
+def attention_core(q, k, v, positions, window) -> torch.Tensor:
+    """q[T,nq,d], k,v[T,nkv,d] (already rotated) -> ctx[T,nq,d].
+    Query head h reads KV head h // (nq/nkv); score = (k.q) * 1/sqrt(d),
+    scale applied after the dot; softmax over the visible keys; weighted sum
+    of the value rows.  src/model/modules/attention.rs:82-121 ;
+    src/kernels/mod.rs:494-526"""
+    T, nq, d = q.shape
+    nkv = k.shape[1]
+    g = nq // nkv
+    scale = 1.0 / math.sqrt(d)
+    mask = visible(positions, window)
+    out = torch.empty_like(q)
+    for h in range(nq):
+        kvh = h // g
+        s = (q[:, h, :] @ k[:, kvh, :].t()) * scale               # [T, T]
+        s = s.masked_fill(~mask, float("-inf"))
+        p = softmax(s)
+        out[:, h, :] = p @ v[:, kvh, :]
+    return out
+
+
+def attention(x, w, prefix, cfg, positions) -> torch.Tensor:
+    """Projections, rotation of q and k, attention, output projection.
+    src/model/modules/attention.rs:42-135"""
+    nq = cfg["num_attention_heads"]
+    nkv = cfg.get("num_key_value_heads") or nq
+    d = cfg.get("head_dim") or cfg["hidden_size"] // nq
+    T = x.shape[0]
+    q = linear(x, w[prefix + "self_attn.q_proj.weight"]).view(T, nq, d)
+    k = linear(x, w[prefix + "self_attn.k_proj.weight"]).view(T, nkv, d)
+    v = linear(x, w[prefix + "self_attn.v_proj.weight"]).view(T, nkv, d)
+    theta = cfg.get("rope_theta", 10000.0)
+    q = rope(q, positions, theta)
+    k = rope(k, positions, theta)
+    ctx = attention_core(q, k, v, positions, cfg.get("sliding_window"))
+    return linear(ctx.reshape(T, nq * d), w[prefix + "self_attn.o_proj.weight"])
+
+
+def silu(x: torch.Tensor) -> torch.Tensor:
+    """x / (1 + exp(-x)).  src/kernels/mod.rs:546-548"""
+    return x / (1.0 + torch.exp(-x))
+
+
+def swiglu(x, w, prefix) -> torch.Tensor:
+    """down( silu(gate x) * (up x) ).  src/model/modules/mlp.rs:23-45"""
+    g = linear(x, w[prefix + "mlp.gate_proj.weight"])
+    u = linear(x, w[prefix + "mlp.up_proj.weight"])
+    return linear(silu(g) * u, w[prefix + "mlp.down_proj.weight"])
+
+
+def block(x, w, prefix, cfg, positions) -> torch.Tensor:
+    """x + attn(norm1(x)), then x + mlp(norm2(x)).
+    src/model/modules/layer.rs:28-56"""
+    eps = cfg["rms_norm_eps"]
+    x = x + attention(rmsnorm(x, w[prefix + "input_layernorm.weight"], eps),
+                      w, prefix, cfg, positions)
+    x = x + swiglu(rmsnorm(x, w[prefix + "post_attention_layernorm.weight"], eps),
+                   w, prefix)
+    return x
+
+
+def forward(weights: dict, cfg: dict, ids, dtype=torch.float64) -> torch.Tensor:
+    """Logits [T, V] of one whole sequence.  src/model/mod.rs:430-447"""
+    w = {k: v.to(dtype) for k, v in weights.items()}
+    ids = torch.as_tensor(ids)
+    T = ids.shape[0]
+    positions = torch.arange(T)
+    x = embedding(w["model.embed_tokens.weight"], ids)
+    for i in range(cfg["num_hidden_layers"]):
+        x = block(x, w, f"model.layers.{i}.", cfg, positions)
+    x = rmsnorm(x, w["model.norm.weight"], cfg["rms_norm_eps"])
+    head = "model.embed_tokens.weight" if cfg.get("tie_word_embeddings") else "lm_head.weight"
+    return linear(x, w[head])
+
+
+# --- sampling --------------------------------------------------------------
+
+def greedy(logits: torch.Tensor) -> int:
+    """Index of the largest logit; of equal maxima the last, as Rust's
+    `max_by` keeps it.  src/sampler/mod.rs:60-68"""
+    best, idx = None, 0
+    for i, v in enumerate(logits.tolist()):
+        if best is None or v >= best:
+            best, idx = v, i
+    return idx
+
+
+def top_k_filter(z: torch.Tensor, k: int) -> torch.Tensor:
+    """Keep the k largest, others to -inf; ties at the threshold are kept in
+    index order until k are kept.  src/sampler/mod.rs:93-119"""
+    z = z.clone()
+    thr = torch.sort(z, descending=True).values[min(k, z.numel()) - 1]
+    if int((z >= thr).sum()) <= k:
+        z[z < thr] = float("-inf")
+        return z
+    kept = 0
+    for i in range(z.numel()):
+        if z[i] >= thr and kept < k:
+            kept += 1
+        else:
+            z[i] = float("-inf")
+    return z
+
+
+def top_p_filter(p: torch.Tensor, top_p: float) -> torch.Tensor:
+    """Sort descending, keep the shortest prefix whose sum is >= top_p, zero the
+    rest, divide by the new sum.  src/sampler/mod.rs:144-170"""
+    p = p.clone()
+    order = torch.argsort(p, descending=True, stable=True)
+    cum, cutoff = 0.0, p.numel()
+    for n, i in enumerate(order.tolist()):
+        cum += float(p[i])
+        if cum >= top_p:
+            cutoff = n + 1
+            break
+    p[order[cutoff:]] = 0.0
+    s = p.sum()
+    if s > 0:
+        p = p / s
+    return p
+
+
+def sample_distribution(logits, temperature, top_k=None, top_p=None) -> torch.Tensor:
+    """Probabilities that the draw is made from: temperature, top-k, softmax,
+    top-p, in this order.  src/sampler/mod.rs:194-222"""
+    z = logits.to(torch.float64) / temperature
+    if top_k is not None and 0 < top_k < z.numel():
+        z = top_k_filter(z, top_k)
+    p = softmax(z)
+    if top_p is not None and 0.0 < top_p < 1.0:
+        p = top_p_filter(p, top_p)
+    return p
+
+
+def draw(p: torch.Tensor, r: float) -> int:
+    """First index whose running sum reaches r, else the last index.
+    src/sampler/mod.rs:225-238"""
+    cum = 0.0
+    for i, v in enumerate(p.tolist()):
+        cum += v
+        if cum >= r:
+            return i
+    return p.numel() - 1
+
+
+def sample(logits, r, temperature, top_k=None, top_p=None) -> int:
+    """src/sampler/mod.rs:194-222"""
+    if temperature <= 0.0:
+        return greedy(logits)
+    return draw(sample_distribution(logits, temperature, top_k, top_p), r)
+
+
+def generate_greedy(weights, cfg, prompt, max_tokens, stop_ids=(), dtype=torch.float64):
+    """Feed the prompt, then the argmax of the last row again and again; a stop
+    id ends the sequence and is not part of the output.
+    src/sampler/mod.rs:269-305 ; src/main.rs:557-597"""
+    ids = list(prompt)
+    out = []
+    for _ in range(max_tokens):
+        logits = forward(weights, cfg, ids, dtype)[-1]
+        t = greedy(logits)
+        if t in stop_ids:
+            return out, "stop"
+        out.append(t)
+        ids.append(t)
+    return out, "length"

@@ -1,0 +1,87 @@
+// Shared helpers of the gfx950 kernels: element types, loads that widen to
+// float, wave and block reductions, and the error channel of the C interface.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+namespace tl {
+
+typedef __bf16 bf16;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+constexpr int WAVE = 64;
+constexpr int PAGE = 64;          // positions per cache page
+
+// dtype codes of the C interface
+constexpr int DT_F32 = 0;
+constexpr int DT_BF16 = 1;
+
+__device__ __forceinline__ float to_f32(float v) { return v; }
+__device__ __forceinline__ float to_f32(bf16 v) { return (float)v; }
+
+template <typename T> __device__ __forceinline__ T from_f32(float v);
+template <> __device__ __forceinline__ float from_f32<float>(float v) { return v; }
+template <> __device__ __forceinline__ bf16 from_f32<bf16>(float v) { return (bf16)v; }  // nearest even
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = WAVE / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, WAVE));
+  return v;
+}
+
+// Sum over a block of NT threads (NT a multiple of 64, at most 1024); every
+// thread gets the result.  `sh` holds at least NT/64 floats.
+template <int NT> __device__ __forceinline__ float block_sum(float v, float* sh) {
+  v = wave_sum(v);
+  const int w = threadIdx.x / WAVE, l = threadIdx.x % WAVE;
+  __syncthreads();
+  if (l == 0) sh[w] = v;
+  __syncthreads();
+  float r = 0.f;
+#pragma unroll
+  for (int i = 0; i < NT / WAVE; ++i) r += sh[i];
+  return r;
+}
+template <int NT> __device__ __forceinline__ float block_max(float v, float* sh) {
+  v = wave_max(v);
+  const int w = threadIdx.x / WAVE, l = threadIdx.x % WAVE;
+  __syncthreads();
+  if (l == 0) sh[w] = v;
+  __syncthreads();
+  float r = sh[0];
+#pragma unroll
+  for (int i = 1; i < NT / WAVE; ++i) r = fmaxf(r, sh[i]);
+  return r;
+}
+
+// ---- error channel -------------------------------------------------------
+void set_error(const char* fmt, ...);
+
+#define TL_REQUIRE(cond, ...)            \
+  do {                                   \
+    if (!(cond)) {                       \
+      tl::set_error(__VA_ARGS__);        \
+      return 1;                          \
+    }                                    \
+  } while (0)
+
+#define TL_LAUNCH_CHECK(name)                                              \
+  do {                                                                     \
+    hipError_t e_ = hipGetLastError();                                     \
+    if (e_ != hipSuccess) {                                                \
+      tl::set_error("%s: launch failed: %s", name, hipGetErrorString(e_)); \
+      return 2;                                                            \
+    }                                                                      \
+  } while (0)
+
+}  // namespace tl

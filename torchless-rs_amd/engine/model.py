@@ -1,0 +1,120 @@
+"""A model put together from a `ModelSpec`: parts built, weights bound, runs of
+the schedule tied to their places in the cache.
+
+The reference's `Mistral::load` binds tensors by hard-coded names and its
+`forward` walks embedding, layers, norm and head for one token
+(src/model/mod.rs:354-447).  Here the same walk goes over the rows of a whole
+step, and which parts it meets is data.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from ..cache.cache import Cache, KVRequest, StateRequest
+from ..config.base import ModelConfig
+from ..parts.base import ModelSpec, PartSpec, RunBinding, StepContext, make_part
+from ..weights.binding import bind_weights
+
+
+class Model:
+    def __init__(self, spec: ModelSpec, config: Optional[ModelConfig], dtype: torch.dtype, device):
+        if dtype not in (torch.float32, torch.bfloat16):
+            raise ValueError(f"compute dtype must be float32 or bfloat16, got {dtype}")
+        self.spec = spec
+        self.config = config
+        self.dtype = dtype
+        self.device = torch.device(device)
+        self.embedding = make_part("embedding", spec.embedding)
+        self.blocks = [make_part("block", PartSpec(ls.block.kind, dict(ls.block.params, layer=ls)))
+                       for ls in spec.layers]
+        self.final_norm = make_part("norm", spec.final_norm)
+        self.head = make_part("head", spec.head)
+        for i, run in enumerate(spec.schedule):
+            if not (0 <= run.layer < len(self.blocks)):
+                raise ValueError(f"schedule entry {i} names layer {run.layer}, there are "
+                                 f"{len(self.blocks)}")
+            if run.kv_from is not None and not (0 <= run.kv_from < i):
+                raise ValueError(f"schedule entry {i} reads the cache of entry {run.kv_from}, which "
+                                 "is not an earlier one")
+        self.runs: List[RunBinding] = []
+        self.loaded = False
+
+    # ---- weights -----------------------------------------------------------
+    def load_weights(self, source) -> None:
+        """`source`: anything with names/shape/dtype/tensor (a model folder's
+        files, or tensors in memory)."""
+        spec = self.spec
+        t = bind_weights(spec.weight_specs(), source, self.dtype, self.device, spec.ignore_tensors)
+
+        def sub(prefix: str) -> Dict[str, torch.Tensor]:
+            return {k[len(prefix):]: v for k, v in t.items() if k.startswith(prefix)}
+
+        self.embedding.load(sub(spec.embedding_prefix), self.dtype)
+        for ls, blk in zip(spec.layers, self.blocks):
+            blk.load(sub(ls.prefix), self.dtype)
+        self.final_norm.load(sub(spec.final_norm_prefix), self.dtype)
+        head_t = sub(spec.head_prefix)
+        head_t["__embedding__"] = getattr(self.embedding, "table", None)
+        self.head.load(head_t, self.dtype)
+        self.loaded = True
+
+    # ---- cache ---------------------------------------------------------------
+    def cache_requests(self):
+        kv: Dict[int, KVRequest] = {}
+        st: Dict[int, StateRequest] = {}
+        for i, run in enumerate(self.spec.schedule):
+            mixer = self.blocks[run.layer].mixer
+            if run.kv_from is None:
+                r = mixer.kv_request()
+                if r is not None:
+                    kv[i] = r
+            s = mixer.state_request()
+            if s is not None:
+                st[i] = s
+        return kv, st
+
+    def make_cache(self, max_tokens: int, max_slots: Optional[int] = None, allocate: bool = True) -> Cache:
+        kv, st = self.cache_requests()
+        cache = Cache(kv, st, max_tokens, self.dtype, self.device, max_slots, allocate)
+        self.bind_cache(cache)
+        return cache
+
+    def bind_cache(self, cache: Cache) -> None:
+        read_later = {r.kv_from for r in self.spec.schedule if r.kv_from is not None}
+        self.runs = []
+        for i, run in enumerate(self.spec.schedule):
+            src = i if run.kv_from is None else run.kv_from
+            b = RunBinding(index=i, kv_owner=run.kv_from is None, kv_source=src,
+                           kv_read_later=i in read_later, state=cache.state.get(i))
+            if src in cache.group_of_run:
+                b.kv_group_index = cache.group_of_run[src]
+                b.kv_group, b.kv_layer = cache.kv_layer(src)
+            elif run.kv_from is not None:
+                raise ValueError(f"schedule entry {i} reads the cache of entry {src}, which keeps none")
+            self.runs.append(b)
+
+    # ---- one step ------------------------------------------------------------
+    def forward(self, ctx: StepContext, want_rows: Optional[torch.Tensor], n_want: int) -> torch.Tensor:
+        """Run the rows of `ctx` through the schedule and return float32 logits
+        [n_want, V] at `want_rows` (int32 row indices on the device)."""
+        if not self.loaded:
+            raise RuntimeError("the model has no weights yet")
+        H, V = self.spec.hidden_size, self.spec.vocab_size
+        ws = ctx.workspace
+        x = ws.get("residual", (ctx.n_rows, H), torch.float32)
+        self.embedding.forward(ctx, ctx.tokens, x)
+        for run, binding in zip(self.spec.schedule, self.runs):
+            self.blocks[run.layer].forward(ctx, binding, x)
+        for commit in ctx.host.pop("deferred", []):
+            commit()
+        logits = ws.get("logits", (n_want, V), torch.float32)
+        if n_want:
+            xs = ws.get("head_x", (n_want, H), torch.float32)
+            from ..kernels import ops
+            ops.gather_rows(x, want_rows, xs)
+            y = ws.get("head_y", (n_want, H), ctx.dtype)
+            self.final_norm.forward(ctx, xs, y)
+            self.head.forward(ctx, y, logits)
+        return logits

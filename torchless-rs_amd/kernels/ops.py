@@ -1,0 +1,203 @@
+"""Python faces of the HIP kernels.
+
+Every function checks on the host that its operands are on the GPU,
+contiguous, of the type and shape that the kernel and its grid assume, and
+launches on torch's current stream.  A failure of the launcher raises
+`KernelError` with the library's message.  There is no fallback: without the
+library nothing here runs.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from .build import load
+
+DT_F32, DT_BF16 = 0, 1
+_CODES = {torch.float32: DT_F32, torch.bfloat16: DT_BF16}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+_configured = False
+
+
+def lib() -> ctypes.CDLL:
+    global _configured
+    L = load()
+    if not _configured:
+        L.tl_last_error.restype = ctypes.c_char_p
+        _configured = True
+    return L
+
+
+def _check(rc: int) -> None:
+    if rc != 0:
+        raise KernelError(lib().tl_last_error().decode())
+
+
+def _code(dt: torch.dtype) -> int:
+    if dt not in _CODES:
+        raise KernelError(f"dtype {dt} is not served by the kernels (float32 and bfloat16 are)")
+    return _CODES[dt]
+
+
+def _p(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _stream() -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _req(t: torch.Tensor, name: str, dtype=None, shape=None) -> None:
+    if not t.is_cuda:
+        raise KernelError(f"{name}: must be on the GPU")
+    if not t.is_contiguous():
+        raise KernelError(f"{name}: must be contiguous")
+    if dtype is not None and t.dtype != dtype:
+        raise KernelError(f"{name}: dtype {t.dtype}, kernel needs {dtype}")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise KernelError(f"{name}: shape {tuple(t.shape)}, kernel needs {tuple(shape)}")
+
+
+def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> None:
+    """out[n, :] = table[ids[n], :] widened to float32."""
+    n, H = ids.shape[0], table.shape[1]
+    _req(table, "embed.table")
+    _req(ids, "embed.ids", torch.int32, (n,))
+    _req(out, "embed.out", torch.float32, (n, H))
+    _check(lib().tl_embed(_p(table), _code(table.dtype), _p(ids), n, H, _p(out), _stream()))
+
+
+def rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float, out: torch.Tensor) -> None:
+    """out = x / sqrt(mean(x^2) + eps) * w, x float32 [n, H], w float32 [H]."""
+    n, H = x.shape
+    _req(x, "rmsnorm.x", torch.float32)
+    _req(w, "rmsnorm.w", torch.float32, (H,))
+    _req(out, "rmsnorm.out", None, (n, H))
+    _check(lib().tl_rmsnorm(_p(x), _p(w), ctypes.c_float(eps), _p(out), _code(out.dtype), n, H,
+                            _stream()))
+
+
+def rope_split(qkv: torch.Tensor, row_pos: torch.Tensor, inv_freq: torch.Tensor, nq: int, nkv: int,
+               d: int, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> None:
+    """Rotate q and k of the fused projection by their rows' positions and
+    write q [n,nq,d], k, v [n,nkv,d]."""
+    n = qkv.shape[0]
+    _req(qkv, "rope.qkv", torch.float32, (n, (nq + 2 * nkv) * d))
+    _req(row_pos, "rope.row_pos", torch.int32, (n,))
+    _req(inv_freq, "rope.inv_freq", torch.float32, (d // 2,))
+    _req(q, "rope.q", None, (n, nq, d))
+    if nkv:
+        _req(k, "rope.k", q.dtype, (n, nkv, d))
+        _req(v, "rope.v", q.dtype, (n, nkv, d))
+    _check(lib().tl_rope_split(_p(qkv), _p(row_pos), _p(inv_freq), n, nq, nkv, d, _p(q), _p(k), _p(v),
+                               _code(q.dtype), _stream()))
+
+
+def kv_commit(k: torch.Tensor, v: torch.Tensor, row_seq, row_pos, len_after, table: torch.Tensor,
+              ring_pages: int, pages: torch.Tensor) -> None:
+    """Write this step's keys and values into the pages of one layer.
+    pages: [n_pages, 2, nkv, PAGE, d]; table: [B, stride] page ids."""
+    n, nkv, d = k.shape
+    _req(k, "kv_commit.k", pages.dtype)
+    _req(v, "kv_commit.v", pages.dtype, (n, nkv, d))
+    _req(row_seq, "kv_commit.row_seq", torch.int32, (n,))
+    _req(row_pos, "kv_commit.row_pos", torch.int32, (n,))
+    _req(len_after, "kv_commit.len_after", torch.int32)
+    _req(table, "kv_commit.table", torch.int32)
+    _req(pages, "kv_commit.pages")
+    if pages.dim() != 5 or tuple(pages.shape[1:]) != (2, nkv, 64, d):
+        raise KernelError(f"kv_commit.pages: shape {tuple(pages.shape)}, kernel needs [*, 2, {nkv}, 64, {d}]")
+    if table.dim() != 2 or table.shape[0] != len_after.shape[0]:
+        raise KernelError("kv_commit.table: needs one row per sequence")
+    _check(lib().tl_kv_commit(_p(k), _p(v), _code(k.dtype), _p(row_seq), _p(row_pos), _p(len_after),
+                              _p(table), table.shape[1], ring_pages, n, nkv, d, _p(pages), _stream()))
+
+
+def attn_plain(q, k_new, v_new, pages, table, ring_pages: int, row_seq, row_pos, cu_seqlens, n_cached,
+               window: Optional[int], scale: float, out) -> None:
+    """Attention of every row over its sequence's cached keys (j < n_cached)
+    and this step's keys (k_new/v_new rows), causal, with an optional window."""
+    n, nq, d = q.shape
+    nkv = pages.shape[2]
+    B = n_cached.shape[0]
+    _req(q, "attn.q", pages.dtype)
+    if k_new is not None:
+        _req(k_new, "attn.k_new", pages.dtype, (n, nkv, d))
+        _req(v_new, "attn.v_new", pages.dtype, (n, nkv, d))
+    _req(pages, "attn.pages")
+    if pages.dim() != 5 or tuple(pages.shape[1:]) != (2, nkv, 64, d):
+        raise KernelError(f"attn.pages: shape {tuple(pages.shape)}, kernel needs [*, 2, nkv, 64, {d}]")
+    _req(table, "attn.table", torch.int32)
+    _req(row_seq, "attn.row_seq", torch.int32, (n,))
+    _req(row_pos, "attn.row_pos", torch.int32, (n,))
+    _req(cu_seqlens, "attn.cu_seqlens", torch.int32, (B + 1,))
+    _req(n_cached, "attn.n_cached", torch.int32, (B,))
+    _req(out, "attn.out", pages.dtype, (n, nq, d))
+    if table.dim() != 2 or table.shape[0] != B:
+        raise KernelError("attn.table: needs one row per sequence")
+    _check(lib().tl_attn_plain(_p(q), _p(k_new), _p(v_new), _p(pages), _code(q.dtype), _p(table),
+                               table.shape[1], ring_pages, _p(row_seq), _p(row_pos), _p(cu_seqlens),
+                               _p(n_cached), n, nq, nkv, d, int(window or 0), ctypes.c_float(scale),
+                               _p(out), _stream()))
+
+
+def silu_mul(gu: torch.Tensor, out: torch.Tensor) -> None:
+    """out[n, i] = silu(gu[n, i]) * gu[n, I + i]."""
+    n, I2 = gu.shape
+    _req(gu, "silu_mul.gu", torch.float32)
+    _req(out, "silu_mul.out", None, (n, I2 // 2))
+    _check(lib().tl_silu_mul(_p(gu), n, I2 // 2, _p(out), _code(out.dtype), _stream()))
+
+
+def gather_rows(x: torch.Tensor, idx: torch.Tensor, out: torch.Tensor) -> None:
+    m, H = idx.shape[0], x.shape[1]
+    _req(x, "gather.x", torch.float32)
+    _req(idx, "gather.idx", torch.int32, (m,))
+    _req(out, "gather.out", torch.float32, (m, H))
+    _check(lib().tl_gather_rows(_p(x), _p(idx), m, H, _p(out), _stream()))
+
+
+def gemm_plain(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
+    """out[M,N] (+)= a[M,K] @ w[N,K]^T, float32 accumulation in plain FMA."""
+    M, K = a.shape
+    N = w.shape[0]
+    _req(a, "gemm.a")
+    _req(w, "gemm.w", None, (N, K))
+    _req(out, "gemm.out", torch.float32, (M, N))
+    _check(lib().tl_gemm_plain(_p(a), _code(a.dtype), _p(w), _code(w.dtype), _p(out), M, N, K, K, K, N,
+                               int(accumulate), _stream()))
+
+
+def sample(logits: torch.Tensor, temperature: float, top_k: int, top_p: float, seed: int,
+           counters: torch.Tensor, probs: torch.Tensor, out: torch.Tensor) -> None:
+    """One token per row.  counters[b] = (sequence, step) feeds the generator;
+    probs receives the distribution the draw was made from (when T > 0)."""
+    B, V = logits.shape
+    _req(logits, "sample.logits", torch.float32)
+    _req(counters, "sample.counters", torch.int32, (B, 2))
+    _req(probs, "sample.probs", torch.float32, (B, V))
+    _req(out, "sample.out", torch.int32, (B,))
+    _check(lib().tl_sample(_p(logits), B, V, ctypes.c_float(temperature), int(top_k),
+                           ctypes.c_float(top_p), ctypes.c_ulonglong(seed & (2 ** 64 - 1)),
+                           _p(counters), _p(probs), _p(out), _stream()))
+
+
+def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
+    """out[M,N] (+)= a[M,K] @ w[N,K]^T with float32 accumulation.  The kernel
+    follows from the operand types and the number of rows."""
+    gemm_plain(a, w, out, accumulate)
+
+
+def attention(q, k_new, v_new, pages, table, ring_pages: int, ctx, n_cached, window, scale: float,
+              out) -> None:
+    """Attention of a step's rows (see `attn_plain` for the operands); `ctx`
+    brings the step's row and sequence indices."""
+    attn_plain(q, k_new, v_new, pages, table, ring_pages, ctx.row_seq, ctx.row_pos, ctx.cu_seqlens,
+               n_cached, window, scale, out)

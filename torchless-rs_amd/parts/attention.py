@@ -1,0 +1,112 @@
+"""Grouped-query attention over the cache, with an optional sliding window.
+
+q = Wq y, k = Wk y, v = Wv y (no bias); q and k rotated by the position
+encoding before k enters the cache; query head h reads KV head h // (nq/nkv);
+score = (k.q) / sqrt(d); softmax over the visible keys; output projection
+(src/model/modules/attention.rs:42-135 of the reference).  Key j is visible
+to the query at p iff j <= p and, with a window W, j > p - W
+(src/model/models/gpt_oss.rs:168-175; the reference's Mistral path reads the
+window from the file and never applies it).
+
+The three projections are bound under their own names and laid side by side
+at load so that one product serves them.  Rows of a step that bring more
+than one token attend to the cache for older positions and to the step's own
+keys for the new ones, and the keys are committed afterwards; single-token
+steps commit first and read everything from the cache.
+"""
+from __future__ import annotations
+
+import math
+from typing import Dict, Optional
+
+import torch
+
+from ..cache.cache import KVRequest
+from ..kernels import ops
+from ..weights.binding import WeightSpec
+from .base import Mixer, PartSpec, make_part, register_part
+from .linear import Linear
+
+
+class AttentionMixer(Mixer):
+    def __init__(self, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int,
+                 position: PartSpec, window: Optional[int] = None, own_kv: bool = True,
+                 prefix: str = "self_attn."):
+        if n_heads % n_kv_heads:
+            raise ValueError(f"attention: {n_heads} heads are not a multiple of {n_kv_heads} KV heads")
+        self.H, self.nq, self.nkv, self.d = int(hidden_size), int(n_heads), int(n_kv_heads), int(head_dim)
+        self.window = int(window) if window else None
+        self.own_kv = bool(own_kv)
+        self.prefix = prefix
+        self.position = make_part("position", position)
+        self.scale = 1.0 / math.sqrt(self.d)
+        self.qkv = None
+        self.o = None
+
+    def kv_request(self):
+        return KVRequest(self.nkv, self.d, self.window) if self.own_kv else None
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        p = self.prefix
+        out = {p + "q_proj.weight": WeightSpec((self.nq * self.d, self.H))}
+        if self.own_kv:
+            out[p + "k_proj.weight"] = WeightSpec((self.nkv * self.d, self.H))
+            out[p + "v_proj.weight"] = WeightSpec((self.nkv * self.d, self.H))
+        out[p + "o_proj.weight"] = WeightSpec((self.H, self.nq * self.d))
+        return out
+
+    def load(self, tensors, compute_dtype) -> None:
+        p = self.prefix
+        ws = [tensors[p + "q_proj.weight"]]
+        if self.own_kv:
+            ws += [tensors[p + "k_proj.weight"], tensors[p + "v_proj.weight"]]
+        if len({w.dtype for w in ws}) > 1:
+            ws = [w.to(torch.float32) for w in ws]
+        self.qkv = Linear(torch.cat(ws, dim=0))
+        self.o = Linear(tensors[p + "o_proj.weight"])
+
+    def forward(self, ctx, run, y: torch.Tensor, x: torch.Tensor) -> None:
+        n, nq, nkv, d = y.shape[0], self.nq, self.nkv, self.d
+        ws = ctx.workspace
+        group = run.kv_group
+        pages = group.storage[run.kv_layer]
+        table = ctx.tables[run.kv_group_index]
+        inv_freq = self.position.inv_freq(y.device)
+        q = ws.get("attn_q", (n, nq, d), ctx.dtype)
+        out = ws.get("attn_out", (n, nq, d), ctx.dtype)
+        if self.own_kv:
+            tag = f"_{run.index}" if run.kv_read_later else ""
+            qkv = ws.get("attn_qkv", (n, (nq + 2 * nkv) * d), torch.float32)
+            self.qkv(y, qkv)
+            k = ws.get("attn_k" + tag, (n, nkv, d), ctx.dtype)
+            v = ws.get("attn_v" + tag, (n, nkv, d), ctx.dtype)
+            ops.rope_split(qkv, ctx.row_pos, inv_freq, nq, nkv, d, q, k, v)
+            if run.kv_read_later:
+                ctx.host[f"kv_new_{run.index}"] = (k, v)
+        else:
+            qf = ws.get("attn_qkv", (n, nq * d), torch.float32)
+            self.qkv(y, qf)
+            ops.rope_split(qf, ctx.row_pos, inv_freq, nq, 0, d, q, None, None)
+            k, v = ctx.host[f"kv_new_{run.kv_source}"]
+        if ctx.all_single and not self.own_kv:
+            ops.attention(q, None, None, pages, table, group.ring_pages, ctx, ctx.len_after,
+                          self.window, self.scale, out)
+        elif ctx.all_single:
+            ops.kv_commit(k, v, ctx.row_seq, ctx.row_pos, ctx.len_after, table, group.ring_pages, pages)
+            ops.attention(q, None, None, pages, table, group.ring_pages, ctx, ctx.len_after,
+                          self.window, self.scale, out)
+        else:
+            ops.attention(q, k, v, pages, table, group.ring_pages, ctx, ctx.len_before,
+                          self.window, self.scale, out)
+            if self.own_kv:
+                def commit():
+                    ops.kv_commit(k, v, ctx.row_seq, ctx.row_pos, ctx.len_after, table,
+                                  group.ring_pages, pages)
+                if run.kv_read_later:       # a later run still reads the old rows of the ring
+                    ctx.host.setdefault("deferred", []).append(commit)
+                else:
+                    commit()
+        self.o(out.view(n, nq * d), x, accumulate=True)
+
+
+register_part("mixer", "attention", AttentionMixer)

@@ -1,0 +1,209 @@
+"""What a model is made of: parts, their registry, and the description of a
+model as data.
+
+A *part* is a mixer (attention, or anything else that mixes positions), a
+feed-forward, a norm, a position encoding, or a block that arranges them.
+Every part takes its sizes and constants as constructor parameters and knows
+nothing about the model it sits in.  A model is a `ModelSpec`: for each layer
+a `LayerSpec` naming the kind and parameters of its parts, and a schedule,
+the list of layer indices in the order in which they run.  A layer may be
+named twice (it then runs twice with the same weights and a cache of its own
+for each run), and a run may read the cache that an earlier run wrote.
+
+The reference hard-wires one arrangement (src/model/modules/layer.rs:28-56)
+and one mixer; its per-architecture switches live in `ArchitectureConfig`
+(src/model/architecture.rs:396-421, 487-502).  Here the switches are the
+parts themselves.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Callable, Dict, List, Optional, Tuple
+
+import torch
+
+from ..weights.binding import WeightSpec
+
+CATEGORIES = ("mixer", "ffn", "norm", "position", "block", "embedding", "head")
+_PARTS: Dict[str, Dict[str, type]] = {c: {} for c in CATEGORIES}
+
+
+def register_part(category: str, kind: str, cls: type) -> None:
+    if category not in _PARTS:
+        raise KeyError(f"unknown part category {category!r}; there are {CATEGORIES}")
+    _PARTS[category][kind] = cls
+
+
+def unregister_part(category: str, kind: str) -> None:
+    _PARTS[category].pop(kind, None)
+
+
+def registered_parts(category: str) -> List[str]:
+    return sorted(_PARTS[category])
+
+
+@dataclass
+class PartSpec:
+    """Kind (a name in the registry) and constructor parameters of one part."""
+    kind: str
+    params: Dict[str, Any] = field(default_factory=dict)
+
+
+def make_part(category: str, spec: PartSpec):
+    kinds = _PARTS[category]
+    if spec.kind not in kinds:
+        raise KeyError(f"no {category} of kind {spec.kind!r}; registered: {sorted(kinds)}")
+    return kinds[spec.kind](**spec.params)
+
+
+@dataclass
+class LayerSpec:
+    prefix: str                       # the layer's tensors are named prefix + local name
+    mixer: PartSpec
+    ffn: PartSpec
+    mixer_norm: PartSpec
+    ffn_norm: PartSpec
+    block: PartSpec = field(default_factory=lambda: PartSpec("pre_norm"))
+
+
+@dataclass
+class Run:
+    """One entry of the schedule: run `layer`; `kv_from`, if set, is the index
+    of an earlier entry whose cache this run reads instead of owning one."""
+    layer: int
+    kv_from: Optional[int] = None
+
+
+@dataclass
+class ModelSpec:
+    hidden_size: int
+    vocab_size: int
+    embedding: PartSpec
+    embedding_prefix: str
+    layers: List[LayerSpec]
+    schedule: List[Run]
+    final_norm: PartSpec
+    final_norm_prefix: str
+    head: PartSpec
+    head_prefix: str
+    ignore_tensors: Tuple[str, ...] = ()
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        """Every tensor name the model binds, in a fixed order."""
+        out: Dict[str, WeightSpec] = {}
+        for k, v in make_part("embedding", self.embedding).weight_specs().items():
+            out[self.embedding_prefix + k] = v
+        for ls in self.layers:
+            blk = make_part("block", PartSpec(ls.block.kind, dict(ls.block.params, layer=ls)))
+            for k, v in blk.weight_specs().items():
+                out[ls.prefix + k] = v
+        for k, v in make_part("norm", self.final_norm).weight_specs().items():
+            out[self.final_norm_prefix + k] = v
+        for k, v in make_part("head", self.head).weight_specs().items():
+            out.setdefault(self.head_prefix + k, v)
+        return out
+
+
+class Part:
+    """Base of all parts.  `weight_specs` names the tensors it binds (local
+    names); `load` receives them, already resident on the device in their
+    stored width, and `compute_dtype` (float32 or bfloat16)."""
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        return {}
+
+    def load(self, tensors: Dict[str, torch.Tensor], compute_dtype: torch.dtype) -> None:
+        pass
+
+
+class Norm(Part):
+    def forward(self, ctx: "StepContext", x: torch.Tensor, out: torch.Tensor) -> None:
+        """x: float32 [n, H] -> out [n, H] in the compute dtype."""
+        raise NotImplementedError
+
+
+class Position(Part):
+    pass
+
+
+class Mixer(Part):
+    """A part that mixes information between positions of a sequence."""
+
+    def kv_request(self):
+        """A `KVRequest` if the mixer keeps keys and values per position."""
+        return None
+
+    def state_request(self):
+        """A `StateRequest` if the mixer keeps a block of fixed size per sequence."""
+        return None
+
+    def forward(self, ctx: "StepContext", run: "RunBinding", y: torch.Tensor, x: torch.Tensor) -> None:
+        """y: normed input [n, H] (compute dtype); ADD the result to x (float32 [n, H])."""
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, ctx: "StepContext", y: torch.Tensor, x: torch.Tensor) -> None:
+        """y: normed input [n, H]; ADD the result to x (float32 [n, H])."""
+        raise NotImplementedError
+
+
+@dataclass
+class RunBinding:
+    """What one run of the schedule owns or reads in the cache."""
+    index: int
+    kv_group: Any = None          # cache.KVGroup
+    kv_group_index: int = -1
+    kv_layer: int = 0             # layer index inside the group's storage
+    kv_owner: bool = True         # False: reads another run's keys and values
+    kv_source: int = -1           # the run that owns them (its own index for an owner)
+    kv_read_later: bool = False   # a later run reads this run's keys and values
+    state: Optional[torch.Tensor] = None      # [max_slots, *shape]
+
+
+class Workspace:
+    """Scratch tensors by name, kept between steps so that a step allocates
+    nothing once sizes have been seen (and a captured graph keeps its
+    addresses)."""
+
+    def __init__(self, device):
+        self.device = device
+        self._bufs: Dict[str, torch.Tensor] = {}
+
+    def get(self, name: str, shape: Tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
+        n = 1
+        for s in shape:
+            n *= int(s)
+        key = f"{name}:{dtype}"
+        buf = self._bufs.get(key)
+        if buf is None or buf.numel() < n:
+            buf = torch.empty(max(n, 1), dtype=dtype, device=self.device)
+            self._bufs[key] = buf
+        return buf[:n].view(shape)
+
+    def clear(self) -> None:
+        self._bufs.clear()
+
+
+@dataclass
+class StepContext:
+    """One step's batch as the parts see it.  Rows are the tokens of all
+    sequences, packed sequence after sequence."""
+    n_rows: int
+    n_seqs: int
+    dtype: torch.dtype                    # compute dtype of activations and cache
+    device: Any
+    tokens: torch.Tensor                  # int32 [n]
+    row_pos: torch.Tensor                 # int32 [n]  position of the row in its sequence
+    row_seq: torch.Tensor                 # int32 [n]  index of the row's sequence in this batch
+    cu_seqlens: torch.Tensor              # int32 [B+1]
+    slots: torch.Tensor                   # int32 [B]
+    len_before: torch.Tensor              # int32 [B]
+    len_after: torch.Tensor               # int32 [B]
+    tables: Dict[int, torch.Tensor]       # group index -> int32 [B, stride] page ids
+    all_single: bool                      # every sequence brings exactly one token
+    max_new: int
+    max_len_after: int
+    workspace: Workspace
+    cache: Any
+    host: Dict[str, Any] = field(default_factory=dict)     # the same data on the host

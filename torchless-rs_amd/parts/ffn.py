@@ -1,0 +1,48 @@
+"""SwiGLU feed-forward: down( silu(gate y) * (up y) ), silu(g) = g / (1 + e^-g)
+(src/model/modules/mlp.rs:23-45, src/kernels/mod.rs:546-548 of the reference).
+gate and up are bound under their own names and laid side by side at load so
+that one product serves both."""
+from __future__ import annotations
+
+from typing import Dict
+
+import torch
+
+from ..kernels import ops
+from ..weights.binding import WeightSpec
+from .base import FeedForward, register_part
+from .linear import Linear
+
+
+class SwiGLU(FeedForward):
+    def __init__(self, hidden_size: int, intermediate_size: int, prefix: str = "mlp."):
+        self.H = int(hidden_size)
+        self.I = int(intermediate_size)
+        self.prefix = prefix
+        self.gate_up = None
+        self.down = None
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        p = self.prefix
+        return {p + "gate_proj.weight": WeightSpec((self.I, self.H)),
+                p + "up_proj.weight": WeightSpec((self.I, self.H)),
+                p + "down_proj.weight": WeightSpec((self.H, self.I))}
+
+    def load(self, tensors, compute_dtype) -> None:
+        p = self.prefix
+        g, u = tensors[p + "gate_proj.weight"], tensors[p + "up_proj.weight"]
+        if g.dtype != u.dtype:
+            g, u = g.to(torch.float32), u.to(torch.float32)
+        self.gate_up = Linear(torch.cat([g, u], dim=0))
+        self.down = Linear(tensors[p + "down_proj.weight"])
+
+    def forward(self, ctx, y: torch.Tensor, x: torch.Tensor) -> None:
+        n = y.shape[0]
+        gu = ctx.workspace.get("ffn_gu", (n, 2 * self.I), torch.float32)
+        self.gate_up(y, gu)
+        h = ctx.workspace.get("ffn_h", (n, self.I), ctx.dtype)
+        ops.silu_mul(gu, h)
+        self.down(h, x, accumulate=True)
+
+
+register_part("ffn", "swiglu", SwiGLU)

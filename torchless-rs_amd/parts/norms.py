@@ -1,0 +1,30 @@
+"""RMSNorm.  y = x / sqrt(mean(x^2) + eps) * w, in float32
+(src/kernels/mod.rs:558-568 of the reference; weight used as it is)."""
+from __future__ import annotations
+
+from typing import Dict
+
+import torch
+
+from ..kernels import ops
+from ..weights.binding import WeightSpec
+from .base import Norm, register_part
+
+
+class RMSNorm(Norm):
+    def __init__(self, size: int, eps: float):
+        self.size = int(size)
+        self.eps = float(eps)
+        self.weight = None
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        return {"weight": WeightSpec((self.size,), init="ones")}
+
+    def load(self, tensors, compute_dtype) -> None:
+        self.weight = tensors["weight"].to(torch.float32).contiguous()
+
+    def forward(self, ctx, x: torch.Tensor, out: torch.Tensor) -> None:
+        ops.rmsnorm(x, self.weight, self.eps, out)
+
+
+register_part("norm", "rmsnorm", RMSNorm)
