@@ -1,0 +1,49 @@
+"""The library's entry point in Python.
+
+The reference's library use is load -> model -> state -> generate
+(src/lib.rs:28-91): `Parameters::load(path)`, `Mistral::load(params)`,
+`InferenceState::new(config)`, `generate(&model, &mut state, token, &cfg)`,
+`generate_until_eos(...)`.  The same steps here:
+
+    model  = load_model("dir", dtype="bfloat16")           # config.json picks the class
+    engine = Engine(model, max_tokens=8192)                 # cache sized in positions
+    out    = generate_until_eos(engine, prompts, SamplingConfig.greedy(), max_tokens=32,
+                                eos_token_ids=[2])
+    out[0].tokens, out[0].stopped_at_eos
+"""
+from __future__ import annotations
+
+from typing import Callable, List, Optional, Sequence
+
+from .engine.engine import Engine, SeqInput, load_model, model_from_tensors
+from .engine.generate import GenerationResult, generate as _generate
+from .sampling.config import SamplingConfig
+
+
+def generate_until_eos(engine: Engine, prompts: Sequence[Sequence[int]], config: SamplingConfig,
+                       max_tokens: int, eos_token_ids: Sequence[int] = (),
+                       on_token: Optional[Callable[[int, int], None]] = None,
+                       max_batch: Optional[int] = None) -> List[GenerationResult]:
+    """Generate for each prompt (a list of token ids) until `max_tokens` tokens
+    are out or one of `eos_token_ids` is drawn; the stop id is not returned."""
+    from .sampling.sampler import Sampler
+    return _generate(engine, Sampler(config, engine.device), prompts, max_tokens, eos_token_ids,
+                     max_batch, on_token)
+
+
+def generate(model_dir: str, prompts: Sequence[Sequence[int]], max_tokens: int = 16,
+             temperature: float = 0.7, top_k: Optional[int] = None, top_p: Optional[float] = None,
+             seed: int = 0, stop_ids: Optional[Sequence[int]] = None, dtype: str = "bfloat16",
+             max_seq_len: Optional[int] = None, device: str = "cuda:0") -> List[GenerationResult]:
+    """Load the model folder and generate for every prompt.  `stop_ids` None
+    means config.json's eos_token_id, if it has one."""
+    model = load_model(model_dir, dtype, device)
+    if stop_ids is None:
+        stop_ids = list(getattr(model.config, "eos_token_ids", []) or [])
+    longest = max(len(p) for p in prompts) + max_tokens
+    if max_seq_len is not None and longest > max_seq_len:
+        raise ValueError(f"a request needs {longest} positions, --max-seq-len allows {max_seq_len}")
+    per_seq = -(-longest // 64) * 64
+    engine = Engine(model, max_tokens=per_seq * len(prompts), max_slots=len(prompts))
+    cfg = SamplingConfig(temperature=temperature, top_k=top_k, top_p=top_p, seed=seed)
+    return generate_until_eos(engine, prompts, cfg, max_tokens, stop_ids)

@@ -150,6 +150,12 @@ class Cache:
                 while len(pages) < g.pages_needed(self.length[slot] + n_new):
                     pages.append(g.pool.take())
 
+    def fits(self, lengths: List[int]) -> bool:
+        """Would new sequences of these final lengths find slots and pages now?"""
+        if len(lengths) > self.slots.n_free:
+            return False
+        return all(sum(g.pages_needed(n) for n in lengths) <= g.pool.n_free for g in self.groups)
+
     def commit(self, growth: List[Tuple[int, int]]) -> None:
         for slot, n_new in growth:
             self.length[slot] += n_new

@@ -101,6 +101,10 @@ class Engine:
     def length(self, slot: int) -> int:
         return self.cache.length[slot]
 
+    def fits(self, lengths: List[int]) -> bool:
+        """Can new sequences that grow to these lengths be held now?"""
+        return self.cache.fits(list(lengths))
+
     # ---- the step ----------------------------------------------------------
     def build_context(self, batch: Sequence[SeqInput]) -> Tuple[StepContext, Optional[torch.Tensor], int]:
         cache = self.cache

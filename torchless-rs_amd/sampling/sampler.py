@@ -1,0 +1,37 @@
+"""Drawing one token per sequence from float32 logits on the GPU.
+
+The draw of sequence s at its step t uses the uniform number that
+Philox4x32-10 gives for key = seed and counter = (t, s, 0, 0): it does not
+depend on which other sequences share the batch."""
+from __future__ import annotations
+
+from typing import List, Sequence
+
+import torch
+
+from ..kernels import ops
+from .config import SamplingConfig
+
+
+class Sampler:
+    def __init__(self, config: SamplingConfig, device):
+        self.config = config
+        self.device = device
+        self._probs = None
+
+    def sample(self, logits: torch.Tensor, seq_ids: Sequence[int], steps: Sequence[int]) -> List[int]:
+        """logits: float32 [B, V] on the GPU -> B token ids."""
+        B, V = logits.shape
+        c = self.config
+        counters = torch.tensor([[int(s), int(t)] for s, t in zip(seq_ids, steps)], dtype=torch.int32,
+                                device=logits.device).view(B, 2)
+        if self._probs is None or self._probs.shape[0] < B or self._probs.shape[1] != V:
+            self._probs = torch.empty((B, V), dtype=torch.float32, device=logits.device)
+        out = torch.empty((B,), dtype=torch.int32, device=logits.device)
+        ops.sample(logits.contiguous(), float(c.temperature), int(c.top_k or 0), float(c.top_p or 0.0),
+                   int(c.seed), counters, self._probs[:B], out)
+        return out.tolist()
+
+    def last_distribution(self, B: int) -> torch.Tensor:
+        """The probabilities the last draw was made from (temperature > 0)."""
+        return self._probs[:B]
