@@ -159,19 +159,22 @@ def greedy(logits: torch.Tensor) -> int:
 
 
 def top_k_filter(z: torch.Tensor, k: int) -> torch.Tensor:
-    """Keep the k largest, others to -inf; ties at the threshold are kept in
-    index order until k are kept.  src/sampler/mod.rs:93-119"""
+    """Keep the k largest, others to -inf.  On ties at the threshold: every
+    value above it is kept and then values equal to it, in index order, until
+    k are kept.  src/sampler/mod.rs:93-119 (the rule is the one its comment at
+    :107-109 states; its loop at :110-117 would also drop larger values that
+    come after k ties, which no caller can want)."""
     z = z.clone()
     thr = torch.sort(z, descending=True).values[min(k, z.numel()) - 1]
-    if int((z >= thr).sum()) <= k:
-        z[z < thr] = float("-inf")
-        return z
-    kept = 0
+    room = k - int((z > thr).sum())
     for i in range(z.numel()):
-        if z[i] >= thr and kept < k:
-            kept += 1
-        else:
+        if z[i] < thr:
             z[i] = float("-inf")
+        elif z[i] == thr:
+            if room > 0:
+                room -= 1
+            else:
+                z[i] = float("-inf")
     return z
 
 

@@ -1,0 +1,106 @@
+"""The generation loop's decisions, with a model of straw (no GPU): stop ids,
+sequences that end earlier, batches one after another, slots used again."""
+from typing import List
+
+import pytest
+import torch
+
+from torchless_rs_amd.engine.generate import generate, plan_batches
+
+V = 50
+
+
+class StrawEngine:
+    """Next token = (last token + 1) mod V.  Keeps books like the real one."""
+
+    def __init__(self, slots=4, pages=64):
+        self.free_slots = list(range(slots - 1, -1, -1))
+        self.held = {}
+        self.pages = pages
+        self.steps: List[List[int]] = []          # lengths of each step's entries
+        self.alloc_log: List[int] = []
+
+    def alloc(self):
+        s = self.free_slots.pop()
+        self.held[s] = []
+        self.alloc_log.append(s)
+        return s
+
+    def free(self, s):
+        assert s in self.held, "freed twice"
+        del self.held[s]
+        self.free_slots.append(s)
+
+    def fits(self, lengths):
+        return len(lengths) <= len(self.free_slots) and sum(-(-n // 64) for n in lengths) <= self.pages
+
+    def step(self, batch):
+        self.steps.append([len(b.tokens) for b in batch])
+        out = torch.zeros(len(batch), V)
+        for i, b in enumerate(batch):
+            assert b.slot in self.held and list(b.want) == [len(b.tokens) - 1]
+            self.held[b.slot] += list(b.tokens)
+            out[i, (self.held[b.slot][-1] + 1) % V] = 1.0
+        return out
+
+
+class ArgmaxSampler:
+    def __init__(self):
+        self.calls = []
+
+    def sample(self, logits, seq_ids, steps):
+        self.calls.append((list(seq_ids), list(steps)))
+        return logits.argmax(-1).tolist()
+
+
+def test_counts_and_order():
+    eng, smp = StrawEngine(), ArgmaxSampler()
+    out = generate(eng, smp, [[1, 2, 3], [10], [20, 21]], max_tokens=4)
+    assert [r.tokens for r in out] == [[4, 5, 6, 7], [11, 12, 13, 14], [22, 23, 24, 25]]
+    assert all(r.finish_reason == "length" and not r.stopped_at_eos for r in out)
+    assert eng.steps == [[3, 1, 2], [1, 1, 1], [1, 1, 1], [1, 1, 1]]     # prompts whole, then one each
+    assert not eng.held                                                   # every slot given back
+    assert smp.calls[1] == ([0, 1, 2], [1, 1, 1])                         # (request, its step) feed the draw
+
+
+def test_stop_id_ends_one_sequence_only():
+    eng, smp = StrawEngine(), ArgmaxSampler()
+    seen = []
+    out = generate(eng, smp, [[1], [40], [7]], max_tokens=6, stop_ids=[43, 9],
+                   on_token=lambda i, t: seen.append((i, t)))
+    assert out[0].tokens == [2, 3, 4, 5, 6, 7] and out[0].finish_reason == "length"
+    assert out[1].tokens == [41, 42] and out[1].stopped_at_eos           # 43 is not part of the output
+    assert out[2].tokens == [8] and out[2].finish_reason == "stop"
+    assert eng.steps == [[1, 1, 1], [1, 1, 1], [1, 1], [1], [1], [1]]     # the batch shrinks
+    assert (1, 43) not in seen and (1, 42) in seen and len(seen) == 9
+    assert not eng.held
+
+
+def test_stop_at_first_token_and_zero_budget():
+    eng, smp = StrawEngine(), ArgmaxSampler()
+    out = generate(eng, smp, [[4]], max_tokens=3, stop_ids=[5])
+    assert out[0].tokens == [] and out[0].stopped_at_eos
+    out = generate(eng, smp, [[4]], max_tokens=0)
+    assert out[0].tokens == [] and out[0].finish_reason == "length" and eng.steps == [[1]]
+    with pytest.raises(ValueError, match="empty"):
+        generate(eng, smp, [[1], []], max_tokens=2)
+
+
+def test_batches_one_after_another_reuse_slots():
+    eng, smp = StrawEngine(slots=2), ArgmaxSampler()
+    prompts = [[i] for i in range(5)]
+    out = generate(eng, smp, prompts, max_tokens=2)
+    assert [r.tokens for r in out] == [[i + 1, i + 2] for i in range(5)]
+    assert [len(s) for s in eng.steps] == [2, 2, 2, 2, 1, 1]              # batches of 2, 2, 1
+    assert len(eng.alloc_log) == 5 and set(eng.alloc_log) == {0, 1}       # the same slots again
+    out = generate(StrawEngine(slots=4), smp, prompts, max_tokens=1, max_batch=3)
+    assert [r.tokens for r in out] == [[i + 1] for i in range(5)]
+
+
+def test_plan_by_pages():
+    fits = lambda ls: sum(-(-n // 64) for n in ls) <= 4
+    assert plan_batches([64, 64, 128, 65, 200, 10], fits, None) == [[0, 1, 2], [3], [4], [5]] or \
+        plan_batches([64, 64, 128, 65, 200, 10], fits, None) == [[0, 1, 2], [3], [4, 5]]
+    assert plan_batches([1] * 5, fits, 2) == [[0, 1], [2, 3], [4]]
+    with pytest.raises(ValueError, match="more than the cache holds"):
+        plan_batches([10, 300], fits, None)

@@ -1,0 +1,354 @@
+"""The engine against the plain implementation, in float32 and bfloat16: each
+request alone and whole; with the last 32 tokens one by one; in batches of
+unequal lengths whose shorter requests end earlier, one batch after another
+so that slots are used again; long decoding; the first tokens of a sequence;
+generation through the entry point; trace replay."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import plain_mistral as plain
+from test_gpu_kernels import philox_uniform
+from util import CONFIGS, TOL, make_model_dir, prompts, read_model_dir, rel_err
+
+pytestmark = pytest.mark.gpu
+REPO = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LENGTHS = {"A": [5, 11, 17, 40], "B": [1, 9, 30, 64], "C": [2, 70, 150, 33]}
+NAMES = ["A", "B", "C"]
+DTYPES = ["float32", "bfloat16"]
+
+
+@pytest.fixture(scope="module")
+def zoo(tmp_path_factory):
+    """Model folders (bfloat16 weights, read by both paths), their tensors,
+    prompts and the plain logits of every prompt."""
+    tmp = tmp_path_factory.mktemp("models")
+    out = {}
+    for name in NAMES:
+        d = make_model_dir(tmp, name)
+        cfg, w = read_model_dir(d)
+        ps = prompts(cfg["vocab_size"], LENGTHS[name], seed=1 + len(name))
+        out[name] = dict(dir=d, cfg=cfg, w=w, prompts=ps, want=[plain.forward(w, cfg, p) for p in ps])
+    return out
+
+
+_engines = {}
+
+
+def engine_for(zoo, name, dtype, poison=True):
+    from torchless_rs_amd.engine import Engine, load_model
+    key = (name, dtype)
+    if key not in _engines:
+        _engines[key] = Engine(load_model(zoo[name]["dir"], dtype), max_tokens=64 * 24, max_slots=8)
+    eng = _engines[key]
+    assert not eng.cache.length, "a test left slots held"
+    if poison:                      # stale rows must never be read: make them NaN
+        for g in eng.cache.groups:
+            g.storage.fill_(float("nan"))
+    return eng
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_each_request_alone_and_whole(zoo, name, dtype):
+    from torchless_rs_amd.engine import SeqInput
+    eng, z = engine_for(zoo, name, dtype), zoo[name]
+    for p, want in zip(z["prompts"], z["want"]):
+        s = eng.alloc()
+        got = eng.step([SeqInput(s, p, list(range(len(p))))]).clone()
+        eng.free(s)
+        assert rel_err(got, want) < TOL[dtype], (name, dtype, len(p))
+    eng.cache.check()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_last_32_one_by_one(zoo, name, dtype):
+    from torchless_rs_amd.engine import SeqInput
+    eng, z = engine_for(zoo, name, dtype), zoo[name]
+    for p, want in zip(z["prompts"], z["want"]):
+        k = min(32, len(p) - 1)
+        s = eng.alloc()
+        outs = []
+        if len(p) - k:
+            head = len(p) - k
+            outs.append(eng.step([SeqInput(s, p[:head], list(range(head)))]).clone())
+        for t in p[len(p) - k:]:
+            outs.append(eng.step([SeqInput(s, [t], [0])]).clone())
+        eng.free(s)
+        assert rel_err(torch.cat(outs), want) < TOL[dtype], (name, dtype, len(p))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_unequal_batches_one_after_another(zoo, name, dtype):
+    """Prompts are cut at different places: the head goes in as one step of
+    the batch, the rest is fed one token a step, so the shorter requests end
+    earlier.  Three batches in a row take the same slots again."""
+    from torchless_rs_amd.engine import SeqInput
+    eng, z = engine_for(zoo, name, dtype), zoo[name]
+    ps, wants = z["prompts"], z["want"]
+    heads_of = [[max(1, len(p) // 2) for p in ps], [1] * len(ps), [max(1, len(p) - 3) for p in ps]]
+    used = []
+    for heads in heads_of:
+        slots = [eng.alloc() for _ in ps]
+        used.append(sorted(slots))
+        got = [[] for _ in ps]
+        lg = eng.step([SeqInput(s, p[:h], list(range(h))) for s, p, h in zip(slots, ps, heads)]).clone()
+        off = 0
+        for i, h in enumerate(heads):
+            got[i].append(lg[off:off + h])
+            off += h
+        fed = list(heads)
+        live = [i for i in range(len(ps)) if fed[i] < len(ps[i])]
+        for i in set(range(len(ps))) - set(live):
+            eng.free(slots[i])
+        while live:
+            lg = eng.step([SeqInput(slots[i], [ps[i][fed[i]]], [0]) for i in live]).clone()
+            for r, i in enumerate(live):
+                got[i].append(lg[r:r + 1])
+                fed[i] += 1
+            for i in [i for i in live if fed[i] == len(ps[i])]:
+                eng.free(slots[i])
+            live = [i for i in live if fed[i] < len(ps[i])]
+        for i, want in enumerate(wants):
+            assert rel_err(torch.cat(got[i]), want) < TOL[dtype], (name, dtype, heads, i)
+        eng.cache.check()
+    assert used[0] == used[1] == used[2]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_long_decoding_past_window_and_ring(zoo, name, dtype):
+    """300 tokens, the first 5 as a prompt and the rest one by one: the window
+    is exceeded many times and the ring of pages wraps."""
+    from torchless_rs_amd.engine import SeqInput
+    eng, z = engine_for(zoo, name, dtype), zoo[name]
+    ids = prompts(z["cfg"]["vocab_size"], [300], seed=77)[0]
+    want = plain.forward(z["w"], z["cfg"], ids)
+    s = eng.alloc()
+    outs = [eng.step([SeqInput(s, ids[:5], [0, 1, 2, 3, 4])]).clone()]
+    for t in ids[5:]:
+        outs.append(eng.step([SeqInput(s, [t], [0])]).clone())
+    held = len(eng.cache.groups[0].pages_of_slot[s])
+    eng.free(s)
+    got = torch.cat(outs)
+    assert rel_err(got, want) < TOL[dtype]
+    assert rel_err(got[-20:], want[-20:]) < TOL[dtype]
+    assert held == -(-z["cfg"]["sliding_window"] // 64)        # a ring, not 5 pages
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_prompt_in_chunks_longer_than_the_ring(zoo, dtype):
+    """Steps of 100 tokens into a window of 70 (ring of 128 positions)."""
+    from torchless_rs_amd.engine import SeqInput
+    eng, z = engine_for(zoo, "C", dtype), zoo["C"]
+    ids = prompts(z["cfg"]["vocab_size"], [450], seed=78)[0]
+    want = plain.forward(z["w"], z["cfg"], ids)
+    s = eng.alloc()
+    outs = []
+    for c0 in (0, 100, 300, 449):
+        part = ids[c0:{0: 100, 100: 300, 300: 449, 449: 450}[c0]]
+        outs.append(eng.step([SeqInput(s, part, list(range(len(part))))]).clone())
+    eng.free(s)
+    assert rel_err(torch.cat(outs), want) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_first_tokens(zoo, name, dtype):
+    from torchless_rs_amd.engine import SeqInput
+    eng, z = engine_for(zoo, name, dtype), zoo[name]
+    ids = z["prompts"][-1][:3]
+    want = plain.forward(z["w"], z["cfg"], ids)
+    s = eng.alloc()
+    got = torch.cat([eng.step([SeqInput(s, [t], [0])]).clone() for t in ids])
+    eng.free(s)
+    assert rel_err(got, want) < TOL[dtype]
+    assert rel_err(got[:1], want[:1]) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_padding_and_wanted_rows(zoo, dtype):
+    """Logits come back only where wanted, in the order asked; a step that wants
+    nothing still commits its rows."""
+    from torchless_rs_amd.engine import SeqInput
+    eng, z = engine_for(zoo, "B", dtype), zoo["B"]
+    p0, p1 = z["prompts"][2], z["prompts"][1]
+    a, b = eng.alloc(), eng.alloc()
+    assert eng.step([SeqInput(a, p0[:10], []), SeqInput(b, p1[:4], [])]).shape == (0, 384)
+    lg = eng.step([SeqInput(a, p0[10:], [19, 0]), SeqInput(b, p1[4:], [4])]).clone()
+    eng.free(a); eng.free(b)
+    want = torch.stack([z["want"][2][29], z["want"][2][10], z["want"][1][8]])
+    assert rel_err(lg, want) < TOL[dtype]
+
+
+def test_step_errors(zoo):
+    from torchless_rs_amd.cache import CacheFull
+    from torchless_rs_amd.engine import SeqInput, StepError
+    eng = engine_for(zoo, "A", "float32")
+    with pytest.raises(StepError, match="at least one sequence"):
+        eng.step([])
+    with pytest.raises(StepError, match="not held"):
+        eng.step([SeqInput(3, [1], [0])])
+    s = eng.alloc()
+    with pytest.raises(StepError, match="vocabulary"):
+        eng.step([SeqInput(s, [1, 256], [0])])
+    with pytest.raises(StepError, match="wanted index"):
+        eng.step([SeqInput(s, [1, 2], [2])])
+    with pytest.raises(StepError, match="at least one token"):
+        eng.step([SeqInput(s, [], [])])
+    eng.free(s)
+    from torchless_rs_amd.engine import Engine
+    small = Engine(eng.model, max_tokens=64)                   # one page in all... and full attention?
+    t = small.alloc()
+    small.step([SeqInput(t, [1] * 64, [63])])
+    small.step([SeqInput(t, [1], [0])])                        # window of 8: the ring never grows
+    small.free(t)
+    engB = engine_for(zoo, "B", "float32")
+    smallB = Engine(engB.model, max_tokens=64)
+    t = smallB.alloc()
+    with pytest.raises(CacheFull, match="max_tokens"):
+        smallB.step([SeqInput(t, [1] * 65, [64])])
+    smallB.free(t)
+
+
+# ---- generation through the entry point ------------------------------------------
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_greedy_generation_float32(zoo, name):
+    from torchless_rs_amd import SamplingConfig, generate_until_eos
+    eng, z = engine_for(zoo, name, "float32"), zoo[name]
+    ps = z["prompts"][:3]
+    out = generate_until_eos(eng, ps, SamplingConfig.greedy(), max_tokens=8)
+    for p, r in zip(ps, out):
+        want, _ = plain.generate_greedy(z["w"], z["cfg"], p, 8)
+        assert r.tokens == want and r.finish_reason == "length"
+    # a stop id ends one sequence and is not returned; the others go on
+    stop = out[1].tokens[2]
+    out2 = generate_until_eos(eng, ps, SamplingConfig.greedy(), max_tokens=8, eos_token_ids=[stop])
+    for r1, r2 in zip(out, out2):
+        cut = r1.tokens.index(stop) if stop in r1.tokens else None
+        assert r2.tokens == (r1.tokens if cut is None else r1.tokens[:cut])
+        assert r2.stopped_at_eos == (cut is not None)
+    # more requests than slots: batches one after another
+    many = (ps * 4)[:11]
+    out3 = generate_until_eos(eng, many, SamplingConfig.greedy(), max_tokens=4)
+    assert [r.tokens for r in out3] == [out[i % 3].tokens[:4] for i in range(11)]
+    eng.cache.check()
+    assert not eng.cache.length
+
+
+def test_greedy_generation_bfloat16(zoo):
+    """In bfloat16 a near-tie may fall the other way: every token drawn must be
+    the plain argmax up to the tolerance of the logits."""
+    from torchless_rs_amd import SamplingConfig, generate_until_eos
+    eng, z = engine_for(zoo, "B", "bfloat16"), zoo["B"]
+    ps = z["prompts"][:3]
+    out = generate_until_eos(eng, ps, SamplingConfig.greedy(), max_tokens=8)
+    for p, r in zip(ps, out):
+        ids = list(p)
+        for t in r.tokens:
+            lg = plain.forward(z["w"], z["cfg"], ids)[-1]
+            assert float(lg.max() - lg[t]) <= 2 * TOL["bfloat16"] * float(lg.abs().max())
+            ids.append(t)
+
+
+def test_temperature_generation_follows_the_seeded_draws(zoo):
+    from torchless_rs_amd import SamplingConfig, generate_until_eos
+    eng, z = engine_for(zoo, "B", "float32"), zoo["B"]
+    ps = z["prompts"]
+    cfg = SamplingConfig(temperature=0.8, seed=4)
+    out = generate_until_eos(eng, ps, cfg, max_tokens=16)
+    again = generate_until_eos(eng, ps[::-1], cfg, max_tokens=16)[::-1]
+    for i, (p, r) in enumerate(zip(ps, out)):
+        ids = list(p)
+        for step, t in enumerate(r.tokens):
+            lg = plain.forward(z["w"], z["cfg"], ids)[-1]
+            want = plain.sample(lg, philox_uniform(4, step, i), 0.8)
+            if t != want:                                       # the draw fell on a boundary
+                cum = plain.sample_distribution(lg, 0.8).cumsum(0)
+                assert abs(float(cum[min(t, want)]) - philox_uniform(4, step, i)) < 1e-5
+            ids.append(t)
+    # a request's draws are keyed by its own index, so another order of the batch gives other tokens,
+    # but the same requests in the same order give the same tokens
+    assert [r.tokens for r in generate_until_eos(eng, ps, cfg, max_tokens=16)] == [r.tokens for r in out]
+    assert len(again) == len(out)
+
+
+# ---- trace replay ----------------------------------------------------------------
+
+def replay(model_dir, dtype, lines, tmp, max_tokens=1024):
+    out = os.path.join(str(tmp), f"out_{dtype}_{len(os.listdir(str(tmp)))}")
+    env = dict(os.environ)
+    r = subprocess.run([os.path.join(REPO, "bin", "trace_run"), "--model", model_dir, "--dtype", dtype,
+                        "--out", out, "--max-tokens", str(max_tokens)],
+                       input="".join(json.dumps(l) + "\n" for l in lines), text=True, capture_output=True,
+                       env=env, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert r.stdout.split("\n")[:-1] == [f"done {l['step']}" for l in lines]
+    return out
+
+
+def read_logits(out, step, V):
+    return torch.from_numpy(np.fromfile(os.path.join(out, f"{step}.f32"), dtype="<f4").reshape(-1, V).copy())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_trace_replay(zoo, dtype, tmp_path):
+    z = zoo["C"]
+    ps, wants, V = z["prompts"], z["want"], z["cfg"]["vocab_size"]
+    lines, expect = [], {}
+    # each request alone and whole
+    step = 0
+    for i, p in enumerate(ps):
+        lines.append({"step": step, "entries": [{"id": f"w{i}", "tokens": p, "want": list(range(len(p)))}],
+                      "end": [f"w{i}"]})
+        expect[step] = wants[i]
+        step += 1
+    # the longest with its last 32 tokens one by one
+    p, w = ps[2], wants[2]
+    lines.append({"step": step, "entries": [{"id": "s", "tokens": p[:-32], "want": []}], "end": []})
+    step += 1
+    for j in range(len(p) - 32, len(p)):
+        lines.append({"step": step, "entries": [{"id": "s", "tokens": [p[j]], "want": [0]}],
+                      "end": ["s"] if j == len(p) - 1 else []})
+        expect[step] = w[j:j + 1]
+        step += 1
+    # two batches of unequal lengths, shorter requests ending earlier
+    for rnd in range(2):
+        heads = [max(1, len(q) - 4 * (i + 1)) for i, q in enumerate(ps)]
+        lines.append({"step": step, "entries": [{"id": f"b{rnd}_{i}", "tokens": q[:h], "want": [h - 1]}
+                                                for i, (q, h) in enumerate(zip(ps, heads))],
+                      "end": [f"b{rnd}_{i}" for i, (q, h) in enumerate(zip(ps, heads)) if h == len(q)]})
+        expect[step] = torch.stack([wants[i][h - 1] for i, h in enumerate(heads)])
+        step += 1
+        fed = list(heads)
+        while any(f < len(q) for f, q in zip(fed, ps)):
+            live = [i for i, q in enumerate(ps) if fed[i] < len(q)]
+            lines.append({"step": step, "entries": [{"id": f"b{rnd}_{i}", "tokens": [ps[i][fed[i]]], "want": [0]}
+                                                    for i in live],
+                          "end": [f"b{rnd}_{i}" for i in live if fed[i] + 1 == len(ps[i])]})
+            expect[step] = torch.stack([wants[i][fed[i]] for i in live])
+            for i in live:
+                fed[i] += 1
+            step += 1
+    out = replay(z["dir"], dtype, lines, tmp_path, max_tokens=64 * 8)
+    assert sorted(int(f[:-4]) for f in os.listdir(out)) == sorted(expect)
+    for st, want in expect.items():
+        assert rel_err(read_logits(out, st, V), want) < TOL[dtype], st
+
+
+def test_command_line(zoo):
+    z = zoo["A"]
+    r = subprocess.run([os.path.join(REPO, "bin", "torchless"), "--temperature", "0", "--dtype", "float32",
+                        "--max-tokens", "5", z["dir"], "3 1 4 1 5; 9 2 6"], capture_output=True, text=True,
+                       timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    rows = [[int(t) for t in l.split()] for l in r.stdout.strip().split("\n")]
+    assert rows == [plain.generate_greedy(z["w"], z["cfg"], p, 5)[0] for p in ([3, 1, 4, 1, 5], [9, 2, 6])]

@@ -1,0 +1,318 @@
+"""Each kernel alone against a plain float64 computation, at sizes other than
+the engine's tests use."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import plain_mistral as plain
+from util import rel_err
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+# one output rounding of bfloat16 is 2^-9 relative; float32 results differ by summation order only
+KTOL = {"float32": 3e-6, "bfloat16": 6e-3}
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from torchless_rs_amd.kernels import ops as o
+    o.lib()
+    return o
+
+
+def rnd(*shape, seed=0, dtype=torch.float32, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype)
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_embed(ops, dt):
+    table = rnd(77, 130, dtype=DT[dt]).to(DEV)
+    ids = torch.tensor([0, 76, 5, 5, 31], dtype=torch.int32, device=DEV)
+    out = torch.empty(5, 130, device=DEV)
+    ops.embed(table, ids, out)
+    assert torch.equal(out.cpu(), table.cpu().float()[ids.cpu().long()])
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("n,H", [(1, 100), (5, 4097), (3, 64)])
+def test_rmsnorm(ops, dt, n, H):
+    x = rnd(n, H, seed=1, scale=3.0)
+    w = 1 + 0.2 * rnd(H, seed=2)
+    out = torch.empty(n, H, dtype=DT[dt], device=DEV)
+    ops.rmsnorm(x.to(DEV), w.to(DEV), 1e-3, out)
+    assert rel_err(out, plain.rmsnorm(x.double(), w.double(), 1e-3)) < KTOL[dt]
+    tiny = x * 1e-3                                      # eps matters here
+    ops.rmsnorm(tiny.to(DEV), w.to(DEV), 1e-3, out)
+    assert rel_err(out, plain.rmsnorm(tiny.double(), w.double(), 1e-3)) < KTOL[dt]
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("nq,nkv,d,theta", [(3, 1, 48, 500.0), (8, 2, 128, 1e6), (2, 2, 16, 1e4)])
+def test_rope_split(ops, dt, nq, nkv, d, theta):
+    from torchless_rs_amd.parts.position import Rotary
+    n = 6
+    qkv = rnd(n, (nq + 2 * nkv) * d, seed=3)
+    pos = torch.tensor([0, 1, 7, 100, 5000, 40000], dtype=torch.int32)
+    q = torch.empty(n, nq, d, dtype=DT[dt], device=DEV)
+    k = torch.empty(n, nkv, d, dtype=DT[dt], device=DEV)
+    v = torch.empty(n, nkv, d, dtype=DT[dt], device=DEV)
+    ops.rope_split(qkv.to(DEV), pos.to(DEV), Rotary(d, theta).inv_freq(DEV), nq, nkv, d, q, k, v)
+    x = qkv.double()
+    wq = plain.rope(x[:, :nq * d].view(n, nq, d), pos, theta)
+    wk = plain.rope(x[:, nq * d:(nq + nkv) * d].view(n, nkv, d), pos, theta)
+    wv = x[:, (nq + nkv) * d:].view(n, nkv, d)
+    # angles are float32 as the reference's are: pos * inv_freq carries a relative rounding of
+    # 2^-24 from each factor, so a row at position p may be off by 1.2e-7 * p radians
+    for r, p in enumerate(pos.tolist()):
+        tol = KTOL[dt] + 1.2e-7 * p
+        assert rel_err(q[r], wq[r]) < tol and rel_err(k[r], wk[r]) < tol, (r, p)
+    assert rel_err(v, wv) < KTOL[dt]
+    assert torch.equal(q[0].float().cpu(), qkv[0, :nq * d].view(nq, d).to(DT[dt]).float())   # pos 0: identity
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_silu_mul_and_gather(ops, dt):
+    n, I = 5, 301
+    gu = rnd(n, 2 * I, seed=4, scale=4.0)
+    out = torch.empty(n, I, dtype=DT[dt], device=DEV)
+    ops.silu_mul(gu.to(DEV), out)
+    g, u = gu.double()[:, :I], gu.double()[:, I:]
+    assert rel_err(out, plain.silu(g) * u) < KTOL[dt]
+    x = rnd(9, 70, seed=5).to(DEV)
+    idx = torch.tensor([8, 0, 3, 3], dtype=torch.int32, device=DEV)
+    o = torch.empty(4, 70, device=DEV)
+    ops.gather_rows(x, idx, o)
+    assert torch.equal(o, x[idx.long()])
+
+
+@pytest.mark.parametrize("adt,wdt", [("float32", "float32"), ("bfloat16", "bfloat16"),
+                                     ("bfloat16", "float32"), ("float32", "bfloat16")])
+@pytest.mark.parametrize("M,N,K", [(1, 50, 17), (5, 130, 100), (70, 64, 64), (129, 200, 333)])
+def test_gemm_plain(ops, adt, wdt, M, N, K):
+    a = rnd(M, K, seed=6, dtype=DT[adt])
+    w = rnd(N, K, seed=7, dtype=DT[wdt])
+    want = a.double() @ w.double().t()
+    out = torch.empty(M, N, device=DEV)
+    ops.gemm_plain(a.to(DEV), w.to(DEV), out)
+    assert rel_err(out, want) < 3e-6
+    base = rnd(M, N, seed=8)
+    acc = base.clone().to(DEV)
+    ops.gemm_plain(a.to(DEV), w.to(DEV), acc, accumulate=True)
+    assert rel_err(acc, want + base.double()) < 3e-6
+    # [[1,2],[3,4]] . [1,2] = [5,11]  (src/kernels/tests.rs:5-10 of the reference)
+    o2 = torch.empty(1, 2, device=DEV)
+    ops.gemm_plain(torch.tensor([[1., 2.]], device=DEV), torch.tensor([[1., 2.], [3., 4.]], device=DEV), o2)
+    assert o2.tolist() == [[5., 11.]]
+
+
+def test_gemm_row_does_not_depend_on_the_batch(ops):
+    a = rnd(37, 96, seed=9).to(DEV)
+    w = rnd(80, 96, seed=10).to(DEV)
+    full = torch.empty(37, 80, device=DEV)
+    ops.gemm_plain(a, w, full)
+    one = torch.empty(1, 80, device=DEV)
+    ops.gemm_plain(a[20:21].contiguous(), w, one)
+    assert torch.equal(one[0], full[20])
+
+
+# ---- attention over pages ----------------------------------------------------
+
+def paged_case(ops, dt, nq, nkv, d, window, lens_cached, lens_new, seed=0, n_pages=40):
+    """Random sequences with `lens_cached` positions in pages (scattered, rings
+    for windows) and `lens_new` new rows; returns the kernel's output and the
+    plain result for the new rows."""
+    from torchless_rs_amd.cache import PAGE
+    tdt = DT[dt]
+    B = len(lens_cached)
+    ring = -(-window // PAGE) if window else n_pages
+    g = torch.Generator().manual_seed(seed)
+    pages = torch.full((n_pages, 2, nkv, PAGE, d), float("nan"), dtype=tdt)     # stale rows are poison
+    perm = torch.randperm(n_pages, generator=g).tolist()
+    table = torch.zeros(B, ring if window else max(1, max(-(-(c + n) // PAGE) for c, n in zip(lens_cached, lens_new))),
+                        dtype=torch.int32)
+    seqs, q_rows, k_rows, v_rows, want = [], [], [], [], []
+    row_seq, row_pos, cu = [], [], [0]
+    for b in range(B):
+        T = lens_cached[b] + lens_new[b]
+        q = torch.randn(T, nq, d, generator=g).to(tdt)
+        k = torch.randn(T, nkv, d, generator=g).to(tdt)
+        v = torch.randn(T, nkv, d, generator=g).to(tdt)
+        need = min(-(-T // PAGE), ring)
+        mine = [perm.pop() for _ in range(need)]
+        table[b, :need] = torch.tensor(mine, dtype=torch.int32)
+        for p in range(max(0, lens_cached[b] - ring * PAGE), lens_cached[b]):
+            pg = mine[(p // PAGE) % ring]
+            pages[pg, 0, :, p % PAGE] = k[p]
+            pages[pg, 1, :, p % PAGE] = v[p]
+        full = plain.attention_core(q.double(), k.double(), v.double(), torch.arange(T), window)
+        want.append(full[lens_cached[b]:])
+        q_rows.append(q[lens_cached[b]:]); k_rows.append(k[lens_cached[b]:]); v_rows.append(v[lens_cached[b]:])
+        row_seq += [b] * lens_new[b]
+        row_pos += list(range(lens_cached[b], T))
+        cu.append(cu[-1] + lens_new[b])
+    dev = lambda t: t.contiguous().to(DEV)
+    i32 = lambda l: torch.tensor(l, dtype=torch.int32, device=DEV)
+    qn, kn, vn = dev(torch.cat(q_rows)), dev(torch.cat(k_rows)), dev(torch.cat(v_rows))
+    out = torch.empty_like(qn)
+    args = dict(pages=dev(pages), table=dev(table), ring=ring, row_seq=i32(row_seq), row_pos=i32(row_pos),
+                cu=i32(cu), cached=i32(lens_cached), after=i32([c + n for c, n in zip(lens_cached, lens_new)]),
+                q=qn, k=kn, v=vn, out=out, window=window, scale=1.0 / math.sqrt(d), want=torch.cat(want))
+    return args
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("nq,nkv,d,window", [(4, 2, 16, None), (6, 1, 32, 70), (5, 5, 48, 8),
+                                             (8, 2, 128, 100), (2, 1, 256, None), (3, 3, 80, 64)])
+def test_attention_cached_and_new(ops, dt, nq, nkv, d, window):
+    a = paged_case(ops, dt, nq, nkv, d, window, lens_cached=[0, 5, 130, 64, 200], lens_new=[17, 1, 3, 70, 1])
+    ops.attn_plain(a["q"], a["k"], a["v"], a["pages"], a["table"], a["ring"], a["row_seq"], a["row_pos"],
+                   a["cu"], a["cached"], window, a["scale"], a["out"])
+    assert rel_err(a["out"], a["want"]) < KTOL[dt]
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("window", [None, 70, 128])
+def test_commit_then_decode_reads_the_pages_only(ops, dt, window):
+    """One new token per sequence: commit first, then everything comes from
+    the pages, also where the ring has wrapped."""
+    nq, nkv, d = 4, 2, 32
+    a = paged_case(ops, dt, nq, nkv, d, window, lens_cached=[0, 63, 64, 300, 191], lens_new=[1] * 5, seed=3)
+    ops.kv_commit(a["k"], a["v"], a["row_seq"], a["row_pos"], a["after"], a["table"], a["ring"], a["pages"])
+    ops.attn_plain(a["q"], None, None, a["pages"], a["table"], a["ring"], a["row_seq"], a["row_pos"],
+                   a["cu"], a["after"], window, a["scale"], a["out"])
+    assert rel_err(a["out"], a["want"]) < KTOL[dt]
+
+
+def test_commit_of_a_chunk_longer_than_the_ring(ops):
+    """A step of 300 rows into a ring of 2 pages keeps the last 128 positions."""
+    from torchless_rs_amd.cache import PAGE
+    nkv, d, window = 1, 16, 70
+    a = paged_case(ops, "float32", 2, nkv, d, window, lens_cached=[10], lens_new=[300], seed=4)
+    ops.kv_commit(a["k"], a["v"], a["row_seq"], a["row_pos"], a["after"], a["table"], a["ring"], a["pages"])
+    pages, table = a["pages"].cpu(), a["table"].cpu()
+    for p in range(310 - 128, 310):
+        pg = int(table[0, (p // PAGE) % 2])
+        assert torch.equal(pages[pg, 0, 0, p % PAGE], a["k"][p - 10, 0].cpu())
+        assert torch.equal(pages[pg, 1, 0, p % PAGE], a["v"][p - 10, 0].cpu())
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_a_far_key_among_hundreds_and_the_windows_edge(ops, dt):
+    """One key is made to match the query far better than the rest: the output
+    must be its value row iff the key is visible."""
+    from torchless_rs_amd.cache import PAGE
+    nq, nkv, d, T = 2, 1, 32, 700
+    tdt = DT[dt]
+    g = torch.Generator().manual_seed(5)
+    for window, far, visible in [(None, 3, True), (200, 499, False), (200, 500, True), (200, 699, True)]:
+        k = torch.randn(T, nkv, d, generator=g) * 0.1
+        v = torch.randn(T, nkv, d, generator=g)
+        qv = torch.randn(d, generator=g)
+        qv = qv / qv.norm()
+        k[far, 0] = qv * 60.0                           # score 60 * |q| / sqrt(d) above all others
+        q = (qv * 8.0).view(1, 1, d).repeat(1, nq, 1)
+        ring = -(-window // PAGE) if window else 11
+        pages = torch.full((11, 2, nkv, PAGE, d), float("nan"), dtype=tdt)
+        table = torch.tensor([[7, 2, 9, 0, 5, 1, 10, 3, 8, 4, 6][:ring]], dtype=torch.int32)
+        for p in range(max(0, T - ring * PAGE), T):
+            pg = int(table[0, (p // PAGE) % ring])
+            pages[pg, 0, :, p % PAGE] = k[p].to(tdt)
+            pages[pg, 1, :, p % PAGE] = v[p].to(tdt)
+        out = torch.empty(1, nq, d, dtype=tdt, device=DEV)
+        i32 = lambda l: torch.tensor(l, dtype=torch.int32, device=DEV)
+        ops.attn_plain(q.to(tdt).to(DEV), None, None, pages.to(DEV), table.to(DEV), ring, i32([0]),
+                       i32([T - 1]), i32([0, 1]), i32([T]), window, 1.0 / math.sqrt(d), out)
+        hit = rel_err(out[0, 0], v[far, 0].to(tdt)) < 1e-2
+        assert hit == visible, (window, far)
+        assert torch.isfinite(out).all()
+
+
+# ---- sampling ------------------------------------------------------------------
+
+def philox_uniform(seed: int, step: int, seq: int) -> float:
+    """Philox4x32-10, key = seed, counter = (step, seq, 0, 0); first word >> 8 / 2^24."""
+    M0, M1, W0, W1, mask = 0xD2511F53, 0xCD9E8D57, 0x9E3779B9, 0xBB67AE85, 0xFFFFFFFF
+    c = [step & mask, seq & mask, 0, 0]
+    k = [seed & mask, (seed >> 32) & mask]
+    for r in range(10):
+        if r:
+            k = [(k[0] + W0) & mask, (k[1] + W1) & mask]
+        p0, p1 = M0 * c[0], M1 * c[2]
+        c = [(p1 >> 32) ^ c[1] ^ k[0], p1 & mask, (p0 >> 32) ^ c[3] ^ k[1], p0 & mask]
+    return (c[0] >> 8) / 16777216.0
+
+
+def test_philox_known_answer():
+    # counter 0, key 0 -> 0x6627e8d5 (the generator's published test vector)
+    assert int(philox_uniform(0, 0, 0) * 16777216) == 0x6627e8d5 >> 8
+
+
+def run_sample(ops, logits, T, k=0, p=0.0, seed=0, counters=None):
+    B, V = logits.shape
+    counters = counters if counters is not None else [[b, 0] for b in range(B)]
+    c = torch.tensor(counters, dtype=torch.int32, device=DEV)
+    probs = torch.empty(B, V, device=DEV)
+    out = torch.empty(B, dtype=torch.int32, device=DEV)
+    ops.sample(logits.to(DEV).contiguous(), T, k, p, seed, c, probs, out)
+    return out.tolist(), probs.cpu()
+
+
+@pytest.mark.parametrize("V", [7, 384, 32000, 50001])
+def test_greedy(ops, V):
+    logits = rnd(5, V, seed=11)
+    logits[1, V // 2] = 50.0
+    logits[2, 0] = 50.0
+    logits[3, V - 1] = 50.0
+    logits[4, 3] = 50.0
+    logits[4, V - 2] = 50.0                                 # equal maxima: the last index wins
+    ids, _ = run_sample(ops, logits, 0.0)
+    assert ids == [plain.greedy(logits[b]) for b in range(5)]
+    assert ids[4] == V - 2
+    ids, _ = run_sample(ops, logits, 0.0, k=3, p=0.5)       # T = 0 is greedy whatever else is set
+    assert ids[1] == V // 2
+
+
+@pytest.mark.parametrize("V", [13, 384, 32000])
+@pytest.mark.parametrize("T,k,p", [(0.8, 0, 0.0), (1.0, 5, 0.0), (0.7, 0, 0.9), (1.3, 50, 0.6), (1.0, 10 ** 6, 1.0)])
+def test_distribution_and_draw(ops, V, T, k, p):
+    logits = rnd(4, V, seed=12, scale=3.0)
+    seed = 1234567891011
+    counters = [[3, 0], [3, 1], [9, 0], [0, 77]]
+    ids, probs = run_sample(ops, logits, T, k, p, seed, counters)
+    for b in range(4):
+        want = plain.sample_distribution(logits[b], T, k or None, p or None)
+        assert abs(float(probs[b].sum()) - 1) < 1e-4
+        assert float((probs[b].double() - want).abs().max()) < 2e-6
+        assert int((probs[b] > 0).sum()) == int((want > 0).sum())
+        r = philox_uniform(seed, counters[b][1], counters[b][0])
+        mine = plain.draw(probs[b].double(), r)
+        assert ids[b] == mine or abs(float(probs[b].double().cumsum(0)[min(ids[b], mine)]) - r) < 1e-5
+
+
+def test_top_k_ties_keep_index_order(ops):
+    logits = torch.tensor([[1.0, 3.0, 1.0, 1.0, 2.0, -4.0]])
+    _, probs = run_sample(ops, logits, 1.0, k=3)
+    want = plain.sample_distribution(logits[0], 1.0, 3, None)
+    assert (probs[0] > 0).tolist() == [True, True, False, False, True, False]
+    assert float((probs[0].double() - want).abs().max()) < 1e-6
+
+
+def test_draws_do_not_depend_on_batch_mates_and_follow_the_probabilities(ops):
+    V = 8
+    z = torch.tensor([[2.0, 1.0, 0.0, -1.0, 0.5, 1.5, -2.0, 0.2]])
+    n = 4000
+    counters = [[17, t] for t in range(n)]
+    ids, probs = run_sample(ops, z.repeat(n, 1), 1.0, seed=5, counters=counters)
+    freq = np.bincount(ids, minlength=V) / n
+    p = probs[0].double().numpy()
+    assert np.all(np.abs(freq - p) < 4 * np.sqrt(p * (1 - p) / n) + 1e-3)
+    alone, _ = run_sample(ops, z, 1.0, seed=5, counters=[[17, 123]])
+    assert alone[0] == ids[123]
+    again, _ = run_sample(ops, z.repeat(n, 1), 1.0, seed=5, counters=counters)
+    assert again == ids                                      # the seed decides
+    other, _ = run_sample(ops, z.repeat(n, 1), 1.0, seed=6, counters=counters)
+    assert other != ids

@@ -1,0 +1,316 @@
+"""Each part alone against the plain implementation; a schedule that names a
+layer twice and lets a run read another run's cache; and a toy mixer with
+state of its own, defined here, that is registered, built and stepped
+without a change to the framework's files."""
+import math
+
+import pytest
+import torch
+
+import plain_mistral as plain
+from util import TOL, rel_err
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DT = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+PTOL = {"float32": 5e-6, "bfloat16": 1.5e-2}
+
+
+def rnd(*shape, seed=0, scale=1.0, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype)
+
+
+def context(cache, batch, dtype):
+    from torchless_rs_amd.engine.engine import build_context
+    from torchless_rs_amd.parts import Workspace
+    return build_context(cache, batch, 10 ** 6, dtype, torch.device(DEV), Workspace(torch.device(DEV)))[0]
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_norm_part(dt):
+    from torchless_rs_amd.parts import PartSpec, make_part
+    norm = make_part("norm", PartSpec("rmsnorm", {"size": 72, "eps": 1e-4}))
+    assert norm.weight_specs()["weight"].shape == (72,)
+    w = 1 + 0.3 * rnd(72, seed=1, dtype=DT[dt])
+    norm.load({"weight": w.to(DEV)}, DT[dt])
+    x = rnd(5, 72, seed=2, scale=2.0)
+    out = torch.empty(5, 72, dtype=DT[dt], device=DEV)
+    norm.forward(None, x.to(DEV), out)
+    assert rel_err(out, plain.rmsnorm(x.double(), w.double(), 1e-4)) < PTOL[dt]
+
+
+def test_position_part():
+    from torchless_rs_amd.parts import PartSpec, make_part
+    rot = make_part("position", PartSpec("rotary", {"head_dim": 48, "theta": 500.0}))
+    f = rot.inv_freq(DEV).cpu()
+    assert f.shape == (24,) and f[0] == 1.0 and bool((f[1:] < f[:-1]).all())     # kernels/tests.rs:54-69
+    assert rel_err(f, plain.rope_inv_freq(48, 500.0)) < 1e-7
+    with pytest.raises(ValueError):
+        make_part("position", PartSpec("rotary", {"head_dim": 7, "theta": 1.0}))
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_feed_forward_part(dt):
+    from torchless_rs_amd.cache import Cache
+    from torchless_rs_amd.engine import SeqInput
+    from torchless_rs_amd.parts import PartSpec, make_part
+    H, I, n = 72, 200, 7
+    ffn = make_part("ffn", PartSpec("swiglu", {"hidden_size": H, "intermediate_size": I}))
+    w = {"mlp.gate_proj.weight": rnd(I, H, seed=3, scale=0.2, dtype=DT[dt]),
+         "mlp.up_proj.weight": rnd(I, H, seed=4, scale=0.2, dtype=DT[dt]),
+         "mlp.down_proj.weight": rnd(H, I, seed=5, scale=0.2, dtype=DT[dt])}
+    assert {k: v.shape for k, v in ffn.weight_specs().items()} == {k: tuple(v.shape) for k, v in w.items()}
+    ffn.load({k: v.to(DEV) for k, v in w.items()}, DT[dt])
+    cache = Cache({}, {}, 64, DT[dt], DEV, 1)
+    s = cache.alloc_slot()
+    ctx = context(cache, [SeqInput(s, [0] * n, [])], DT[dt])
+    y = rnd(n, H, seed=6, dtype=DT[dt])
+    x0 = rnd(n, H, seed=7)
+    x = x0.clone().to(DEV)
+    ffn.forward(ctx, y.to(DEV), x)
+    want = x0.double() + plain.swiglu(y.double(), {k: v.double() for k, v in w.items()}, "")
+    assert rel_err(x, want) < PTOL[dt]
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("nq,nkv,d,window", [(4, 2, 16, 8), (6, 1, 32, None), (3, 3, 48, 70)])
+def test_attention_part_whole_and_in_steps(dt, nq, nkv, d, window):
+    """The mixer alone: two sequences, whole, and cut into a head and single tokens."""
+    from torchless_rs_amd.cache import Cache
+    from torchless_rs_amd.engine import SeqInput
+    from torchless_rs_amd.parts import PartSpec, RunBinding, make_part
+    H, lens = 40, [90, 13]
+    mixer = make_part("mixer", PartSpec("attention", {
+        "hidden_size": H, "n_heads": nq, "n_kv_heads": nkv, "head_dim": d, "window": window,
+        "position": PartSpec("rotary", {"head_dim": d, "theta": 300.0})}))
+    w = {"self_attn.q_proj.weight": rnd(nq * d, H, seed=1, scale=0.3, dtype=DT[dt]),
+         "self_attn.k_proj.weight": rnd(nkv * d, H, seed=2, scale=0.3, dtype=DT[dt]),
+         "self_attn.v_proj.weight": rnd(nkv * d, H, seed=3, scale=0.3, dtype=DT[dt]),
+         "self_attn.o_proj.weight": rnd(H, nq * d, seed=4, scale=0.3, dtype=DT[dt])}
+    assert {k: v.shape for k, v in mixer.weight_specs().items()} == {k: tuple(v.shape) for k, v in w.items()}
+    mixer.load({k: v.to(DEV) for k, v in w.items()}, DT[dt])
+    cfg = {"num_attention_heads": nq, "num_key_value_heads": nkv, "head_dim": d, "hidden_size": H,
+           "rope_theta": 300.0, "sliding_window": window}
+    ys = [rnd(n, H, seed=10 + i, dtype=DT[dt]) for i, n in enumerate(lens)]
+    wd = {k: v.double() for k, v in w.items()}
+    want = torch.cat([plain.attention(y.double(), wd, "", cfg, torch.arange(y.shape[0])) for y in ys])
+
+    cache = Cache({0: mixer.kv_request()}, {}, 64 * 6, DT[dt], DEV, 2)
+    cache.groups[0].storage.fill_(float("nan"))
+    g = cache.groups[0]
+    run = RunBinding(index=0, kv_group=g, kv_group_index=0, kv_layer=0, kv_source=0)
+    # whole
+    slots = [cache.alloc_slot() for _ in lens]
+    batch = [SeqInput(s, [0] * n, []) for s, n in zip(slots, lens)]
+    ctx = context(cache, batch, DT[dt])
+    x = torch.zeros(sum(lens), H, device=DEV)
+    mixer.forward(ctx, run, torch.cat(ys).to(DEV), x)
+    cache.commit([(s, n) for s, n in zip(slots, lens)])
+    assert rel_err(x, want) < PTOL[dt]
+    for s in slots:
+        cache.free_slot(s)
+    # heads of unequal lengths, then one token each until the shorter one ends
+    slots = [cache.alloc_slot() for _ in lens]
+    heads = [50, 3]
+    got = [[], []]
+    ctx = context(cache, [SeqInput(s, [0] * h, []) for s, h in zip(slots, heads)], DT[dt])
+    x = torch.zeros(sum(heads), H, device=DEV)
+    mixer.forward(ctx, run, torch.cat([y[:h] for y, h in zip(ys, heads)]).to(DEV), x)
+    cache.commit(list(zip(slots, heads)))
+    got[0].append(x[:50].clone()); got[1].append(x[50:].clone())
+    fed = list(heads)
+    while any(f < n for f, n in zip(fed, lens)):
+        live = [i for i in range(2) if fed[i] < lens[i]]
+        ctx = context(cache, [SeqInput(slots[i], [0], []) for i in live], DT[dt])
+        x = torch.zeros(len(live), H, device=DEV)
+        mixer.forward(ctx, run, torch.stack([ys[i][fed[i]] for i in live]).to(DEV), x)
+        cache.commit([(slots[i], 1) for i in live])
+        for r, i in enumerate(live):
+            got[i].append(x[r:r + 1].clone())
+            fed[i] += 1
+    assert rel_err(torch.cat(got[0] + got[1]), want) < PTOL[dt]
+
+
+# ---- the schedule is data ----------------------------------------------------------
+
+def test_a_layer_twice_and_a_run_that_reads_anothers_cache():
+    from torchless_rs_amd.engine import Engine, SeqInput
+    from torchless_rs_amd.engine.model import Model
+    from torchless_rs_amd.parts import LayerSpec, ModelSpec, PartSpec, Run
+    from torchless_rs_amd.weights import TensorDict, random_tensors
+    H, V, nq, nkv, d, I = 48, 90, 3, 1, 16, 80
+    norm = PartSpec("rmsnorm", {"size": H, "eps": 1e-5})
+    rot = PartSpec("rotary", {"head_dim": d, "theta": 1000.0})
+
+    def layer(i, own_kv=True, window=None):
+        return LayerSpec(prefix=f"model.layers.{i}.",
+                         mixer=PartSpec("attention", {"hidden_size": H, "n_heads": nq, "n_kv_heads": nkv,
+                                                      "head_dim": d, "window": window, "position": rot,
+                                                      "own_kv": own_kv}),
+                         ffn=PartSpec("swiglu", {"hidden_size": H, "intermediate_size": I}),
+                         mixer_norm=norm, ffn_norm=norm)
+
+    spec = ModelSpec(hidden_size=H, vocab_size=V,
+                     embedding=PartSpec("tokens", {"vocab_size": V, "hidden_size": H}), embedding_prefix="model.",
+                     layers=[layer(0, window=6), layer(1), layer(2, own_kv=False)],
+                     schedule=[Run(0), Run(1), Run(0), Run(2, kv_from=1)],
+                     final_norm=norm, final_norm_prefix="model.norm.",
+                     head=PartSpec("linear", {"vocab_size": V, "hidden_size": H}), head_prefix="lm_head.")
+    names = spec.weight_specs()
+    assert "model.layers.2.self_attn.k_proj.weight" not in names and "model.layers.2.self_attn.q_proj.weight" in names
+    w = random_tensors(names, seed=3, std=0.15, norm_std=0.1, dtype=torch.float32)
+    model = Model(spec, None, torch.float32, DEV)
+    model.load_weights(TensorDict(w))
+    eng = Engine(model, max_tokens=64 * 4)
+    assert len(eng.cache.groups) == 2                       # windowed runs (0 and 2) and the full one
+    assert sorted(g.runs for g in eng.cache.groups) == [[0, 2], [1]]
+
+    def plain_forward(ids):
+        T = len(ids)
+        pos = torch.arange(T)
+        wd = {k: v.double() for k, v in w.items()}
+        x = wd["model.embed_tokens.weight"][ids]
+        cfg0 = {"num_attention_heads": nq, "num_key_value_heads": nkv, "head_dim": d, "hidden_size": H,
+                "rope_theta": 1000.0, "rms_norm_eps": 1e-5}
+        x = plain.block(x, wd, "model.layers.0.", dict(cfg0, sliding_window=6), pos)
+        # layer 1, keeping its rotated keys and its values
+        p1 = "model.layers.1."
+        y = plain.rmsnorm(x, wd[p1 + "input_layernorm.weight"], 1e-5)
+        k1 = plain.rope(plain.linear(y, wd[p1 + "self_attn.k_proj.weight"]).view(T, nkv, d), pos, 1000.0)
+        v1 = plain.linear(y, wd[p1 + "self_attn.v_proj.weight"]).view(T, nkv, d)
+        x = plain.block(x, wd, p1, dict(cfg0, sliding_window=None), pos)
+        x = plain.block(x, wd, "model.layers.0.", dict(cfg0, sliding_window=6), pos)   # the same weights again
+        p2 = "model.layers.2."
+        y = plain.rmsnorm(x, wd[p2 + "input_layernorm.weight"], 1e-5)
+        q = plain.rope(plain.linear(y, wd[p2 + "self_attn.q_proj.weight"]).view(T, nq, d), pos, 1000.0)
+        a = plain.attention_core(q, k1, v1, pos, None).reshape(T, nq * d)
+        x = x + plain.linear(a, wd[p2 + "self_attn.o_proj.weight"])
+        x = x + plain.swiglu(plain.rmsnorm(x, wd[p2 + "post_attention_layernorm.weight"], 1e-5), wd, p2)
+        return plain.linear(plain.rmsnorm(x, wd["model.norm.weight"], 1e-5), wd["lm_head.weight"])
+
+    g = torch.Generator().manual_seed(8)
+    ids = torch.randint(0, V, (40,), generator=g).tolist()
+    want = plain_forward(ids)
+    s = eng.alloc()
+    whole = eng.step([SeqInput(s, ids, list(range(40)))]).clone()
+    eng.free(s)
+    assert rel_err(whole, want) < TOL["float32"]
+    s = eng.alloc()
+    outs = [eng.step([SeqInput(s, ids[:9], list(range(9)))]).clone(),
+            eng.step([SeqInput(s, ids[9:25], list(range(16)))]).clone()]
+    outs += [eng.step([SeqInput(s, [t], [0])]).clone() for t in ids[25:]]
+    eng.free(s)
+    assert rel_err(torch.cat(outs), want) < TOL["float32"]
+
+
+# ---- a toy mixer with state of its own ----------------------------------------------
+
+def test_a_toy_mixer_with_state_registers_builds_and_steps():
+    """out_t = W (decay-weighted running sum of the inputs up to t): the sum so
+    far is the mixer's state, one row of H floats per sequence, kept in the
+    cache's state area.  Library operations are fine for a toy."""
+    from torchless_rs_amd.cache import StateRequest
+    from torchless_rs_amd.config import config_from_dict, register_architecture, unregister_architecture
+    from torchless_rs_amd.config.base import ModelConfig
+    from torchless_rs_amd.engine import Engine, SeqInput
+    from torchless_rs_amd.engine.model import Model
+    from torchless_rs_amd.models import model_spec_for
+    from torchless_rs_amd.parts import (LayerSpec, Mixer, ModelSpec, PartSpec, Run, register_part,
+                                        unregister_part)
+    from torchless_rs_amd.weights import TensorDict, WeightSpec, random_tensors
+
+    class RunningSum(Mixer):
+        def __init__(self, hidden_size, decay):
+            self.H, self.decay = hidden_size, decay
+
+        def weight_specs(self):
+            return {"mix.weight": WeightSpec((self.H, self.H))}
+
+        def state_request(self):
+            return StateRequest((self.H,), torch.float32)
+
+        def load(self, tensors, compute_dtype):
+            self.w = tensors["mix.weight"].float()
+
+        def forward(self, ctx, run, y, x):
+            cu, slots = ctx.host["cu"], ctx.host["slots"]
+            for b, slot in enumerate(slots):
+                s = run.state[slot].clone()
+                for r in range(int(cu[b]), int(cu[b + 1])):
+                    s = self.decay * s + y[r].float()
+                    x[r] += s @ self.w.t()
+                run.state[slot] = s
+
+    class ToyConfig(ModelConfig):
+        @classmethod
+        def from_dict(cls, d):
+            c = cls(architecture="ToyForCausalLM")
+            c.d = d
+            return c
+
+    def toy_spec(cfg):
+        d = cfg.d
+        H, V = d["width"], d["vocab"]
+        norm = PartSpec("rmsnorm", {"size": H, "eps": d["eps"]})
+        layers = [LayerSpec(prefix=f"toy.{i}.", mixer=PartSpec("running_sum", {"hidden_size": H, "decay": d["decay"]}),
+                            ffn=PartSpec("swiglu", {"hidden_size": H, "intermediate_size": d["inner"]}),
+                            mixer_norm=norm, ffn_norm=norm) for i in range(d["depth"])]
+        return ModelSpec(hidden_size=H, vocab_size=V, embedding=PartSpec("tokens", {"vocab_size": V, "hidden_size": H}),
+                         embedding_prefix="toy.", layers=layers, schedule=[Run(i) for i in range(d["depth"])],
+                         final_norm=norm, final_norm_prefix="toy.norm.",
+                         head=PartSpec("linear", {"vocab_size": V, "hidden_size": H, "tied": True}), head_prefix="toy.head.")
+
+    register_part("mixer", "running_sum", RunningSum)
+    register_architecture("ToyForCausalLM", ToyConfig, toy_spec)
+    try:
+        d = {"architectures": ["ToyForCausalLM"], "width": 40, "vocab": 70, "inner": 56, "depth": 2,
+             "eps": 1e-5, "decay": 0.9}
+        cfg = config_from_dict(d)
+        spec = model_spec_for(cfg)
+        w = random_tensors(spec.weight_specs(), seed=1, std=0.2, dtype=torch.float32)
+        assert "toy.1.mix.weight" in w and "toy.head.weight" not in w
+        model = Model(spec, cfg, torch.float32, DEV)
+        model.load_weights(TensorDict(w))
+        eng = Engine(model, max_tokens=64 * 4, max_slots=3)
+        assert not eng.cache.groups and sorted(eng.cache.state) == [0, 1]
+        assert eng.cache.state[0].shape == (3, 40)
+
+        def plain_forward(ids):
+            wd = {k: v.double() for k, v in w.items()}
+            x = wd["toy.embed_tokens.weight"][ids]
+            for i in range(2):
+                y = plain.rmsnorm(x, wd[f"toy.{i}.input_layernorm.weight"], 1e-5)
+                s = torch.zeros(40, dtype=torch.float64)
+                add = []
+                for t in range(len(ids)):
+                    s = 0.9 * s + y[t]
+                    add.append(wd[f"toy.{i}.mix.weight"] @ s)
+                x = x + torch.stack(add)
+                x = x + plain.swiglu(plain.rmsnorm(x, wd[f"toy.{i}.post_attention_layernorm.weight"], 1e-5), wd, f"toy.{i}.")
+            return plain.rmsnorm(x, wd["toy.norm.weight"], 1e-5) @ wd["toy.embed_tokens.weight"].t()
+
+        g = torch.Generator().manual_seed(2)
+        a = torch.randint(0, 70, (12,), generator=g).tolist()
+        b = torch.randint(0, 70, (5,), generator=g).tolist()
+        wa, wb = plain_forward(a), plain_forward(b)
+        sa, sb = eng.alloc(), eng.alloc()
+        lg = eng.step([SeqInput(sa, a[:7], list(range(7))), SeqInput(sb, b[:2], [0, 1])]).clone()
+        got_a, got_b = [lg[:7]], [lg[7:]]
+        for t in range(3):
+            lg = eng.step([SeqInput(sa, [a[7 + t]], [0]), SeqInput(sb, [b[2 + t]], [0])]).clone()
+            got_a.append(lg[:1]); got_b.append(lg[1:])
+        eng.free(sb)
+        lg = eng.step([SeqInput(sa, a[10:], [0, 1])]).clone()
+        got_a.append(lg)
+        eng.free(sa)
+        assert rel_err(torch.cat(got_a), wa) < 1e-5 and rel_err(torch.cat(got_b), wb) < 1e-5
+        # the slot that is used again starts from a zeroed state
+        s2 = eng.alloc()
+        assert s2 in (sa, sb)
+        again = eng.step([SeqInput(s2, b, list(range(5)))]).clone()
+        eng.free(s2)
+        assert rel_err(again, wb) < 1e-5
+    finally:
+        unregister_part("mixer", "running_sum")
+        unregister_architecture("ToyForCausalLM")

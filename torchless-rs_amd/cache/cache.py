@@ -29,6 +29,7 @@ import torch
 from .pool import CacheFull, CacheMisuse, FreeList
 
 PAGE = 64
+NO_RING = 1 << 24          # "ring" of a group that keeps every position: never wraps
 
 
 @dataclass(frozen=True)
@@ -59,8 +60,8 @@ class KVGroup:
         self.runs = list(runs)
         self.layer_of_run = {r: i for i, r in enumerate(self.runs)}
         self.n_pages = n_pages
-        # pages one sequence can hold: a ring for a window, else everything
-        self.ring_pages = pages_for(request.window) if request.window else n_pages
+        # pages one sequence can hold: a ring for a window, else without bound (the pool is the limit)
+        self.ring_pages = pages_for(request.window) if request.window else NO_RING
         self.pool = FreeList(n_pages, "page")
         self.pages_of_slot: Dict[int, List[int]] = {}
         self.storage = None

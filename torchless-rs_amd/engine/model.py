@@ -38,7 +38,6 @@ class Model:
             if run.kv_from is not None and not (0 <= run.kv_from < i):
                 raise ValueError(f"schedule entry {i} reads the cache of entry {run.kv_from}, which "
                                  "is not an earlier one")
-        self.runs: List[RunBinding] = []
         self.loaded = False
 
     # ---- weights -----------------------------------------------------------
@@ -77,13 +76,12 @@ class Model:
 
     def make_cache(self, max_tokens: int, max_slots: Optional[int] = None, allocate: bool = True) -> Cache:
         kv, st = self.cache_requests()
-        cache = Cache(kv, st, max_tokens, self.dtype, self.device, max_slots, allocate)
-        self.bind_cache(cache)
-        return cache
+        return Cache(kv, st, max_tokens, self.dtype, self.device, max_slots, allocate)
 
-    def bind_cache(self, cache: Cache) -> None:
+    def bind_cache(self, cache: Cache) -> List[RunBinding]:
+        """Tie every run of the schedule to its place in `cache`."""
         read_later = {r.kv_from for r in self.spec.schedule if r.kv_from is not None}
-        self.runs = []
+        runs: List[RunBinding] = []
         for i, run in enumerate(self.spec.schedule):
             src = i if run.kv_from is None else run.kv_from
             b = RunBinding(index=i, kv_owner=run.kv_from is None, kv_source=src,
@@ -93,10 +91,12 @@ class Model:
                 b.kv_group, b.kv_layer = cache.kv_layer(src)
             elif run.kv_from is not None:
                 raise ValueError(f"schedule entry {i} reads the cache of entry {src}, which keeps none")
-            self.runs.append(b)
+            runs.append(b)
+        return runs
 
     # ---- one step ------------------------------------------------------------
-    def forward(self, ctx: StepContext, want_rows: Optional[torch.Tensor], n_want: int) -> torch.Tensor:
+    def forward(self, ctx: StepContext, runs: List[RunBinding], want_rows: Optional[torch.Tensor],
+                n_want: int) -> torch.Tensor:
         """Run the rows of `ctx` through the schedule and return float32 logits
         [n_want, V] at `want_rows` (int32 row indices on the device)."""
         if not self.loaded:
@@ -105,7 +105,7 @@ class Model:
         ws = ctx.workspace
         x = ws.get("residual", (ctx.n_rows, H), torch.float32)
         self.embedding.forward(ctx, ctx.tokens, x)
-        for run, binding in zip(self.spec.schedule, self.runs):
+        for run, binding in zip(self.spec.schedule, runs):
             self.blocks[run.layer].forward(ctx, binding, x)
         for commit in ctx.host.pop("deferred", []):
             commit()
