@@ -316,3 +316,47 @@ def test_draws_do_not_depend_on_batch_mates_and_follow_the_probabilities(ops):
     assert again == ids                                      # the seed decides
     other, _ = run_sample(ops, z.repeat(n, 1), 1.0, seed=6, counters=counters)
     assert other != ids
+
+
+# ---- bfloat16 products on the matrix cores -----------------------------------------
+
+@pytest.mark.parametrize("variant,M", [(1, 1), (1, 7), (1, 16), (4, 5), (2, 17), (2, 32), (3, 33), (3, 64),
+                                       (0, 1), (0, 70), (0, 128), (0, 300)])
+@pytest.mark.parametrize("N,K", [(50, 72), (16, 64), (130, 264), (200, 1000), (384, 96)])
+def test_gemm_bf16_kernels(ops, variant, M, N, K):
+    a = rnd(M, K, seed=21, dtype=torch.bfloat16)
+    w = rnd(N, K, seed=22, dtype=torch.bfloat16)
+    want = a.double() @ w.double().t()
+    out = torch.full((M, N), float("nan"), device=DEV)
+    ops.gemm_bf16(a.to(DEV), w.to(DEV), out, variant=variant)
+    assert rel_err(out, want) < 3e-6
+    base = rnd(M, N, seed=23)
+    acc = base.clone().to(DEV)
+    ops.gemm_bf16(a.to(DEV), w.to(DEV), acc, accumulate=True, variant=variant)
+    assert rel_err(acc, want + base.double()) < 3e-6
+
+
+def test_gemm_bf16_row_does_not_depend_on_the_batch(ops):
+    a = rnd(64, 512, seed=24, dtype=torch.bfloat16).to(DEV)
+    w = rnd(96, 512, seed=25, dtype=torch.bfloat16).to(DEV)
+    outs = {}
+    for M in (1, 9, 16, 17, 40, 64):
+        o = torch.empty(M, 96, device=DEV)
+        ops.gemm(a[:M].contiguous(), w, o)
+        outs[M] = o
+    for M in outs:
+        assert torch.equal(outs[M][0], outs[64][0])
+    big = torch.empty(64, 96, device=DEV)
+    ops.gemm_bf16(a, w, big, variant=0)
+    assert rel_err(big, outs[64]) < 1e-6                    # the tiled kernel agrees up to rounding
+    assert rel_err(outs[64], a.double().cpu() @ w.double().cpu().t()) < 3e-6
+
+
+def test_gemm_dispatch_falls_back_when_k_is_odd(ops):
+    a = rnd(3, 52, seed=26, dtype=torch.bfloat16)
+    w = rnd(20, 52, seed=27, dtype=torch.bfloat16)
+    out = torch.empty(3, 20, device=DEV)
+    ops.gemm(a.to(DEV), w.to(DEV), out)                     # 52 % 8 != 0: plain kernel
+    assert rel_err(out, a.double() @ w.double().t()) < 3e-6
+    with pytest.raises(ops.KernelError, match="multiple of 8"):
+        ops.gemm_bf16(a.to(DEV), w.to(DEV), out)

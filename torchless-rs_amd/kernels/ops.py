@@ -189,10 +189,32 @@ def sample(logits: torch.Tensor, temperature: float, top_k: int, top_p: float, s
                            _p(counters), _p(probs), _p(out), _stream()))
 
 
+def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False,
+              variant: Optional[int] = None) -> None:
+    """out[M,N] (+)= a[M,K] @ w[N,K]^T on the matrix cores: bfloat16 operands,
+    float32 accumulation.  K must be a multiple of 8.  `variant` (tests only)
+    forces one kernel: 0 tiled, 1..4 the skinny ones."""
+    M, K = a.shape
+    N = w.shape[0]
+    _req(a, "gemm.a", torch.bfloat16)
+    _req(w, "gemm.w", torch.bfloat16, (N, K))
+    _req(out, "gemm.out", torch.float32, (M, N))
+    if variant is None:
+        _check(lib().tl_gemm_bf16(_p(a), _p(w), _p(out), M, N, K, int(accumulate), _stream()))
+    else:
+        _check(lib().tl_gemm_bf16_variant(_p(a), _p(w), _p(out), M, N, K, int(accumulate), int(variant),
+                                          _stream()))
+
+
 def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
     """out[M,N] (+)= a[M,K] @ w[N,K]^T with float32 accumulation.  The kernel
-    follows from the operand types and the number of rows."""
-    gemm_plain(a, w, out, accumulate)
+    follows from the operand types: bfloat16 x bfloat16 goes to the matrix
+    cores, anything with float32 in it to the plain FMA kernel."""
+    if (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.shape[1] % 8 == 0
+            and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0):
+        gemm_bf16(a, w, out, accumulate)
+    else:
+        gemm_plain(a, w, out, accumulate)
 
 
 def attention(q, k_new, v_new, pages, table, ring_pages: int, ctx, n_cached, window, scale: float,
