@@ -147,7 +147,7 @@ def paged_case(ops, dt, nq, nkv, d, window, lens_cached, lens_new, seed=0, n_pag
         for p in range(max(0, lens_cached[b] - ring * PAGE), lens_cached[b]):
             pg = mine[(p // PAGE) % ring]
             pages[pg, 0, :, p % PAGE] = k[p]
-            pages[pg, 1, :, p % PAGE] = v[p]
+            pages[pg, 1].view(nkv, d, PAGE)[:, :, p % PAGE] = v[p]      # values lie transposed
         full = plain.attention_core(q.double(), k.double(), v.double(), torch.arange(T), window)
         want.append(full[lens_cached[b]:])
         q_rows.append(q[lens_cached[b]:]); k_rows.append(k[lens_cached[b]:]); v_rows.append(v[lens_cached[b]:])
@@ -197,7 +197,7 @@ def test_commit_of_a_chunk_longer_than_the_ring(ops):
     for p in range(310 - 128, 310):
         pg = int(table[0, (p // PAGE) % 2])
         assert torch.equal(pages[pg, 0, 0, p % PAGE], a["k"][p - 10, 0].cpu())
-        assert torch.equal(pages[pg, 1, 0, p % PAGE], a["v"][p - 10, 0].cpu())
+        assert torch.equal(pages[pg, 1].view(nkv, d, PAGE)[0, :, p % PAGE], a["v"][p - 10, 0].cpu())
 
 
 @pytest.mark.parametrize("dt", ["float32", "bfloat16"])
@@ -221,7 +221,7 @@ def test_a_far_key_among_hundreds_and_the_windows_edge(ops, dt):
         for p in range(max(0, T - ring * PAGE), T):
             pg = int(table[0, (p // PAGE) % ring])
             pages[pg, 0, :, p % PAGE] = k[p].to(tdt)
-            pages[pg, 1, :, p % PAGE] = v[p].to(tdt)
+            pages[pg, 1].view(nkv, d, PAGE)[:, :, p % PAGE] = v[p].to(tdt)
         out = torch.empty(1, nq, d, dtype=tdt, device=DEV)
         i32 = lambda l: torch.tensor(l, dtype=torch.int32, device=DEV)
         ops.attn_plain(q.to(tdt).to(DEV), None, None, pages.to(DEV), table.to(DEV), ring, i32([0]),
@@ -360,3 +360,81 @@ def test_gemm_dispatch_falls_back_when_k_is_odd(ops):
     assert rel_err(out, a.double() @ w.double().t()) < 3e-6
     with pytest.raises(ops.KernelError, match="multiple of 8"):
         ops.gemm_bf16(a.to(DEV), w.to(DEV), out)
+
+
+# ---- bfloat16 attention on the matrix cores -----------------------------------------
+
+SHAPES = [(4, 2, 16, None), (6, 1, 32, 70), (5, 5, 48, 8), (8, 2, 128, 100), (2, 1, 256, None),
+          (3, 3, 80, 64), (32, 8, 128, 200), (20, 1, 64, None), (4, 4, 160, 130)]
+
+
+@pytest.mark.parametrize("nq,nkv,d,window", SHAPES)
+def test_attention_prefill_bf16(ops, nq, nkv, d, window):
+    """Whole prompts, prompts that go on from cached context (page-aligned and not), rows that end
+    inside a block of 128, more than one block."""
+    a = paged_case(ops, "bfloat16", nq, nkv, d, window, lens_cached=[0, 5, 130, 64, 200, 0],
+                   lens_new=[17, 1, 3, 70, 129, 300], n_pages=60)
+    n_tiles = sum(-(-n // 128) for n in [17, 1, 3, 70, 129, 300])
+    ops.attn_prefill_bf16(a["q"], a["k"], a["v"], a["pages"], a["table"], a["ring"], a["row_pos"], a["cu"],
+                          a["cached"], n_tiles, window, a["scale"], a["out"])
+    assert rel_err(a["out"], a["want"]) < KTOL["bfloat16"]
+    plain_out = torch.empty_like(a["out"])
+    ops.attn_plain(a["q"], a["k"], a["v"], a["pages"], a["table"], a["ring"], a["row_seq"], a["row_pos"],
+                   a["cu"], a["cached"], window, a["scale"], plain_out)
+    assert rel_err(a["out"], plain_out.double()) < KTOL["bfloat16"]
+
+
+@pytest.mark.parametrize("splits", [1, 3, 8])
+@pytest.mark.parametrize("nq,nkv,d,window", SHAPES)
+def test_attention_decode_bf16(ops, nq, nkv, d, window, splits):
+    lens = [0, 63, 64, 300, 191, 31, 32, 700]
+    a = paged_case(ops, "bfloat16", nq, nkv, d, window, lens_cached=lens, lens_new=[1] * len(lens), seed=3,
+                   n_pages=60)
+    ops.kv_commit(a["k"], a["v"], a["row_seq"], a["row_pos"], a["after"], a["table"], a["ring"], a["pages"])
+    B = len(lens)
+    part = torch.full((B * nq * splits * (d + 2),), float("nan"), device=DEV)
+    ops.attn_decode_bf16(a["q"], a["pages"], a["table"], a["ring"], a["row_pos"], window, a["scale"], splits,
+                         part, a["out"])
+    assert rel_err(a["out"], a["want"]) < KTOL["bfloat16"]
+
+
+def test_attention_bf16_far_key_and_edge(ops):
+    """As for the plain kernel: a key that stands out far back, and the two sides of the window's
+    edge, through the decode and the prefill kernel."""
+    from torchless_rs_amd.cache import PAGE
+    nq, nkv, d, T = 4, 1, 64, 700
+    g = torch.Generator().manual_seed(5)
+    i32 = lambda l: torch.tensor(l, dtype=torch.int32, device=DEV)
+    for window, far, visible in [(None, 3, True), (200, 499, False), (200, 500, True), (200, 699, True)]:
+        k = torch.randn(T, nkv, d, generator=g) * 0.1
+        v = torch.randn(T, nkv, d, generator=g)
+        qv = torch.randn(d, generator=g)
+        qv = qv / qv.norm()
+        k[far, 0] = qv * 60.0
+        q = (qv * 8.0).view(1, 1, d).repeat(1, nq, 1).to(torch.bfloat16)
+        ring = -(-window // PAGE) if window else 11
+        pages = torch.full((11, 2, nkv, PAGE, d), float("nan"), dtype=torch.bfloat16)
+        table = torch.tensor([[7, 2, 9, 0, 5, 1, 10, 3, 8, 4, 6][:ring]], dtype=torch.int32)
+        for p in range(max(0, T - ring * PAGE), T):
+            pg = int(table[0, (p // PAGE) % ring])
+            pages[pg, 0, :, p % PAGE] = k[p].to(torch.bfloat16)
+            pages[pg, 1].view(nkv, d, PAGE)[:, :, p % PAGE] = v[p].to(torch.bfloat16)
+        out = torch.empty(1, nq, d, dtype=torch.bfloat16, device=DEV)
+        part = torch.empty(nq * 4 * (d + 2), device=DEV)
+        ops.attn_decode_bf16(q.to(DEV), pages.to(DEV), table.to(DEV), ring, i32([T - 1]), window,
+                             1.0 / math.sqrt(d), 4, part, out)
+        assert (rel_err(out[0, 0], v[far, 0].to(torch.bfloat16)) < 1e-2) == visible, (window, far)
+        assert torch.isfinite(out).all()
+        # the same through the prefill kernel: the last 2 rows are new, the rest is cached
+        pages2 = pages.clone()
+        for p in (T - 2, T - 1):
+            pg = int(table[0, (p // PAGE) % ring])
+            pages2[pg, :, :, :, :] = pages2[pg]          # (left as it is: rows >= n_cached are not read)
+        kn = k[T - 2:].to(torch.bfloat16).to(DEV)
+        vn = v[T - 2:].to(torch.bfloat16).to(DEV)
+        q2 = torch.cat([torch.zeros_like(q), q]).to(DEV)
+        out2 = torch.empty(2, nq, d, dtype=torch.bfloat16, device=DEV)
+        ops.attn_prefill_bf16(q2, kn, vn, pages2.to(DEV), table.to(DEV), ring, i32([T - 2, T - 1]), i32([0, 2]),
+                              i32([T - 2]), 1, window, 1.0 / math.sqrt(d), out2)
+        assert (rel_err(out2[1, 0], v[far, 0].to(torch.bfloat16)) < 1e-2) == visible, (window, far)
+        assert torch.isfinite(out2).all()

@@ -1,0 +1,480 @@
+// bfloat16 attention on the matrix cores: one kernel for steps that bring many
+// rows per sequence (prefill), one for single-token steps (decode).
+//
+// Visibility, scaling and softmax are those of the plain kernel (key j is seen
+// by the query at p iff j <= p and, with a window W, j > p - W; score =
+// (k.q) * scale; softmax with a running maximum), with the statistics in
+// float.  Both kernels compute the transposed products S^T = K Q^T and
+// O^T = V^T P^T: a lane then owns one query (or head) column, the softmax
+// over keys runs inside the lane, and the probabilities leave the first
+// product in exactly the register layout the second one takes.  The value
+// operand must be read along keys; pages store values transposed ([d][PAGE])
+// for that, and the prefill kernel transposes the step's own value rows on
+// their way into LDS.
+#include "common.hpp"
+
+namespace tl {
+
+__device__ __forceinline__ bf16x8 ld8(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
+__device__ __forceinline__ bf16x4 ld4(const bf16* p) { return *reinterpret_cast<const bf16x4*>(p); }
+__device__ __forceinline__ bf16x8 z8() {
+  bf16x8 z;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = (bf16)0.f;
+  return z;
+}
+
+// ------------------------------------------------------------------ prefill --
+// One workgroup: 128 consecutive new rows of one sequence (4 waves x 32) and
+// one query head.  Keys go by tiles of 64 positions; a tile is one cache page
+// where it lies below n_cached and rows of this step above.
+constexpr int PF_BM = 128, PF_BN = 64, PF_VLD = PF_BN + 4;
+
+template <int DPAD>
+__global__ void __launch_bounds__(256)
+attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
+                    const bf16* __restrict__ v_new, const bf16* __restrict__ pages,
+                    const int* __restrict__ table, int table_stride, int ring_pages,
+                    const int* __restrict__ row_pos, const int* __restrict__ cu_seqlens,
+                    const int* __restrict__ n_cached, int B, int nq, int nkv, int d, int window,
+                    float scale, bf16* __restrict__ out) {
+  constexpr int KB = DPAD / 16, VB = DPAD / 32, KLD = DPAD + 8, CH = DPAD / 8;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  bf16* Ks = reinterpret_cast<bf16*>(smem);          // [PF_BN][KLD]
+  bf16* Vt = Ks + PF_BN * KLD;                       // [DPAD][PF_VLD]
+
+  // which sequence and which block of its rows
+  int t = blockIdx.x, b = 0;
+  for (; b < B; ++b) {
+    const int tiles = (cu_seqlens[b + 1] - cu_seqlens[b] + PF_BM - 1) / PF_BM;
+    if (t < tiles) break;
+    t -= tiles;
+  }
+  if (b == B) return;
+  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64, l32 = lane % 32, half = lane / 32;
+  const int h = blockIdx.y, kvh = h / (nq / nkv);
+  const int row0 = cu_seqlens[b], n_new = cu_seqlens[b + 1] - row0;
+  const int cached = n_cached[b];
+  const int p_first = row_pos[row0];
+  const int qt0 = t * PF_BM;
+  const int qr = qt0 + wave * 32 + l32;               // this lane's query row among the new rows
+  const bool q_ok = qr < n_new;
+  const int p_me = p_first + qr;
+  const size_t head_elems = (size_t)PAGE * d, page_elems = 2 * (size_t)nkv * head_elems;
+
+  bf16x8 qreg[KB];
+  {
+    const bf16* qp = q + ((size_t)(row0 + min(qr, n_new - 1)) * nq + h) * d;
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb) {
+      const int k = kb * 16 + 8 * half;
+      qreg[kb] = (k + 8 <= d) ? ld8(qp + k) : z8();
+    }
+  }
+  f32x16 o[VB];
+#pragma unroll
+  for (int vb = 0; vb < VB; ++vb)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[vb][r] = 0.f;
+  float m = -INFINITY, l = 0.f;
+
+  const int p_lo = p_first + qt0, p_hi = p_first + min(qt0 + PF_BM, n_new) - 1;
+  const int pw_lo = p_lo + wave * 32, pw_hi = min(p_hi, pw_lo + 31);    // this wave's positions
+  const int j_lo = (window > 0 && p_lo - window + 1 > 0) ? p_lo - window + 1 : 0;
+
+  for (int jt = j_lo / PF_BN; jt * PF_BN <= p_hi; ++jt) {
+    const int j0 = jt * PF_BN;
+    __syncthreads();
+    if (j0 + PF_BN <= cached) {
+      // the tile is one cached page: keys row by row, values already transposed
+      const int page = table[(size_t)b * table_stride + (j0 / PAGE) % ring_pages];
+      const bf16* kbase = pages + (size_t)page * page_elems + (size_t)kvh * head_elems;
+      const bf16* vbase = kbase + (size_t)nkv * head_elems;
+      for (int c = tid; c < PF_BN * CH; c += 256) {
+        const int row = c / CH, col = (c % CH) * 8;
+        *reinterpret_cast<bf16x8*>(&Ks[row * KLD + col]) = (col < d) ? ld8(kbase + (size_t)row * d + col) : z8();
+      }
+      for (int c = tid; c < DPAD * (PF_BN / 8); c += 256) {
+        const int dv = c / (PF_BN / 8), kc = (c % (PF_BN / 8)) * 8;
+        const bf16x8 vv = (dv < d) ? ld8(vbase + (size_t)dv * PAGE + kc) : z8();
+        bf16x4 lo4, hi4;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          lo4[e] = vv[e];
+          hi4[e] = vv[4 + e];
+        }
+        *reinterpret_cast<bf16x4*>(&Vt[dv * PF_VLD + kc]) = lo4;
+        *reinterpret_cast<bf16x4*>(&Vt[dv * PF_VLD + kc + 4]) = hi4;
+      }
+    } else {
+      for (int c = tid; c < PF_BN * CH; c += 256) {
+        const int row = c / CH, col = (c % CH) * 8;
+        const int j = j0 + row;
+        bf16x8 kv = z8(), vv = z8();
+        if (j <= p_hi && col < d) {
+          if (j < cached) {
+            const int page = table[(size_t)b * table_stride + (j / PAGE) % ring_pages];
+            const bf16* base = pages + (size_t)page * page_elems + (size_t)kvh * head_elems;
+            kv = ld8(base + (size_t)(j % PAGE) * d + col);
+            const bf16* vp = base + (size_t)nkv * head_elems + (size_t)col * PAGE + (j % PAGE);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) vv[e] = vp[(size_t)e * PAGE];
+          } else {
+            const size_t r = ((size_t)(row0 + j - cached) * nkv + kvh) * d + col;
+            kv = ld8(k_new + r);
+            vv = ld8(v_new + r);
+          }
+        }
+        *reinterpret_cast<bf16x8*>(&Ks[row * KLD + col]) = kv;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) Vt[(col + e) * PF_VLD + row] = vv[e];
+      }
+    }
+    __syncthreads();
+    // does any query of this wave see any key of this tile?
+    if (pw_lo > p_hi || j0 > pw_hi || (window > 0 && j0 + PF_BN - 1 <= pw_lo - window)) continue;
+
+    f32x16 s[2];
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[nb][r] = 0.f;
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb) {
+        const bf16x8 a = *reinterpret_cast<const bf16x8*>(&Ks[(nb * 32 + l32) * KLD + kb * 16 + 8 * half]);
+        s[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[kb], s[nb], 0, 0, 0);
+      }
+    // s[nb][r] = score of key j0 + 32 nb + 8 (r/4) + 4 half + r%4 with this lane's query
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int j = j0 + nb * 32 + 8 * (r / 4) + 4 * half + (r % 4);
+        const bool ok = q_ok && j <= p_me && (window == 0 || j > p_me - window);
+        const float v = ok ? s[nb][r] * scale : -INFINITY;
+        s[nb][r] = v;
+        tmax = fmaxf(tmax, v);
+      }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
+    const float m_new = fmaxf(m, tmax);
+    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+    const float alpha = __expf(m - m_use);
+    float psum = 0.f;
+    bf16x8 pb[2][2];
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float pv = __expf(s[nb][r] - m_use);
+        psum += pv;
+        pb[nb][r / 8][r % 8] = (bf16)pv;
+      }
+    psum += __shfl_xor(psum, 32, WAVE);
+    l = l * alpha + psum;
+    m = m_new;
+#pragma unroll
+    for (int vb = 0; vb < VB; ++vb) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[vb][r] *= alpha;
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+        for (int mm = 0; mm < 2; ++mm) {
+          // probabilities r = 8 mm .. 8 mm + 7 are keys kk + 4 half + {0..3} and kk + 8 + 4 half + {0..3}
+          const int kk = nb * 32 + 16 * mm + 4 * half;
+          const bf16* vrow = &Vt[(vb * 32 + l32) * PF_VLD + kk];
+          const bf16x4 lo4 = ld4(vrow), hi4 = ld4(vrow + 8);
+          bf16x8 a;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            a[e] = lo4[e];
+            a[4 + e] = hi4[e];
+          }
+          o[vb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[nb][mm], o[vb], 0, 0, 0);
+        }
+    }
+  }
+  if (q_ok) {
+    bf16* op = out + ((size_t)(row0 + qr) * nq + h) * d;
+    const float inv = 1.0f / l;
+#pragma unroll
+    for (int vb = 0; vb < VB; ++vb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int dv = vb * 32 + 8 * (r / 4) + 4 * half + (r % 4);
+        if (dv < d) op[dv] = (bf16)(o[vb][r] * inv);
+      }
+  }
+}
+
+// ------------------------------------------------------------------- decode --
+// One query token per sequence, everything in the pages.  A workgroup owns one
+// (sequence, KV head, group of up to 16 query heads, split); its 4 waves take
+// the split's pages in turn, each page as two groups of 32 keys read straight
+// from global memory into MFMA operands.  Per wave: running (max, sum, O^T);
+// the waves meet in LDS and the workgroup writes one partial per head:
+// part[(b, h, split)] = (max, sum, O[d]).  dec_combine merges the splits.
+constexpr int DC_WAVES = 4;
+
+template <int DPAD>   // multiple of 32
+__global__ void __launch_bounds__(DC_WAVES * 64)
+attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
+                   const int* __restrict__ table, int table_stride, int ring_pages,
+                   const int* __restrict__ row_pos, int nq, int nkv, int d, int window, float scale,
+                   int n_splits, int head_groups, float* __restrict__ part) {
+  constexpr int KB = DPAD / 32, VB = DPAD / 16;
+  __shared__ float red_o[VB * 4 * 64];
+  __shared__ float red_ml[DC_WAVES][2][16];
+  const int g = nq / nkv;
+  const int hg = blockIdx.x % head_groups;
+  const int kvh = (blockIdx.x / head_groups) % nkv;
+  const int b = blockIdx.x / (head_groups * nkv);
+  const int split = blockIdx.y;
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64, li = lane % 16, kg = lane / 16;
+  const int hl = hg * 16 + li;                        // head within the KV group (column of S^T)
+  const bool h_ok = hl < g;
+  const int h = kvh * g + min(hl, g - 1);
+  const int p = row_pos[b];
+  const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  const int pg_lo = lo / PAGE, pg_hi = p / PAGE, n_pg = pg_hi - pg_lo + 1;
+  const int per = (n_pg + n_splits - 1) / n_splits;
+  const int my_lo = pg_lo + split * per, my_hi = min(pg_hi + 1, my_lo + per);   // [my_lo, my_hi)
+  const size_t head_elems = (size_t)PAGE * d, page_elems = 2 * (size_t)nkv * head_elems;
+
+  bf16x8 qreg[KB];
+  {
+    const bf16* qp = q + ((size_t)b * nq + h) * d;
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb) {
+      const int k = kb * 32 + 8 * kg;
+      qreg[kb] = (k + 8 <= d) ? ld8(qp + k) : z8();
+    }
+  }
+  f32x4 o[VB];
+#pragma unroll
+  for (int vb = 0; vb < VB; ++vb) o[vb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+
+  for (int pg = my_lo + wave; pg < my_hi; pg += DC_WAVES) {
+    const int page = table[(size_t)b * table_stride + pg % ring_pages];
+    const bf16* kbase = pages + (size_t)page * page_elems + (size_t)kvh * head_elems;
+    const bf16* vbase = kbase + (size_t)nkv * head_elems;
+#pragma unroll
+    for (int grp = 0; grp < 2; ++grp) {               // 32 keys at a time
+      const int j0 = pg * PAGE + grp * 32;
+      if (j0 > p || j0 + 31 < lo) continue;
+      // block bs holds keys j0 + 8 (i/4) + 4 bs + i%4 in its rows i: then a lane's 8 scores of
+      // the two blocks are 8 consecutive keys, j0 + 8 kg .. + 7
+      f32x4 s[2];
+#pragma unroll
+      for (int bs = 0; bs < 2; ++bs) {
+        s[bs] = f32x4{0.f, 0.f, 0.f, 0.f};
+        const bf16* krow = kbase + (size_t)(grp * 32 + 8 * (li / 4) + 4 * bs + (li % 4)) * d;
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) {
+          const int k = kb * 32 + 8 * kg;
+          const bf16x8 a = (k + 8 <= d) ? ld8(krow + k) : z8();
+          s[bs] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qreg[kb], s[bs], 0, 0, 0);
+        }
+      }
+      float sv[8];
+      float tmax = -INFINITY;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int j = j0 + 8 * kg + e;
+        const bool ok = j <= p && j >= lo;
+        sv[e] = ok ? s[e / 4][e % 4] * scale : -INFINITY;
+        tmax = fmaxf(tmax, sv[e]);
+      }
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, WAVE));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
+      const float m_new = fmaxf(m, tmax);              // finite: the group holds a visible key
+      const float alpha = __expf(m - m_new);
+      float psum = 0.f;
+      bf16x8 pb;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float pv = __expf(sv[e] - m_new);
+        psum += pv;
+        pb[e] = (bf16)pv;
+      }
+      psum += __shfl_xor(psum, 16, WAVE);
+      psum += __shfl_xor(psum, 32, WAVE);
+      l = l * alpha + psum;
+      m = m_new;
+      // O^T[dv][head] += V^T[dv][keys] P^T[keys][head]; values lie as [d][PAGE] in the page
+#pragma unroll
+      for (int vb = 0; vb < VB; ++vb) {
+        const int dv = vb * 16 + li;
+        bf16x8 a = (dv < d) ? ld8(vbase + (size_t)dv * PAGE + grp * 32 + 8 * kg) : z8();
+        if (j0 + 31 > p) {         // rows past the sequence's end were never written: 0 * garbage
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (j0 + 8 * kg + e > p) a[e] = (bf16)0.f;
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[vb][r] *= alpha;
+        o[vb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb, o[vb], 0, 0, 0);
+      }
+    }
+  }
+  // o[vb][r] = O[dv = 16 vb + 4 kg + r][head li]; m, l are per head li (equal in the 4 kg lanes).
+  // Merge the waves: common maximum, then wave after wave adds its scaled share in LDS.
+  if (kg == 0) {
+    red_ml[wave][0][li] = m;
+    red_ml[wave][1][li] = l;
+  }
+  __syncthreads();
+  float mm = -INFINITY;
+#pragma unroll
+  for (int w = 0; w < DC_WAVES; ++w) mm = fmaxf(mm, red_ml[w][0][li]);
+  const float f = (m == -INFINITY) ? 0.f : __expf(m - mm);
+  for (int w = 0; w < DC_WAVES; ++w) {
+    if (wave == w) {
+#pragma unroll
+      for (int vb = 0; vb < VB; ++vb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float* dst = &red_o[(vb * 4 + r) * 64 + lane];
+          *dst = (w == 0) ? o[vb][r] * f : *dst + o[vb][r] * f;
+        }
+    }
+    __syncthreads();
+  }
+  for (int e = threadIdx.x; e < 16 * DPAD; e += DC_WAVES * 64) {
+    const int hd = e / DPAD, dv = e % DPAD;
+    if (hg * 16 + hd >= g || dv >= d) continue;
+    float mh = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < DC_WAVES; ++w) mh = fmaxf(mh, red_ml[w][0][hd]);
+    float ll = 0.f;
+#pragma unroll
+    for (int w = 0; w < DC_WAVES; ++w) {
+      const float mw = red_ml[w][0][hd];
+      ll += (mw == -INFINITY) ? 0.f : red_ml[w][1][hd] * __expf(mw - mh);
+    }
+    const int idx = ((dv / 16) * 4 + (dv % 4)) * 64 + ((dv % 16) / 4) * 16 + hd;
+    float* dst = part + (((size_t)b * nq + kvh * g + hg * 16 + hd) * n_splits + split) * (d + 2);
+    dst[2 + dv] = red_o[idx];
+    if (dv == 0) {
+      dst[0] = mh;
+      dst[1] = ll;
+    }
+  }
+}
+
+__global__ void __launch_bounds__(64)
+attn_decode_combine_kernel(const float* __restrict__ part, int n_splits, int d, bf16* __restrict__ out) {
+  const size_t bh = blockIdx.x;
+  const float* src = part + bh * n_splits * (d + 2);
+  float mm = -INFINITY;
+  for (int s = 0; s < n_splits; ++s) mm = fmaxf(mm, src[(size_t)s * (d + 2)]);
+  float ll = 0.f;
+  for (int s = 0; s < n_splits; ++s) {
+    const float ms = src[(size_t)s * (d + 2)];
+    ll += (ms == -INFINITY) ? 0.f : src[(size_t)s * (d + 2) + 1] * __expf(ms - mm);
+  }
+  for (int dv = threadIdx.x; dv < d; dv += 64) {
+    float acc = 0.f;
+    for (int s = 0; s < n_splits; ++s) {
+      const float ms = src[(size_t)s * (d + 2)];
+      if (ms != -INFINITY) acc += src[(size_t)s * (d + 2) + 2 + dv] * __expf(ms - mm);
+    }
+    out[bh * d + dv] = (bf16)(acc / ll);
+  }
+}
+
+template <int DPAD>
+static int launch_prefill(const bf16* q, const bf16* k_new, const bf16* v_new, const bf16* pages,
+                          const int* table, int table_stride, int ring_pages, const int* row_pos,
+                          const int* cu_seqlens, const int* n_cached, int B, int n_tiles, int nq, int nkv,
+                          int d, int window, float scale, bf16* out, hipStream_t st) {
+  const size_t smem = ((size_t)PF_BN * (DPAD + 8) + (size_t)DPAD * PF_VLD) * sizeof(bf16);
+  if (smem > 48 * 1024) {
+    static bool raised = false;
+    if (!raised) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prefill_kernel<DPAD>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+      if (e != hipSuccess) {
+        set_error("attn_prefill: cannot have %zu bytes of LDS: %s", smem, hipGetErrorString(e));
+        return 2;
+      }
+      raised = true;
+    }
+  }
+  dim3 grid(n_tiles, nq);
+  attn_prefill_kernel<DPAD><<<grid, 256, smem, st>>>(q, k_new, v_new, pages, table, table_stride,
+                                                     ring_pages, row_pos, cu_seqlens, n_cached, B, nq,
+                                                     nkv, d, window, scale, out);
+  TL_LAUNCH_CHECK("attn_prefill");
+  return 0;
+}
+
+template <int DPAD>
+static int launch_decode(const bf16* q, const bf16* pages, const int* table, int table_stride,
+                         int ring_pages, const int* row_pos, int B, int nq, int nkv, int d, int window,
+                         float scale, int n_splits, float* part, bf16* out, hipStream_t st) {
+  const int g = nq / nkv, head_groups = (g + 15) / 16;
+  dim3 grid(B * nkv * head_groups, n_splits);
+  attn_decode_kernel<DPAD><<<grid, DC_WAVES * 64, 0, st>>>(q, pages, table, table_stride, ring_pages,
+                                                            row_pos, nq, nkv, d, window, scale, n_splits,
+                                                            head_groups, part);
+  TL_LAUNCH_CHECK("attn_decode");
+  attn_decode_combine_kernel<<<B * nq, 64, 0, st>>>(part, n_splits, d, out);
+  TL_LAUNCH_CHECK("attn_decode_combine");
+  return 0;
+}
+
+}  // namespace tl
+
+using namespace tl;
+
+#define TL_BY_DPAD(fn, ...)                                          \
+  switch ((d + 31) / 32) {                                           \
+    case 1: return fn<32>(__VA_ARGS__);                              \
+    case 2: return fn<64>(__VA_ARGS__);                              \
+    case 3: return fn<96>(__VA_ARGS__);                              \
+    case 4: return fn<128>(__VA_ARGS__);                             \
+    case 5: return fn<160>(__VA_ARGS__);                             \
+    case 6: return fn<192>(__VA_ARGS__);                             \
+    case 7: return fn<224>(__VA_ARGS__);                             \
+    case 8: return fn<256>(__VA_ARGS__);                             \
+  }
+
+extern "C" int tl_attn_prefill_bf16(const void* q, const void* k_new, const void* v_new,
+                                    const void* pages, const int* table, int table_stride,
+                                    int ring_pages, const int* row_pos, const int* cu_seqlens,
+                                    const int* n_cached, int B, int n_tiles, int nq, int nkv, int d,
+                                    int window, float scale, void* out, hipStream_t st) {
+  TL_REQUIRE(B > 0 && n_tiles > 0 && nq > 0 && nkv > 0 && nq % nkv == 0 && nq <= 65535,
+             "attn_prefill: bad sizes B=%d tiles=%d nq=%d nkv=%d", B, n_tiles, nq, nkv);
+  TL_REQUIRE(d >= 16 && d <= 256 && d % 16 == 0, "attn_prefill: head size %d is not served "
+             "(multiples of 16 up to 256)", d);
+  TL_REQUIRE(ring_pages > 0 && table_stride > 0 && window >= 0,
+             "attn_prefill: bad cache geometry ring_pages=%d table_stride=%d window=%d", ring_pages,
+             table_stride, window);
+  TL_BY_DPAD(launch_prefill, (const bf16*)q, (const bf16*)k_new, (const bf16*)v_new,
+             (const bf16*)pages, table, table_stride, ring_pages, row_pos, cu_seqlens, n_cached, B,
+             n_tiles, nq, nkv, d, window, scale, (bf16*)out, st);
+  return 1;
+}
+
+// part: float scratch of B * nq * n_splits * (d + 2) elements
+extern "C" int tl_attn_decode_bf16(const void* q, const void* pages, const int* table, int table_stride,
+                                   int ring_pages, const int* row_pos, int B, int nq, int nkv, int d,
+                                   int window, float scale, int n_splits, float* part, void* out,
+                                   hipStream_t st) {
+  TL_REQUIRE(B > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attn_decode: bad sizes B=%d nq=%d nkv=%d", B,
+             nq, nkv);
+  TL_REQUIRE(d >= 16 && d <= 256 && d % 16 == 0, "attn_decode: head size %d is not served "
+             "(multiples of 16 up to 256)", d);
+  TL_REQUIRE(ring_pages > 0 && table_stride > 0 && window >= 0 && n_splits > 0 && n_splits <= 65535,
+             "attn_decode: bad geometry ring_pages=%d table_stride=%d window=%d splits=%d", ring_pages,
+             table_stride, window, n_splits);
+  TL_BY_DPAD(launch_decode, (const bf16*)q, (const bf16*)pages, table, table_stride, ring_pages, row_pos,
+             B, nq, nkv, d, window, scale, n_splits, part, (bf16*)out, st);
+  return 1;
+}

@@ -26,6 +26,7 @@ attn_plain_kernel(const T* __restrict__ q, const T* __restrict__ k_new, const T*
   __shared__ float q_s[MAX_D];
   __shared__ float p_s[WAVE];
   __shared__ const T* v_s[WAVE];
+  __shared__ int vstride_s[WAVE];
   const int n = blockIdx.x / nq, h = blockIdx.x % nq;
   const int lane = threadIdx.x;
   const int b = row_seq[n], p = row_pos[n];
@@ -50,12 +51,14 @@ attn_plain_kernel(const T* __restrict__ q, const T* __restrict__ k_new, const T*
     const int j = j0 + lane;
     float s = -INFINITY;
     const T* vp = nullptr;
+    int vstride = 1;                 // values: [d][PAGE] in a page, [d] in the step's rows
     if (j <= p) {
       const T* kp;
       if (j < cached) {
         const int page = table[(size_t)b * table_stride + (j / PAGE) % ring_pages];
         kp = pages + (size_t)page * page_elems + (size_t)kvh * head_elems + (size_t)(j % PAGE) * d;
-        vp = kp + v_off;
+        vp = pages + (size_t)page * page_elems + v_off + (size_t)kvh * head_elems + (j % PAGE);
+        vstride = PAGE;
       } else {
         const size_t r = ((size_t)(row0 + j - cached) * nkv + kvh) * d;
         kp = k_new + r;
@@ -73,6 +76,7 @@ attn_plain_kernel(const T* __restrict__ q, const T* __restrict__ k_new, const T*
     __syncthreads();
     p_s[lane] = pj;
     v_s[lane] = vp;
+    vstride_s[lane] = vstride;
     __syncthreads();
     const int cnt = (p - j0 + 1 < WAVE) ? p - j0 + 1 : WAVE;
 #pragma unroll
@@ -80,7 +84,7 @@ attn_plain_kernel(const T* __restrict__ q, const T* __restrict__ k_new, const T*
       const int dim = lane + WAVE * i;
       if (dim < d) {
         float a = acc[i] * alpha;
-        for (int jj = 0; jj < cnt; ++jj) a = fmaf(p_s[jj], to_f32(v_s[jj][dim]), a);
+        for (int jj = 0; jj < cnt; ++jj) a = fmaf(p_s[jj], to_f32(v_s[jj][(size_t)dim * vstride_s[jj]]), a);
         acc[i] = a;
       }
     }

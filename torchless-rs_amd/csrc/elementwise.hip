@@ -77,7 +77,9 @@ __global__ void rope_split_kernel(const float* __restrict__ qkv, const int* __re
 // ---- commit keys and values of this step to the pages -----------------------
 // Position p of sequence b goes to page table[b][(p / PAGE) % ring_pages], row
 // p % PAGE.  Rows that would be overwritten within this same step (older than
-// the last ring_pages * PAGE positions) are skipped.
+// the last ring_pages * PAGE positions) are skipped.  A page holds, per KV
+// head, keys as [PAGE][d] and values transposed as [d][PAGE], so that both
+// are read along their contraction index by the matrix cores.
 template <typename T>
 __global__ void kv_commit_kernel(const T* __restrict__ k, const T* __restrict__ v,
                                  const int* __restrict__ row_seq, const int* __restrict__ row_pos,
@@ -96,9 +98,8 @@ __global__ void kv_commit_kernel(const T* __restrict__ k, const T* __restrict__ 
   const T* vs = v + (size_t)n * nkv * d;
   for (int t = threadIdx.x; t < nkv * d; t += blockDim.x) {
     const int h = t / d, i = t % d;
-    const size_t o = ((size_t)h * PAGE + r) * d + i;
-    kd[o] = ks[t];
-    vd[o] = vs[t];
+    kd[((size_t)h * PAGE + r) * d + i] = ks[t];
+    vd[((size_t)h * d + i) * PAGE + r] = vs[t];
   }
 }
 

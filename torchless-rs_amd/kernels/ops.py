@@ -217,9 +217,84 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
         gemm_plain(a, w, out, accumulate)
 
 
+def attn_prefill_bf16(q, k_new, v_new, pages, table, ring_pages: int, row_pos, cu_seqlens, n_cached,
+                      n_tiles: int, window: Optional[int], scale: float, out) -> None:
+    """bfloat16 attention for steps with many rows per sequence.  `n_tiles`:
+    sum over the sequences of ceil(rows / 128)."""
+    n, nq, d = q.shape
+    nkv = pages.shape[2]
+    B = n_cached.shape[0]
+    _req(q, "attn.q", torch.bfloat16)
+    _req(k_new, "attn.k_new", torch.bfloat16, (n, nkv, d))
+    _req(v_new, "attn.v_new", torch.bfloat16, (n, nkv, d))
+    _req(pages, "attn.pages", torch.bfloat16)
+    if pages.dim() != 5 or tuple(pages.shape[1:]) != (2, nkv, 64, d):
+        raise KernelError(f"attn.pages: shape {tuple(pages.shape)}, kernel needs [*, 2, nkv, 64, {d}]")
+    _req(table, "attn.table", torch.int32)
+    _req(row_pos, "attn.row_pos", torch.int32, (n,))
+    _req(cu_seqlens, "attn.cu_seqlens", torch.int32, (B + 1,))
+    _req(n_cached, "attn.n_cached", torch.int32, (B,))
+    _req(out, "attn.out", torch.bfloat16, (n, nq, d))
+    if table.dim() != 2 or table.shape[0] != B:
+        raise KernelError("attn.table: needs one row per sequence")
+    _check(lib().tl_attn_prefill_bf16(_p(q), _p(k_new), _p(v_new), _p(pages), _p(table), table.shape[1],
+                                      ring_pages, _p(row_pos), _p(cu_seqlens), _p(n_cached), B,
+                                      int(n_tiles), nq, nkv, d, int(window or 0), ctypes.c_float(scale),
+                                      _p(out), _stream()))
+
+
+def attn_decode_bf16(q, pages, table, ring_pages: int, row_pos, window: Optional[int], scale: float,
+                     n_splits: int, part, out) -> None:
+    """bfloat16 attention of one new token per sequence over its pages (the
+    token's own key is already committed).  `part`: float32 scratch of at
+    least B * nq * n_splits * (d + 2) elements."""
+    B, nq, d = q.shape
+    nkv = pages.shape[2]
+    _req(q, "attn.q", torch.bfloat16)
+    _req(pages, "attn.pages", torch.bfloat16)
+    if pages.dim() != 5 or tuple(pages.shape[1:]) != (2, nkv, 64, d):
+        raise KernelError(f"attn.pages: shape {tuple(pages.shape)}, kernel needs [*, 2, nkv, 64, {d}]")
+    _req(table, "attn.table", torch.int32)
+    _req(row_pos, "attn.row_pos", torch.int32, (B,))
+    _req(part, "attn.part", torch.float32)
+    _req(out, "attn.out", torch.bfloat16, (B, nq, d))
+    if table.dim() != 2 or table.shape[0] != B:
+        raise KernelError("attn.table: needs one row per sequence")
+    if part.numel() < B * nq * n_splits * (d + 2):
+        raise KernelError(f"attn.part: {part.numel()} elements, kernel needs {B * nq * n_splits * (d + 2)}")
+    _check(lib().tl_attn_decode_bf16(_p(q), _p(pages), _p(table), table.shape[1], ring_pages, _p(row_pos),
+                                     B, nq, nkv, d, int(window or 0), ctypes.c_float(scale),
+                                     int(n_splits), _p(part), _p(out), _stream()))
+
+
+def decode_splits(B: int, nq: int, nkv: int, max_pages: int) -> int:
+    """Into how many parts the keys of a decode step are cut so that the chip
+    has some two workgroups a compute unit to run."""
+    groups = B * nkv * (-(-(nq // nkv) // 16))
+    return max(1, min(max_pages, -(-512 // groups)))
+
+
 def attention(q, k_new, v_new, pages, table, ring_pages: int, ctx, n_cached, window, scale: float,
               out) -> None:
-    """Attention of a step's rows (see `attn_plain` for the operands); `ctx`
-    brings the step's row and sequence indices."""
-    attn_plain(q, k_new, v_new, pages, table, ring_pages, ctx.row_seq, ctx.row_pos, ctx.cu_seqlens,
-               n_cached, window, scale, out)
+    """Attention of a step's rows: keys j < n_cached[b] from the pages, later
+    ones from this step's rows (`k_new`/`v_new`; None when everything is in
+    the pages).  bfloat16 with head sizes in steps of 16 runs on the matrix
+    cores, single-token steps and steps with longer rows each in their own
+    kernel; everything else runs in the plain kernel."""
+    n, nq, d = q.shape
+    fast = q.dtype == torch.bfloat16 and d % 16 == 0 and 16 <= d <= 256
+    if fast and k_new is None and ctx.all_single:
+        nkv = pages.shape[2]
+        max_pages = min(-(-ctx.max_len_after // 64), ring_pages)
+        if window:
+            max_pages = min(max_pages, -(-window // 64) + 1)
+        splits = decode_splits(n, nq, nkv, max_pages)
+        part = ctx.workspace.get("attn_part", (n * nq * splits * (d + 2),), torch.float32)
+        attn_decode_bf16(q, pages, table, ring_pages, ctx.row_pos, window, scale, splits, part, out)
+    elif fast and k_new is not None:
+        n_tiles = int(sum(-(-int(x) // 128) for x in ctx.host["n_new"]))
+        attn_prefill_bf16(q, k_new, v_new, pages, table, ring_pages, ctx.row_pos, ctx.cu_seqlens,
+                          n_cached, n_tiles, window, scale, out)
+    else:
+        attn_plain(q, k_new, v_new, pages, table, ring_pages, ctx.row_seq,
+                   ctx.row_pos, ctx.cu_seqlens, n_cached, window, scale, out)
