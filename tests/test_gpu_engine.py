@@ -352,3 +352,36 @@ def test_command_line(zoo):
     assert r.returncode == 0, r.stderr[-2000:]
     rows = [[int(t) for t in l.split()] for l in r.stdout.strip().split("\n")]
     assert rows == [plain.generate_greedy(z["w"], z["cfg"], p, 5)[0] for p in ([3, 1, 4, 1, 5], [9, 2, 6])]
+
+
+# ---- captured graphs ---------------------------------------------------------------
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_graph_replays_equal_eager_steps(zoo, dtype):
+    """Single-token steps are captured as a graph the second time their shape is seen.  Every
+    replay is checked against an engine that never captures, with eager prefill steps of other
+    sequences and synchronisations between the replays."""
+    from torchless_rs_amd.engine import Engine, SeqInput, load_model
+    z = zoo["C"]
+    model = load_model(z["dir"], dtype)
+    eng_g = Engine(model, max_tokens=64 * 16, max_slots=6, use_graphs=True)
+    eng_e = Engine(model, max_tokens=64 * 16, max_slots=6, use_graphs=False)
+    ids = prompts(z["cfg"]["vocab_size"], [90, 140, 75], seed=5)
+    for eng in (eng_g, eng_e):
+        eng.slots_ = [eng.alloc() for _ in ids]
+        eng.step([SeqInput(s, p[:10], []) for s, p in zip(eng.slots_, ids)])
+    replays = 0
+    for t in range(10, 75):
+        outs = []
+        for eng in (eng_g, eng_e):
+            outs.append(eng.step([SeqInput(s, [p[t]], [0]) for s, p in zip(eng.slots_, ids)]).clone())
+            if t % 7 == 0:                                # eager work of another sequence in between
+                extra = eng.alloc()
+                eng.step([SeqInput(extra, ids[1][:t], [t - 1])])
+                eng.free(extra)
+            torch.cuda.synchronize()
+        assert torch.equal(outs[0], outs[1]), t
+        replays += any(g.graph is not None for g in eng_g._graphs.values())
+    assert replays > 50 and not eng_e._graphs
+    want = plain.forward(z["w"], z["cfg"], ids[0][:75])[74:75]
+    assert rel_err(outs[0][:1], want) < TOL[dtype]

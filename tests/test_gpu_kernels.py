@@ -72,6 +72,17 @@ def test_rope_split(ops, dt, nq, nkv, d, theta):
         assert rel_err(q[r], wq[r]) < tol and rel_err(k[r], wk[r]) < tol, (r, p)
     assert rel_err(v, wv) < KTOL[dt]
     assert torch.equal(q[0].float().cpu(), qkv[0, :nq * d].view(nq, d).to(DT[dt]).float())   # pos 0: identity
+    # the values also transposed: two sequences of 2 and 4 rows, the second going on from 70 cached
+    pos2 = torch.tensor([0, 1, 70, 71, 72, 73], dtype=torch.int32, device=DEV)
+    seq2 = torch.tensor([0, 0, 1, 1, 1, 1], dtype=torch.int32, device=DEV)
+    off, cols = ops.aligned_columns([0, 70], [2, 4])
+    assert (off, cols) == ([0, 64], 128)
+    vt = torch.full((nkv, d, cols), 7.0, dtype=DT[dt], device=DEV)
+    ops.rope_split(qkv.to(DEV), pos2, Rotary(d, theta).inv_freq(DEV), nq, nkv, d, q, k, v, vt, seq2,
+                   torch.tensor(off, dtype=torch.int32, device=DEV), torch.tensor([0, 70], dtype=torch.int32, device=DEV))
+    for r, col in enumerate([0, 1, 64 + 6, 64 + 7, 64 + 8, 64 + 9]):
+        assert torch.equal(vt[:, :, col], v[r])
+    assert int((vt == 7.0).sum()) == nkv * d * (cols - 6)
 
 
 @pytest.mark.parametrize("dt", ["float32", "bfloat16"])
@@ -320,8 +331,9 @@ def test_draws_do_not_depend_on_batch_mates_and_follow_the_probabilities(ops):
 
 # ---- bfloat16 products on the matrix cores -----------------------------------------
 
-@pytest.mark.parametrize("variant,M", [(1, 1), (1, 7), (1, 16), (4, 5), (2, 17), (2, 32), (3, 33), (3, 64),
-                                       (0, 1), (0, 70), (0, 128), (0, 300)])
+@pytest.mark.parametrize("variant,M", [(112, 1), (112, 7), (111, 16), (212, 3), (411, 5), (222, 17), (222, 32),
+                                       (421, 20), (242, 33), (441, 64), (142, 50), (0, 1), (0, 70), (0, 128),
+                                       (0, 300), (1, 3), (1, 129), (1, 300), (1, 600)])
 @pytest.mark.parametrize("N,K", [(50, 72), (16, 64), (130, 264), (200, 1000), (384, 96)])
 def test_gemm_bf16_kernels(ops, variant, M, N, K):
     a = rnd(M, K, seed=21, dtype=torch.bfloat16)
@@ -368,6 +380,20 @@ SHAPES = [(4, 2, 16, None), (6, 1, 32, 70), (5, 5, 48, 8), (8, 2, 128, 100), (2,
           (3, 3, 80, 64), (32, 8, 128, 200), (20, 1, 64, None), (4, 4, 160, 130)]
 
 
+def transposed_values(ops, a, lens_cached, lens_new):
+    """The step's values as the prefill kernel takes them: [nkv, d, columns], poisoned elsewhere."""
+    off, cols = ops.aligned_columns(lens_cached, lens_new)
+    v = a["v"].cpu()
+    n, nkv, d = v.shape
+    vt = torch.full((nkv, d, cols), float("nan"), dtype=v.dtype)
+    r = 0
+    for b, (c, nn) in enumerate(zip(lens_cached, lens_new)):
+        for i in range(nn):
+            vt[:, :, off[b] + (c % 64) + i] = v[r]
+            r += 1
+    return vt.to(DEV), torch.tensor(off, dtype=torch.int32, device=DEV)
+
+
 @pytest.mark.parametrize("nq,nkv,d,window", SHAPES)
 def test_attention_prefill_bf16(ops, nq, nkv, d, window):
     """Whole prompts, prompts that go on from cached context (page-aligned and not), rows that end
@@ -375,7 +401,8 @@ def test_attention_prefill_bf16(ops, nq, nkv, d, window):
     a = paged_case(ops, "bfloat16", nq, nkv, d, window, lens_cached=[0, 5, 130, 64, 200, 0],
                    lens_new=[17, 1, 3, 70, 129, 300], n_pages=60)
     n_tiles = sum(-(-n // 128) for n in [17, 1, 3, 70, 129, 300])
-    ops.attn_prefill_bf16(a["q"], a["k"], a["v"], a["pages"], a["table"], a["ring"], a["row_pos"], a["cu"],
+    vt, off = transposed_values(ops, a, [0, 5, 130, 64, 200, 0], [17, 1, 3, 70, 129, 300])
+    ops.attn_prefill_bf16(a["q"], a["k"], vt, off, a["pages"], a["table"], a["ring"], a["row_pos"], a["cu"],
                           a["cached"], n_tiles, window, a["scale"], a["out"])
     assert rel_err(a["out"], a["want"]) < KTOL["bfloat16"]
     plain_out = torch.empty_like(a["out"])
@@ -426,15 +453,56 @@ def test_attention_bf16_far_key_and_edge(ops):
         assert (rel_err(out[0, 0], v[far, 0].to(torch.bfloat16)) < 1e-2) == visible, (window, far)
         assert torch.isfinite(out).all()
         # the same through the prefill kernel: the last 2 rows are new, the rest is cached
-        pages2 = pages.clone()
-        for p in (T - 2, T - 1):
-            pg = int(table[0, (p // PAGE) % ring])
-            pages2[pg, :, :, :, :] = pages2[pg]          # (left as it is: rows >= n_cached are not read)
+        pages2 = pages.clone()                            # rows >= n_cached are there but are not read
         kn = k[T - 2:].to(torch.bfloat16).to(DEV)
         vn = v[T - 2:].to(torch.bfloat16).to(DEV)
         q2 = torch.cat([torch.zeros_like(q), q]).to(DEV)
         out2 = torch.empty(2, nq, d, dtype=torch.bfloat16, device=DEV)
-        ops.attn_prefill_bf16(q2, kn, vn, pages2.to(DEV), table.to(DEV), ring, i32([T - 2, T - 1]), i32([0, 2]),
-                              i32([T - 2]), 1, window, 1.0 / math.sqrt(d), out2)
+        off, cols = ops.aligned_columns([T - 2], [2])
+        vt = torch.full((nkv, d, cols), float("nan"), dtype=torch.bfloat16, device=DEV)
+        vt[:, :, (T - 2) % 64] = vn[0]
+        vt[:, :, (T - 2) % 64 + 1] = vn[1]
+        ops.attn_prefill_bf16(q2, kn, vt, i32(off), pages2.to(DEV), table.to(DEV), ring, i32([T - 2, T - 1]),
+                              i32([0, 2]), i32([T - 2]), 1, window, 1.0 / math.sqrt(d), out2)
         assert (rel_err(out2[1, 0], v[far, 0].to(torch.bfloat16)) < 1e-2) == visible, (window, far)
         assert torch.isfinite(out2).all()
+
+
+@pytest.mark.parametrize("variant,M", [(411, 1), (411, 9), (421, 30), (441, 64), (0, 5), (0, 200), (1, 7), (1, 520)])
+@pytest.mark.parametrize("I,K", [(64, 72), (160, 64), (96, 200)])
+def test_gemm_bf16_paired_silu_epilogue(ops, variant, M, I, K):
+    """gate and up rows interleaved in groups of 32: the product writes silu(gate) * up."""
+    from torchless_rs_amd.parts.linear import interleave_pairs
+    a = rnd(M, K, seed=31, dtype=torch.bfloat16)
+    g = rnd(I, K, seed=32, dtype=torch.bfloat16, scale=0.3)
+    u = rnd(I, K, seed=33, dtype=torch.bfloat16, scale=0.3)
+    w = interleave_pairs(g, u)
+    assert torch.equal(w[:32], g[:32]) and torch.equal(w[32:64], u[:32]) and torch.equal(w[64:96], g[32:64])
+    want = plain.silu(a.double() @ g.double().t()) * (a.double() @ u.double().t())
+    out = torch.full((M, I), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.gemm_bf16(a.to(DEV), w.to(DEV), out, variant=variant, silu_pair=True)
+    assert rel_err(out, want) < KTOL["bfloat16"]
+    out2 = torch.empty_like(out)
+    ops.gemm_bf16(a.to(DEV), w.to(DEV), out2, silu_pair=True)           # the kernel the size picks
+    assert rel_err(out2, want) < KTOL["bfloat16"]
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("window", [None, 70])
+def test_rope_commit_equals_rope_split_then_commit(ops, dt, window):
+    from torchless_rs_amd.parts.position import Rotary
+    nq, nkv, d = 6, 2, 48
+    a = paged_case(ops, dt, nq, nkv, d, window, lens_cached=[0, 63, 64, 300], lens_new=[1] * 4, seed=7)
+    n = 4
+    qkv = rnd(n, (nq + 2 * nkv) * d, seed=8).to(DEV)
+    inv = Rotary(d, 777.0).inv_freq(DEV)
+    q1, k1, v1 = (torch.empty(n, h, d, dtype=DT[dt], device=DEV) for h in (nq, nkv, nkv))
+    ops.rope_split(qkv, a["row_pos"], inv, nq, nkv, d, q1, k1, v1)
+    pages1 = a["pages"].clone()
+    ops.kv_commit(k1, v1, a["row_seq"], a["row_pos"], a["after"], a["table"], a["ring"], pages1)
+    q2 = torch.empty_like(q1)
+    pages2 = a["pages"].clone()
+    ops.rope_commit(qkv, a["row_pos"], inv, a["table"], a["ring"], nq, nkv, d, q2, pages2)
+    assert torch.equal(q1, q2)
+    assert torch.equal(torch.nan_to_num(pages1.float(), nan=-7.0), torch.nan_to_num(pages2.float(), nan=-7.0))
+    assert not torch.equal(torch.nan_to_num(pages2.float(), nan=-7.0), torch.nan_to_num(a["pages"].float(), nan=-7.0))

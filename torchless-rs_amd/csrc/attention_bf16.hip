@@ -26,25 +26,30 @@ __device__ __forceinline__ bf16x8 z8() {
 
 // ------------------------------------------------------------------ prefill --
 // One workgroup: 128 consecutive new rows of one sequence (4 waves x 32) and
-// one query head.  Keys go by tiles of 64 positions; a tile is one cache page
-// where it lies below n_cached and rows of this step above.
+// one query head.  Keys go by tiles of 64 positions (aligned to 64, so a tile
+// below n_cached is one cache page).  The step's own values come transposed,
+// vt_new[kv head][d][column], column = tile_off[b] + (position - 64 *
+// (n_cached[b] / 64)): positions that are multiples of 64 lie on columns that
+// are, so tiles are read with aligned 16-byte loads.  The next tile is
+// fetched into registers while the current one is worked on.
 constexpr int PF_BM = 128, PF_BN = 64, PF_VLD = PF_BN + 4;
 
 template <int DPAD>
 __global__ void __launch_bounds__(256)
 attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
-                    const bf16* __restrict__ v_new, const bf16* __restrict__ pages,
-                    const int* __restrict__ table, int table_stride, int ring_pages,
-                    const int* __restrict__ row_pos, const int* __restrict__ cu_seqlens,
+                    const bf16* __restrict__ vt_new, int vt_cols, const int* __restrict__ tile_off,
+                    const bf16* __restrict__ pages, const int* __restrict__ table, int table_stride,
+                    int ring_pages, const int* __restrict__ row_pos, const int* __restrict__ cu_seqlens,
                     const int* __restrict__ n_cached, int B, int nq, int nkv, int d, int window,
                     float scale, bf16* __restrict__ out) {
   constexpr int KB = DPAD / 16, VB = DPAD / 32, KLD = DPAD + 8, CH = DPAD / 8;
+  constexpr int PT = DPAD / 32;        // 16-byte chunks of keys, and of values, per thread and tile
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   bf16* Ks = reinterpret_cast<bf16*>(smem);          // [PF_BN][KLD]
   bf16* Vt = Ks + PF_BN * KLD;                       // [DPAD][PF_VLD]
 
-  // which sequence and which block of its rows
-  int t = blockIdx.x, b = 0;
+  // which sequence and which block of its rows; late blocks (most keys) first
+  int t = gridDim.x - 1 - blockIdx.x, b = 0;
   for (; b < B; ++b) {
     const int tiles = (cu_seqlens[b + 1] - cu_seqlens[b] + PF_BM - 1) / PF_BM;
     if (t < tiles) break;
@@ -61,6 +66,8 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
   const bool q_ok = qr < n_new;
   const int p_me = p_first + qr;
   const size_t head_elems = (size_t)PAGE * d, page_elems = 2 * (size_t)nkv * head_elems;
+  const int j_base = (cached / PAGE) * PAGE;
+  const bf16* vt_head = vt_new + (size_t)kvh * d * vt_cols + tile_off[b];
 
   bf16x8 qreg[KB];
   {
@@ -82,55 +89,70 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
   const int pw_lo = p_lo + wave * 32, pw_hi = min(p_hi, pw_lo + 31);    // this wave's positions
   const int j_lo = (window > 0 && p_lo - window + 1 > 0) ? p_lo - window + 1 : 0;
 
-  for (int jt = j_lo / PF_BN; jt * PF_BN <= p_hi; ++jt) {
-    const int j0 = jt * PF_BN;
-    __syncthreads();
-    if (j0 + PF_BN <= cached) {
-      // the tile is one cached page: keys row by row, values already transposed
+  bf16x8 kfetch[PT], vfetch[PT];
+  // tile j0 -> registers: keys as rows [key][d], values as rows [dv][key]
+  auto fetch = [&](int j0) {
+    const bool has_cached = j0 < cached, has_new = j0 + PF_BN > cached;
+    const bf16* kpage = nullptr;
+    if (has_cached) {
       const int page = table[(size_t)b * table_stride + (j0 / PAGE) % ring_pages];
-      const bf16* kbase = pages + (size_t)page * page_elems + (size_t)kvh * head_elems;
-      const bf16* vbase = kbase + (size_t)nkv * head_elems;
-      for (int c = tid; c < PF_BN * CH; c += 256) {
-        const int row = c / CH, col = (c % CH) * 8;
-        *reinterpret_cast<bf16x8*>(&Ks[row * KLD + col]) = (col < d) ? ld8(kbase + (size_t)row * d + col) : z8();
-      }
-      for (int c = tid; c < DPAD * (PF_BN / 8); c += 256) {
-        const int dv = c / (PF_BN / 8), kc = (c % (PF_BN / 8)) * 8;
-        const bf16x8 vv = (dv < d) ? ld8(vbase + (size_t)dv * PAGE + kc) : z8();
-        bf16x4 lo4, hi4;
+      kpage = pages + (size_t)page * page_elems + (size_t)kvh * head_elems;
+    }
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          lo4[e] = vv[e];
-          hi4[e] = vv[4 + e];
+    for (int i = 0; i < PT; ++i) {
+      const int c = tid + 256 * i;
+      {   // keys: chunk c = (row, 8 columns)
+        const int row = c / CH, col = (c % CH) * 8, j = j0 + row;
+        bf16x8 kv = z8();
+        if (col < d && j <= p_hi) {
+          if (j < cached) kv = ld8(kpage + (size_t)row * d + col);
+          else kv = ld8(k_new + ((size_t)(row0 + j - cached) * nkv + kvh) * d + col);
         }
-        *reinterpret_cast<bf16x4*>(&Vt[dv * PF_VLD + kc]) = lo4;
-        *reinterpret_cast<bf16x4*>(&Vt[dv * PF_VLD + kc + 4]) = hi4;
+        kfetch[i] = kv;
       }
-    } else {
-      for (int c = tid; c < PF_BN * CH; c += 256) {
-        const int row = c / CH, col = (c % CH) * 8;
-        const int j = j0 + row;
-        bf16x8 kv = z8(), vv = z8();
-        if (j <= p_hi && col < d) {
-          if (j < cached) {
-            const int page = table[(size_t)b * table_stride + (j / PAGE) % ring_pages];
-            const bf16* base = pages + (size_t)page * page_elems + (size_t)kvh * head_elems;
-            kv = ld8(base + (size_t)(j % PAGE) * d + col);
-            const bf16* vp = base + (size_t)nkv * head_elems + (size_t)col * PAGE + (j % PAGE);
+      {   // values: chunk c = (dv, 8 keys)
+        const int dv = c / (PF_BN / 8), kc = (c % (PF_BN / 8)) * 8;
+        bf16x8 vv = z8();
+        if (dv < d) {
+          bf16x8 cv = z8(), nv = z8();
+          if (has_cached) cv = ld8(kpage + (size_t)nkv * head_elems + (size_t)dv * PAGE + kc);
+          if (has_new) nv = ld8(vt_head + (size_t)dv * vt_cols + (j0 - j_base) + kc);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) vv[e] = vp[(size_t)e * PAGE];
-          } else {
-            const size_t r = ((size_t)(row0 + j - cached) * nkv + kvh) * d + col;
-            kv = ld8(k_new + r);
-            vv = ld8(v_new + r);
+          for (int e = 0; e < 8; ++e) {
+            const int j = j0 + kc + e;
+            vv[e] = (j < cached) ? cv[e] : ((j <= p_hi) ? nv[e] : (bf16)0.f);
           }
         }
-        *reinterpret_cast<bf16x8*>(&Ks[row * KLD + col]) = kv;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) Vt[(col + e) * PF_VLD + row] = vv[e];
+        vfetch[i] = vv;
       }
     }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int i = 0; i < PT; ++i) {
+      const int c = tid + 256 * i;
+      const int row = c / CH, col = (c % CH) * 8;
+      *reinterpret_cast<bf16x8*>(&Ks[row * KLD + col]) = kfetch[i];
+      const int dv = c / (PF_BN / 8), kc = (c % (PF_BN / 8)) * 8;
+      bf16x4 lo4, hi4;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        lo4[e] = vfetch[i][e];
+        hi4[e] = vfetch[i][4 + e];
+      }
+      *reinterpret_cast<bf16x4*>(&Vt[dv * PF_VLD + kc]) = lo4;
+      *reinterpret_cast<bf16x4*>(&Vt[dv * PF_VLD + kc + 4]) = hi4;
+    }
+  };
+
+  const int jt_first = j_lo / PF_BN;
+  fetch(jt_first * PF_BN);
+  for (int jt = jt_first; jt * PF_BN <= p_hi; ++jt) {
+    const int j0 = jt * PF_BN;
+    __syncthreads();                  // the previous tile has been worked on
+    stash();
     __syncthreads();
+    if ((jt + 1) * PF_BN <= p_hi) fetch((jt + 1) * PF_BN);
     // does any query of this wave see any key of this tile?
     if (pw_lo > p_hi || j0 > pw_hi || (window > 0 && j0 + PF_BN - 1 <= pw_lo - window)) continue;
 
@@ -258,27 +280,40 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
   for (int vb = 0; vb < VB; ++vb) o[vb] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
 
-  for (int pg = my_lo + wave; pg < my_hi; pg += DC_WAVES) {
+  // the split's groups of 32 keys go round the waves
+  for (int gi = 2 * my_lo + wave; gi < 2 * my_hi; gi += DC_WAVES) {
+    const int pg = gi / 2, grp = gi % 2;
     const int page = table[(size_t)b * table_stride + pg % ring_pages];
     const bf16* kbase = pages + (size_t)page * page_elems + (size_t)kvh * head_elems;
     const bf16* vbase = kbase + (size_t)nkv * head_elems;
-#pragma unroll
-    for (int grp = 0; grp < 2; ++grp) {               // 32 keys at a time
+    {
       const int j0 = pg * PAGE + grp * 32;
       if (j0 > p || j0 + 31 < lo) continue;
       // block bs holds keys j0 + 8 (i/4) + 4 bs + i%4 in its rows i: then a lane's 8 scores of
       // the two blocks are 8 consecutive keys, j0 + 8 kg .. + 7
-      f32x4 s[2];
+      // all loads of the group first: keys (two blocks) and values
+      bf16x8 kreg[2][KB], vreg[VB];
 #pragma unroll
       for (int bs = 0; bs < 2; ++bs) {
-        s[bs] = f32x4{0.f, 0.f, 0.f, 0.f};
         const bf16* krow = kbase + (size_t)(grp * 32 + 8 * (li / 4) + 4 * bs + (li % 4)) * d;
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb) {
           const int k = kb * 32 + 8 * kg;
-          const bf16x8 a = (k + 8 <= d) ? ld8(krow + k) : z8();
-          s[bs] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qreg[kb], s[bs], 0, 0, 0);
+          kreg[bs][kb] = (k + 8 <= d) ? ld8(krow + k) : z8();
         }
+      }
+#pragma unroll
+      for (int vb = 0; vb < VB; ++vb) {
+        const int dv = vb * 16 + li;
+        vreg[vb] = (dv < d) ? ld8(vbase + (size_t)dv * PAGE + grp * 32 + 8 * kg) : z8();
+      }
+      f32x4 s[2];
+#pragma unroll
+      for (int bs = 0; bs < 2; ++bs) {
+        s[bs] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb)
+          s[bs] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[bs][kb], qreg[kb], s[bs], 0, 0, 0);
       }
       float sv[8];
       float tmax = -INFINITY;
@@ -308,8 +343,7 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
       // O^T[dv][head] += V^T[dv][keys] P^T[keys][head]; values lie as [d][PAGE] in the page
 #pragma unroll
       for (int vb = 0; vb < VB; ++vb) {
-        const int dv = vb * 16 + li;
-        bf16x8 a = (dv < d) ? ld8(vbase + (size_t)dv * PAGE + grp * 32 + 8 * kg) : z8();
+        bf16x8 a = vreg[vb];
         if (j0 + 31 > p) {         // rows past the sequence's end were never written: 0 * garbage
 #pragma unroll
           for (int e = 0; e < 8; ++e)
@@ -368,28 +402,35 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
 
 __global__ void __launch_bounds__(64)
 attn_decode_combine_kernel(const float* __restrict__ part, int n_splits, int d, bf16* __restrict__ out) {
+  extern __shared__ float fac[];                       // [n_splits] weight of each split
   const size_t bh = blockIdx.x;
   const float* src = part + bh * n_splits * (d + 2);
+  const int lane = threadIdx.x;
   float mm = -INFINITY;
-  for (int s = 0; s < n_splits; ++s) mm = fmaxf(mm, src[(size_t)s * (d + 2)]);
+  for (int s = lane; s < n_splits; s += 64) mm = fmaxf(mm, src[(size_t)s * (d + 2)]);
+  mm = wave_max(mm);
   float ll = 0.f;
-  for (int s = 0; s < n_splits; ++s) {
+  for (int s = lane; s < n_splits; s += 64) {
     const float ms = src[(size_t)s * (d + 2)];
-    ll += (ms == -INFINITY) ? 0.f : src[(size_t)s * (d + 2) + 1] * __expf(ms - mm);
+    const float f = (ms == -INFINITY) ? 0.f : __expf(ms - mm);
+    fac[s] = f;
+    ll += src[(size_t)s * (d + 2) + 1] * f;
   }
-  for (int dv = threadIdx.x; dv < d; dv += 64) {
+  ll = wave_sum(ll);
+  __syncthreads();
+  for (int dv = lane; dv < d; dv += 64) {
     float acc = 0.f;
     for (int s = 0; s < n_splits; ++s) {
-      const float ms = src[(size_t)s * (d + 2)];
-      if (ms != -INFINITY) acc += src[(size_t)s * (d + 2) + 2 + dv] * __expf(ms - mm);
+      const float f = fac[s];
+      if (f != 0.f) acc += src[(size_t)s * (d + 2) + 2 + dv] * f;
     }
     out[bh * d + dv] = (bf16)(acc / ll);
   }
 }
 
 template <int DPAD>
-static int launch_prefill(const bf16* q, const bf16* k_new, const bf16* v_new, const bf16* pages,
-                          const int* table, int table_stride, int ring_pages, const int* row_pos,
+static int launch_prefill(const bf16* q, const bf16* k_new, const bf16* vt_new, int vt_cols,
+                          const int* tile_off, const bf16* pages, const int* table, int table_stride, int ring_pages, const int* row_pos,
                           const int* cu_seqlens, const int* n_cached, int B, int n_tiles, int nq, int nkv,
                           int d, int window, float scale, bf16* out, hipStream_t st) {
   const size_t smem = ((size_t)PF_BN * (DPAD + 8) + (size_t)DPAD * PF_VLD) * sizeof(bf16);
@@ -406,9 +447,9 @@ static int launch_prefill(const bf16* q, const bf16* k_new, const bf16* v_new, c
     }
   }
   dim3 grid(n_tiles, nq);
-  attn_prefill_kernel<DPAD><<<grid, 256, smem, st>>>(q, k_new, v_new, pages, table, table_stride,
-                                                     ring_pages, row_pos, cu_seqlens, n_cached, B, nq,
-                                                     nkv, d, window, scale, out);
+  attn_prefill_kernel<DPAD><<<grid, 256, smem, st>>>(q, k_new, vt_new, vt_cols, tile_off, pages, table,
+                                                     table_stride, ring_pages, row_pos, cu_seqlens,
+                                                     n_cached, B, nq, nkv, d, window, scale, out);
   TL_LAUNCH_CHECK("attn_prefill");
   return 0;
 }
@@ -423,7 +464,7 @@ static int launch_decode(const bf16* q, const bf16* pages, const int* table, int
                                                             row_pos, nq, nkv, d, window, scale, n_splits,
                                                             head_groups, part);
   TL_LAUNCH_CHECK("attn_decode");
-  attn_decode_combine_kernel<<<B * nq, 64, 0, st>>>(part, n_splits, d, out);
+  attn_decode_combine_kernel<<<B * nq, 64, n_splits * sizeof(float), st>>>(part, n_splits, d, out);
   TL_LAUNCH_CHECK("attn_decode_combine");
   return 0;
 }
@@ -444,8 +485,10 @@ using namespace tl;
     case 8: return fn<256>(__VA_ARGS__);                             \
   }
 
-extern "C" int tl_attn_prefill_bf16(const void* q, const void* k_new, const void* v_new,
-                                    const void* pages, const int* table, int table_stride,
+// vt_new: this step's values transposed, [nkv][d][vt_cols]; the value of sequence b at position p
+// lies in column tile_off[b] + p - 64 * (n_cached[b] / 64); tile_off and vt_cols multiples of 64
+extern "C" int tl_attn_prefill_bf16(const void* q, const void* k_new, const void* vt_new, int vt_cols,
+                                    const int* tile_off, const void* pages, const int* table, int table_stride,
                                     int ring_pages, const int* row_pos, const int* cu_seqlens,
                                     const int* n_cached, int B, int n_tiles, int nq, int nkv, int d,
                                     int window, float scale, void* out, hipStream_t st) {
@@ -456,7 +499,10 @@ extern "C" int tl_attn_prefill_bf16(const void* q, const void* k_new, const void
   TL_REQUIRE(ring_pages > 0 && table_stride > 0 && window >= 0,
              "attn_prefill: bad cache geometry ring_pages=%d table_stride=%d window=%d", ring_pages,
              table_stride, window);
-  TL_BY_DPAD(launch_prefill, (const bf16*)q, (const bf16*)k_new, (const bf16*)v_new,
+  TL_REQUIRE(vt_cols > 0 && vt_cols % 64 == 0 && ((uintptr_t)vt_new % 16 == 0),
+             "attn_prefill: the transposed values need a multiple of 64 columns (%d) and 16-byte alignment",
+             vt_cols);
+  TL_BY_DPAD(launch_prefill, (const bf16*)q, (const bf16*)k_new, (const bf16*)vt_new, vt_cols, tile_off,
              (const bf16*)pages, table, table_stride, ring_pages, row_pos, cu_seqlens, n_cached, B,
              n_tiles, nq, nkv, d, window, scale, (bf16*)out, st);
   return 1;
@@ -471,7 +517,7 @@ extern "C" int tl_attn_decode_bf16(const void* q, const void* pages, const int* 
              nq, nkv);
   TL_REQUIRE(d >= 16 && d <= 256 && d % 16 == 0, "attn_decode: head size %d is not served "
              "(multiples of 16 up to 256)", d);
-  TL_REQUIRE(ring_pages > 0 && table_stride > 0 && window >= 0 && n_splits > 0 && n_splits <= 65535,
+  TL_REQUIRE(ring_pages > 0 && table_stride > 0 && window >= 0 && n_splits > 0 && n_splits <= 4096,
              "attn_decode: bad geometry ring_pages=%d table_stride=%d window=%d splits=%d", ring_pages,
              table_stride, window, n_splits);
   TL_BY_DPAD(launch_decode, (const bf16*)q, (const bf16*)pages, table, table_stride, ring_pages, row_pos,

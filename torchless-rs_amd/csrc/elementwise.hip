@@ -46,23 +46,69 @@ __global__ void __launch_bounds__(256) rmsnorm_kernel(const float* __restrict__ 
   for (int i = threadIdx.x; i < H; i += 256) o[i] = from_f32<TO>((xr[i] / rms) * w[i]);
 }
 
+// The same with the row held in registers: one read of x.  H % 4 == 0, H <= 1024 * IT.
+template <typename TO, int IT>
+__global__ void __launch_bounds__(256) rmsnorm_reg_kernel(const float* __restrict__ x,
+                                                          const float* __restrict__ w, float eps,
+                                                          TO* __restrict__ out, int H) {
+  __shared__ float sh[4];
+  const int n = blockIdx.x;
+  const float4* xr = reinterpret_cast<const float4*>(x + (size_t)n * H);
+  const float4* wr = reinterpret_cast<const float4*>(w);
+  const int nv = H / 4;
+  float4 v[IT], g[IT];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < IT; ++i) {
+    const int c = threadIdx.x + 256 * i;
+    if (c < nv) {
+      v[i] = xr[c];
+      g[i] = wr[c];
+      ss += v[i].x * v[i].x + v[i].y * v[i].y + v[i].z * v[i].z + v[i].w * v[i].w;
+    }
+  }
+  ss = block_sum<256>(ss, sh);
+  const float rms = sqrtf(ss / (float)H + eps);
+  TO* o = out + (size_t)n * H;
+#pragma unroll
+  for (int i = 0; i < IT; ++i) {
+    const int c = threadIdx.x + 256 * i;
+    if (c < nv) {
+      o[4 * c + 0] = from_f32<TO>((v[i].x / rms) * g[i].x);
+      o[4 * c + 1] = from_f32<TO>((v[i].y / rms) * g[i].y);
+      o[4 * c + 2] = from_f32<TO>((v[i].z / rms) * g[i].z);
+      o[4 * c + 3] = from_f32<TO>((v[i].w / rms) * g[i].w);
+    }
+  }
+}
+
 // ---- rotation and split ------------------------------------------------------
 // qkv[n, :] = [q (nq*d) | k (nkv*d) | v (nkv*d)] in float.  q and k are rotated
 // in pairs (i, i + d/2) by the angle pos * inv_freq[i]; v is copied.
 // src/kernels/mod.rs:582-608, src/model/modules/attention.rs:68-78.
+constexpr int ROPE_MAX_HALF = 128;      // head sizes up to 256
+
 template <typename TO>
 __global__ void rope_split_kernel(const float* __restrict__ qkv, const int* __restrict__ row_pos,
                                   const float* __restrict__ inv_freq, int nq, int nkv, int d,
-                                  TO* __restrict__ q, TO* __restrict__ k, TO* __restrict__ v) {
+                                  TO* __restrict__ q, TO* __restrict__ k, TO* __restrict__ v,
+                                  TO* __restrict__ vt, int vt_cols, const int* __restrict__ row_seq,
+                                  const int* __restrict__ tile_off, const int* __restrict__ n_cached) {
+  __shared__ float cs[ROPE_MAX_HALF], sn[ROPE_MAX_HALF];
   const int n = blockIdx.x;
   const int half = d / 2;
   const float pos = (float)row_pos[n];
+  for (int i = threadIdx.x; i < half; i += blockDim.x) {     // the row's angles, once
+    const float ang = inv_freq[i] * pos;
+    cs[i] = cosf(ang);
+    sn[i] = sinf(ang);
+  }
+  __syncthreads();
   const float* src = qkv + (size_t)n * (nq + 2 * nkv) * d;
   const int n_rot = (nq + nkv) * half;
   for (int t = threadIdx.x; t < n_rot; t += blockDim.x) {
     const int h = t / half, i = t % half;
-    const float ang = inv_freq[i] * pos;
-    const float c = cosf(ang), s = sinf(ang);
+    const float c = cs[i], s = sn[i];
     const float a = src[h * d + i], b = src[h * d + i + half];
     const float ra = a * c - b * s, rb = a * s + b * c;
     TO* dst = (h < nq) ? q + ((size_t)n * nq + h) * d : k + ((size_t)n * nkv + (h - nq)) * d;
@@ -72,6 +118,11 @@ __global__ void rope_split_kernel(const float* __restrict__ qkv, const int* __re
   const float* vs = src + (size_t)(nq + nkv) * d;
   TO* vd = v + (size_t)n * nkv * d;
   for (int t = threadIdx.x; t < nkv * d; t += blockDim.x) vd[t] = from_f32<TO>(vs[t]);
+  if (vt != nullptr) {      // the same values transposed: [kv head][d][column of this row]
+    const int b = row_seq[n];
+    const int col = tile_off[b] + row_pos[n] - (n_cached[b] / PAGE) * PAGE;
+    for (int t = threadIdx.x; t < nkv * d; t += blockDim.x) vt[(size_t)t * vt_cols + col] = from_f32<TO>(vs[t]);
+  }
 }
 
 // ---- commit keys and values of this step to the pages -----------------------
@@ -101,6 +152,43 @@ __global__ void kv_commit_kernel(const T* __restrict__ k, const T* __restrict__ 
     kd[((size_t)h * PAGE + r) * d + i] = ks[t];
     vd[((size_t)h * d + i) * PAGE + r] = vs[t];
   }
+}
+
+// ---- single-token steps: rotate, and put k and v straight into the pages ------
+// Row n is the one new token of sequence n (position row_pos[n]).
+template <typename T>
+__global__ void rope_commit_kernel(const float* __restrict__ qkv, const int* __restrict__ row_pos,
+                                   const float* __restrict__ inv_freq, const int* __restrict__ table,
+                                   int table_stride, int ring_pages, int nq, int nkv, int d,
+                                   T* __restrict__ q, T* __restrict__ pages) {
+  const int n = blockIdx.x;
+  const int half = d / 2;
+  const int p = row_pos[n];
+  const float pos = (float)p;
+  const float* src = qkv + (size_t)n * (nq + 2 * nkv) * d;
+  const int page = table[(size_t)n * table_stride + (p / PAGE) % ring_pages];
+  const int r = p % PAGE;
+  T* kd = pages + (size_t)page * 2 * nkv * PAGE * d;
+  T* vd = kd + (size_t)nkv * PAGE * d;
+  __shared__ float cs[ROPE_MAX_HALF], sn[ROPE_MAX_HALF];
+  for (int i = threadIdx.x; i < half; i += blockDim.x) {
+    const float ang = inv_freq[i] * pos;
+    cs[i] = cosf(ang);
+    sn[i] = sinf(ang);
+  }
+  __syncthreads();
+  const int n_rot = (nq + nkv) * half;
+  for (int t = threadIdx.x; t < n_rot; t += blockDim.x) {
+    const int h = t / half, i = t % half;
+    const float c = cs[i], s = sn[i];
+    const float a = src[h * d + i], b = src[h * d + i + half];
+    const float ra = a * c - b * s, rb = a * s + b * c;
+    T* dst = (h < nq) ? q + ((size_t)n * nq + h) * d : kd + ((size_t)(h - nq) * PAGE + r) * d;
+    dst[i] = from_f32<T>(ra);
+    dst[i + half] = from_f32<T>(rb);
+  }
+  const float* vs = src + (size_t)(nq + nkv) * d;
+  for (int t = threadIdx.x; t < nkv * d; t += blockDim.x) vd[(size_t)t * PAGE + r] = from_f32<T>(vs[t]);
 }
 
 // ---- h = silu(gate) * up, silu(g) = g / (1 + exp(-g)) ------------------------
@@ -150,27 +238,43 @@ int tl_rmsnorm(const float* x, const float* w, float eps, void* out, int out_dt,
                hipStream_t st) {
   TL_REQUIRE(n >= 0 && H > 0, "rmsnorm: bad sizes n=%d H=%d", n, H);
   if (n == 0) return 0;
-  if (out_dt == DT_F32)
+  TL_REQUIRE(out_dt == DT_F32 || out_dt == DT_BF16, "rmsnorm: unknown dtype code %d", out_dt);
+  const bool vec = H % 4 == 0 && H <= 8192 && ((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0);
+#define TL_RMS(IT)                                                                        \
+  do {                                                                                    \
+    if (out_dt == DT_F32) rmsnorm_reg_kernel<float, IT><<<n, 256, 0, st>>>(x, w, eps, (float*)out, H); \
+    else rmsnorm_reg_kernel<bf16, IT><<<n, 256, 0, st>>>(x, w, eps, (bf16*)out, H);        \
+  } while (0)
+  if (vec && H <= 1024) TL_RMS(1);
+  else if (vec && H <= 2048) TL_RMS(2);
+  else if (vec && H <= 4096) TL_RMS(4);
+  else if (vec) TL_RMS(8);
+  else if (out_dt == DT_F32)
     rmsnorm_kernel<float><<<n, 256, 0, st>>>(x, w, eps, (float*)out, H);
-  else if (out_dt == DT_BF16)
-    rmsnorm_kernel<bf16><<<n, 256, 0, st>>>(x, w, eps, (bf16*)out, H);
   else
-    TL_REQUIRE(false, "rmsnorm: unknown dtype code %d", out_dt);
+    rmsnorm_kernel<bf16><<<n, 256, 0, st>>>(x, w, eps, (bf16*)out, H);
+#undef TL_RMS
   TL_LAUNCH_CHECK("rmsnorm");
   return 0;
 }
 
+// vt (may be null): values also transposed, [nkv][d][vt_cols], row n in column
+// tile_off[row_seq[n]] + row_pos[n] - 64 * (n_cached[row_seq[n]] / 64)
 int tl_rope_split(const float* qkv, const int* row_pos, const float* inv_freq, int n, int nq,
-                  int nkv, int d, void* q, void* k, void* v, int out_dt, hipStream_t st) {
+                  int nkv, int d, void* q, void* k, void* v, void* vt, int vt_cols, const int* row_seq,
+                  const int* tile_off, const int* n_cached, int out_dt, hipStream_t st) {
   TL_REQUIRE(n >= 0 && nq > 0 && nkv >= 0 && d > 0 && d % 2 == 0,
              "rope_split: bad sizes n=%d nq=%d nkv=%d d=%d (d must be even)", n, nq, nkv, d);
+  TL_REQUIRE(d <= 2 * ROPE_MAX_HALF, "rope_split: head size %d is not served (at most %d)", d, 2 * ROPE_MAX_HALF);
   if (n == 0) return 0;
   if (out_dt == DT_F32)
     rope_split_kernel<float><<<n, 256, 0, st>>>(qkv, row_pos, inv_freq, nq, nkv, d, (float*)q,
-                                                 (float*)k, (float*)v);
+                                                 (float*)k, (float*)v, (float*)vt, vt_cols, row_seq,
+                                                 tile_off, n_cached);
   else if (out_dt == DT_BF16)
     rope_split_kernel<bf16><<<n, 256, 0, st>>>(qkv, row_pos, inv_freq, nq, nkv, d, (bf16*)q,
-                                                (bf16*)k, (bf16*)v);
+                                                (bf16*)k, (bf16*)v, (bf16*)vt, vt_cols, row_seq, tile_off,
+                                                n_cached);
   else
     TL_REQUIRE(false, "rope_split: unknown dtype code %d", out_dt);
   TL_LAUNCH_CHECK("rope_split");
@@ -196,6 +300,26 @@ int tl_kv_commit(const void* k, const void* v, int dt, const int* row_seq, const
   else
     TL_REQUIRE(false, "kv_commit: unknown dtype code %d", dt);
   TL_LAUNCH_CHECK("kv_commit");
+  return 0;
+}
+
+int tl_rope_commit(const float* qkv, const int* row_pos, const float* inv_freq, const int* table,
+                   int table_stride, int ring_pages, int n, int nq, int nkv, int d, void* q, void* pages,
+                   int dt, hipStream_t st) {
+  TL_REQUIRE(n >= 0 && nq > 0 && nkv > 0 && d > 0 && d % 2 == 0 && ring_pages > 0 && table_stride > 0,
+             "rope_commit: bad sizes n=%d nq=%d nkv=%d d=%d ring_pages=%d table_stride=%d", n, nq, nkv, d,
+             ring_pages, table_stride);
+  TL_REQUIRE(d <= 2 * ROPE_MAX_HALF, "rope_commit: head size %d is not served (at most %d)", d, 2 * ROPE_MAX_HALF);
+  if (n == 0) return 0;
+  if (dt == DT_F32)
+    rope_commit_kernel<float><<<n, 256, 0, st>>>(qkv, row_pos, inv_freq, table, table_stride, ring_pages,
+                                                  nq, nkv, d, (float*)q, (float*)pages);
+  else if (dt == DT_BF16)
+    rope_commit_kernel<bf16><<<n, 256, 0, st>>>(qkv, row_pos, inv_freq, table, table_stride, ring_pages, nq,
+                                                 nkv, d, (bf16*)q, (bf16*)pages);
+  else
+    TL_REQUIRE(false, "rope_commit: unknown dtype code %d", dt);
+  TL_LAUNCH_CHECK("rope_commit");
   return 0;
 }
 

@@ -24,13 +24,17 @@ __device__ __forceinline__ bf16x8 zero8() {
   return z;
 }
 
-// ---------------------------------------------------------------- skinny ----
-constexpr int SK_WAVES = 8;
+// what happens to the product
+constexpr int EPI_STORE = 0;        // C = product (float)
+constexpr int EPI_ACCUMULATE = 1;   // C += product (float; the residual stream)
+constexpr int EPI_SILU_PAIR = 2;    // W's rows come in groups of 64 (32 gate rows, their 32 up rows):
+                                    // C is bfloat16 [M, N/2] = silu(gate) * up
 
-template <int NT, int MT>
+// ---------------------------------------------------------------- skinny ----
+template <int NT, int MT, int SK_WAVES>
 __global__ void __launch_bounds__(SK_WAVES * 64)
 gemm_skinny_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float* __restrict__ C, int M,
-                   int N, int K, int accumulate) {
+                   int N, int K, int epilogue) {
   __shared__ float red[SK_WAVES][NT * MT * 256];
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const int li = lane % 16, kg = lane / 16;
@@ -98,26 +102,47 @@ gemm_skinny_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float
       for (int r = 0; r < 4; ++r) red[wave][((t * MT + u) * 4 + r) * 64 + lane] = acc[t][u][r];
   __syncthreads();
   constexpr int NB = 16 * NT;
-  for (int e = threadIdx.x; e < NB * 16 * MT; e += SK_WAVES * 64) {
-    const int nl = e % NB, m = e / NB;
+  auto total = [&](int nl, int m) {
     const int t = nl / 16, u = m / 16;
     const int idx = ((t * MT + u) * 4 + (nl % 4)) * 64 + ((nl % 16) / 4) * 16 + (m % 16);
     float v = 0.f;
 #pragma unroll
     for (int w = 0; w < SK_WAVES; ++w) v += red[w][idx];
+    return v;
+  };
+  if (epilogue == EPI_SILU_PAIR) {
+    // rows come in groups of 64: 32 gate rows, then the 32 up rows that belong to them
+    if constexpr (NB % 64 == 0) {
+      bf16* H = reinterpret_cast<bf16*>(C);
+      const int NH = N / 2;
+      for (int e = threadIdx.x; e < (NB / 2) * 16 * MT; e += SK_WAVES * 64) {
+        const int jl = e % (NB / 2), m = e / (NB / 2);
+        const int grp = jl / 32, j = jl % 32;
+        const int n = (n0 / 2) + jl;
+        if (n < NH && m < M) {
+          const float g = total(grp * 64 + j, m), u = total(grp * 64 + 32 + j, m);
+          H[(size_t)m * NH + n] = (bf16)((g / (1.0f + expf(-g))) * u);
+        }
+      }
+    }
+    return;
+  }
+  for (int e = threadIdx.x; e < NB * 16 * MT; e += SK_WAVES * 64) {
+    const int nl = e % NB, m = e / NB;
+    const float v = total(nl, m);
     const int n = n0 + nl;
     if (n < N && m < M) {
       float* c = C + (size_t)m * N + n;
-      *c = accumulate ? *c + v : v;
+      *c = (epilogue == EPI_ACCUMULATE) ? *c + v : v;
     }
   }
 }
 
-template <int NT, int MT>
-static int launch_skinny(const bf16* A, const bf16* W, float* C, int M, int N, int K, int accumulate,
+template <int NT, int MT, int SK_WAVES = 8>
+static int launch_skinny(const bf16* A, const bf16* W, float* C, int M, int N, int K, int epilogue,
                          hipStream_t st) {
   const int grid = (N + 16 * NT - 1) / (16 * NT);
-  gemm_skinny_kernel<NT, MT><<<grid, SK_WAVES * 64, 0, st>>>(A, W, C, M, N, K, accumulate);
+  gemm_skinny_kernel<NT, MT, SK_WAVES><<<grid, SK_WAVES * 64, 0, st>>>(A, W, C, M, N, K, epilogue);
   TL_LAUNCH_CHECK("gemm_skinny");
   return 0;
 }
@@ -127,7 +152,7 @@ constexpr int TM = 128, TN = 128, TK = 64, TPAD = 8, TLD = TK + TPAD;
 
 __global__ void __launch_bounds__(256)
 gemm_tiled_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float* __restrict__ C, int M,
-                  int N, int K, int accumulate) {
+                  int N, int K, int epilogue) {
   __shared__ __attribute__((aligned(16))) bf16 As[TM * TLD];
   __shared__ __attribute__((aligned(16))) bf16 Ws[TN * TLD];
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
@@ -191,6 +216,25 @@ gemm_tiled_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float*
     }
   }
   // acc[i][j][r]: row = 8*(r/4) + 4*kh + r%4, column = l32 of the 32x32 block
+  if (epilogue == EPI_SILU_PAIR) {
+    // the wave's 64 columns are one group: block j=0 gate, block j=1 up
+    bf16* H = reinterpret_cast<bf16*>(C);
+    const int NH = N / 2;
+    const int n = (n0 + wn) / 2 + l32;
+    if (n < NH) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int m = m0 + wm + 32 * i + 8 * (r / 4) + 4 * kh + (r % 4);
+          if (m < M) {
+            const float g = acc[i][0][r], u = acc[i][1][r];
+            H[(size_t)m * NH + n] = (bf16)((g / (1.0f + expf(-g))) * u);
+          }
+        }
+    }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -202,50 +246,216 @@ gemm_tiled_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float*
         const int m = m0 + wm + 32 * i + 8 * (r / 4) + 4 * kh + (r % 4);
         if (m < M) {
           float* c = C + (size_t)m * N + n;
-          *c = accumulate ? *c + acc[i][j][r] : acc[i][j][r];
+          *c = (epilogue == EPI_ACCUMULATE) ? *c + acc[i][j][r] : acc[i][j][r];
         }
       }
     }
+}
+
+// ------------------------------------------------------------------- big ----
+// 256x128x64 tiles staged through LDS (two workgroups a CU), 4 waves of 128x64.
+// Workgroups are numbered so that those that follow each other on one XCD
+// (every 8th id) take neighbouring row blocks of the same weight tile.
+constexpr int GM = 256, GN = 128, GK = 64, GLD = GK + 8;
+constexpr int G_BUF = (GM + GN) * GLD;                 // elements of one buffer
+
+__global__ void __launch_bounds__(256, 2)
+gemm_big_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float* __restrict__ C, int M,
+                int N, int K, int epilogue, int tiles_m, int tiles_n) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char g_smem[];
+  bf16* smem = reinterpret_cast<bf16*>(g_smem);
+  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+  const int l32 = lane % 32, kh = lane / 32;
+  const int wm = (wave / 2) * 128, wn = (wave % 2) * 64;
+  // id -> tile: ids 8 apart run on one XCD; give them consecutive tiles, rows fastest
+  const int total = tiles_m * tiles_n;
+  const int bid = blockIdx.x;
+  const int per_xcd = (total + 7) / 8;
+  const int logical = (bid % 8) * per_xcd + bid / 8;
+  if (logical >= total) return;
+  const int m0 = (logical % tiles_m) * GM, n0 = (logical / tiles_m) * GN;
+
+  const int lc = (tid % 8) * 8, lr = tid / 8;
+  const bf16* ap[8];
+  const bf16* wp[4];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) ap[i] = A + (size_t)min(m0 + lr + 32 * i, M - 1) * K + lc;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) wp[i] = W + (size_t)min(n0 + lr + 32 * i, N - 1) * K + lc;
+  bf16x8 ra[8], rw[4];
+  auto fetch = [&](int k0) {
+    const bool ok = k0 + lc + 8 <= K;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) ra[i] = ok ? load8(ap[i] + k0) : zero8();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) rw[i] = ok ? load8(wp[i] + k0) : zero8();
+  };
+  auto stash = [&](int buf) {
+    bf16* As = smem + buf * G_BUF;
+    bf16* Ws = As + GM * GLD;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) *reinterpret_cast<bf16x8*>(&As[(lr + 32 * i) * GLD + lc]) = ra[i];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) *reinterpret_cast<bf16x8*>(&Ws[(lr + 32 * i) * GLD + lc]) = rw[i];
+  };
+
+  f32x16 acc[4][2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  const int nk = (K + GK - 1) / GK;
+  const bf16* As = smem;
+  const bf16* Ws = As + GM * GLD;
+  fetch(0);
+  for (int kt = 0; kt < nk; ++kt) {
+    __syncthreads();                 // everyone is done reading the previous tile
+    stash(0);
+    __syncthreads();
+    if (kt + 1 < nk) fetch((kt + 1) * GK);
+#pragma unroll
+    for (int kk = 0; kk < GK; kk += 16) {
+      bf16x8 a[4], b[2];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        a[i] = *reinterpret_cast<const bf16x8*>(&As[(wm + 32 * i + l32) * GLD + kk + 8 * kh]);
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        b[j] = *reinterpret_cast<const bf16x8*>(&Ws[(wn + 32 * j + l32) * GLD + kk + 8 * kh]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+  }
+  if (epilogue == EPI_SILU_PAIR) {
+    bf16* H = reinterpret_cast<bf16*>(C);
+    const int NH = N / 2;
+    const int n = (n0 + wn) / 2 + l32;
+    if (n < NH) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int m = m0 + wm + 32 * i + 8 * (r / 4) + 4 * kh + (r % 4);
+          if (m < M) {
+            const float g = acc[i][0][r], u = acc[i][1][r];
+            H[(size_t)m * NH + n] = (bf16)((g / (1.0f + expf(-g))) * u);
+          }
+        }
+    }
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int n = n0 + wn + 32 * j + l32;
+      if (n >= N) continue;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm + 32 * i + 8 * (r / 4) + 4 * kh + (r % 4);
+        if (m < M) {
+          float* c = C + (size_t)m * N + n;
+          *c = (epilogue == EPI_ACCUMULATE) ? *c + acc[i][j][r] : acc[i][j][r];
+        }
+      }
+    }
+}
+
+static int launch_big(const bf16* A, const bf16* W, float* C, int M, int N, int K, int epilogue,
+                      hipStream_t st) {
+  constexpr int smem = G_BUF * (int)sizeof(bf16);
+  static bool raised = false;
+  if (!raised) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_big_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) {
+      set_error("gemm_big: cannot have %d bytes of LDS: %s", smem, hipGetErrorString(e));
+      return 2;
+    }
+    raised = true;
+  }
+  const int tiles_m = (M + GM - 1) / GM, tiles_n = (N + GN - 1) / GN;
+  const int grid = ((tiles_m * tiles_n + 7) / 8) * 8;
+  gemm_big_kernel<<<grid, 256, smem, st>>>(A, W, C, M, N, K, epilogue, tiles_m, tiles_n);
+  TL_LAUNCH_CHECK("gemm_big");
+  return 0;
 }
 
 }  // namespace tl
 
 using namespace tl;
 
-extern "C" int tl_gemm_bf16(const void* A, const void* W, float* C, int M, int N, int K, int accumulate,
+// epilogue: 0 store float, 1 accumulate into float, 2 silu(gate) * up into bfloat16 [M, N/2]
+// (W's rows in groups of 64: 32 gate rows and their 32 up rows; N a multiple of 64)
+extern "C" int tl_gemm_bf16(const void* A, const void* W, void* C, int M, int N, int K, int epilogue,
                             hipStream_t st) {
   TL_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_bf16: bad sizes M=%d N=%d K=%d", M, N, K);
   TL_REQUIRE(K % 8 == 0, "gemm_bf16: K=%d must be a multiple of 8", K);
   TL_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "gemm_bf16: operands must be 16-byte aligned");
+  TL_REQUIRE(epilogue >= 0 && epilogue <= 2, "gemm_bf16: unknown epilogue %d", epilogue);
+  TL_REQUIRE(epilogue != EPI_SILU_PAIR || N % 64 == 0, "gemm_bf16: the paired epilogue needs N=%d to be "
+             "a multiple of 64", N);
   if (M == 0) return 0;
   const bf16* a = (const bf16*)A;
   const bf16* w = (const bf16*)W;
-  if (M <= 16) return launch_skinny<1, 1>(a, w, C, M, N, K, accumulate, st);
-  if (M <= 32) return launch_skinny<2, 2>(a, w, C, M, N, K, accumulate, st);
-  if (M <= 64) return launch_skinny<2, 4>(a, w, C, M, N, K, accumulate, st);
-  TL_REQUIRE((M + TM - 1) / TM <= 65535, "gemm_bf16: M=%d has more row tiles than a grid holds", M);
+  float* c = (float*)C;
+  const bool wide = N >= 16384 || epilogue == EPI_SILU_PAIR;     // many rows: 64 a workgroup
+  if (M <= 16) {
+    if (wide && (M > 4 || epilogue == EPI_SILU_PAIR)) return launch_skinny<4, 1, 4>(a, w, c, M, N, K, epilogue, st);
+    return launch_skinny<1, 1, 8>(a, w, c, M, N, K, epilogue, st);
+  }
+  if (M <= 32) {
+    if (wide) return launch_skinny<4, 2, 4>(a, w, c, M, N, K, epilogue, st);
+    return launch_skinny<2, 2, 8>(a, w, c, M, N, K, epilogue, st);
+  }
+  if (M <= 64) {
+    if (wide) return launch_skinny<4, 4, 4>(a, w, c, M, N, K, epilogue, st);
+    return launch_skinny<1, 4, 8>(a, w, c, M, N, K, epilogue, st);
+  }
+  if (M > 128 && (long long)((M + GM - 1) / GM) * ((N + GN - 1) / GN) >= 512)
+    return launch_big(a, w, c, M, N, K, epilogue, st);      // enough tiles to fill the chip twice
   dim3 grid((N + TN - 1) / TN, (M + TM - 1) / TM);
-  gemm_tiled_kernel<<<grid, 256, 0, st>>>(a, w, C, M, N, K, accumulate);
+  gemm_tiled_kernel<<<grid, 256, 0, st>>>(a, w, c, M, N, K, epilogue);
   TL_LAUNCH_CHECK("gemm_tiled");
   return 0;
 }
 
-// For tests: force one of the two kernels whatever M is (M <= 64 for skinny).
-extern "C" int tl_gemm_bf16_variant(const void* A, const void* W, float* C, int M, int N, int K,
-                                    int accumulate, int variant, hipStream_t st) {
+// For tests and tuning: force one kernel whatever M is.  variant 0: tiled; 1: big; else NT*100 + MT*10 + waves/4.
+extern "C" int tl_gemm_bf16_variant(const void* A, const void* W, void* C, int M, int N, int K,
+                                    int epilogue, int variant, hipStream_t st) {
   TL_REQUIRE(M > 0 && N > 0 && K > 0 && K % 8 == 0, "gemm_bf16: bad sizes M=%d N=%d K=%d", M, N, K);
+  TL_REQUIRE(epilogue != EPI_SILU_PAIR || N % 64 == 0, "gemm_bf16: the paired epilogue needs N=%d to be "
+             "a multiple of 64", N);
   const bf16* a = (const bf16*)A;
   const bf16* w = (const bf16*)W;
+  float* c = (float*)C;
   if (variant == 0) {
     dim3 grid((N + TN - 1) / TN, (M + TM - 1) / TM);
-    gemm_tiled_kernel<<<grid, 256, 0, st>>>(a, w, C, M, N, K, accumulate);
+    gemm_tiled_kernel<<<grid, 256, 0, st>>>(a, w, c, M, N, K, epilogue);
     TL_LAUNCH_CHECK("gemm_tiled");
     return 0;
   }
-  TL_REQUIRE(M <= 64, "gemm_skinny: M=%d is more than 64", M);
-  if (variant == 1 && M <= 16) return launch_skinny<1, 1>(a, w, C, M, N, K, accumulate, st);
-  if (variant == 2 && M <= 32) return launch_skinny<2, 2>(a, w, C, M, N, K, accumulate, st);
-  if (variant == 3) return launch_skinny<2, 4>(a, w, C, M, N, K, accumulate, st);
-  if (variant == 4 && M <= 16) return launch_skinny<4, 1>(a, w, C, M, N, K, accumulate, st);
-  TL_REQUIRE(false, "gemm_bf16: variant %d does not take M=%d", variant, M);
+  if (variant == 1) return launch_big(a, w, c, M, N, K, epilogue, st);
+  const int mt = (variant / 10) % 10;
+  TL_REQUIRE(M <= 16 * mt, "gemm_skinny: variant %d takes at most %d rows, not %d", variant, 16 * mt, M);
+  TL_REQUIRE(epilogue != EPI_SILU_PAIR || variant / 100 == 4, "gemm_skinny: the paired epilogue needs 64 rows "
+             "a workgroup (variant 4xx)");
+  switch (variant) {
+    case 112: return launch_skinny<1, 1, 8>(a, w, c, M, N, K, epilogue, st);
+    case 111: return launch_skinny<1, 1, 4>(a, w, c, M, N, K, epilogue, st);
+    case 212: return launch_skinny<2, 1, 8>(a, w, c, M, N, K, epilogue, st);
+    case 411: return launch_skinny<4, 1, 4>(a, w, c, M, N, K, epilogue, st);
+    case 222: return launch_skinny<2, 2, 8>(a, w, c, M, N, K, epilogue, st);
+    case 421: return launch_skinny<4, 2, 4>(a, w, c, M, N, K, epilogue, st);
+    case 242: return launch_skinny<2, 4, 8>(a, w, c, M, N, K, epilogue, st);
+    case 441: return launch_skinny<4, 4, 4>(a, w, c, M, N, K, epilogue, st);
+    case 142: return launch_skinny<1, 4, 8>(a, w, c, M, N, K, epilogue, st);
+  }
+  TL_REQUIRE(false, "gemm_bf16: unknown variant %d", variant);
 }

@@ -80,12 +80,38 @@ def model_from_tensors(config: ModelConfig, tensors: Dict[str, torch.Tensor], dt
     return model
 
 
-def build_context(cache: Cache, batch: Sequence[SeqInput], vocab_size: int, dtype: torch.dtype, device,
-                  workspace: Workspace) -> Tuple[StepContext, Optional[torch.Tensor], int]:
-    """Check a step's entries, get their pages, and lay the batch out on the
-    device: tokens, row positions, row-to-sequence map, prefix sums, lengths and
-    page tables in one upload.  Returns the context, the wanted rows (device,
-    int32) and their number."""
+@dataclass
+class PackedStep:
+    """A step's batch on the host: one int32 array and where its pieces lie."""
+    flat: np.ndarray
+    sizes: List[int]                 # lengths of the pieces, in the order of `context_from`
+    n_rows: int
+    n_seqs: int
+    n_want: int
+    strides: Tuple[int, ...]         # page-table width of each cache group
+    all_single: bool
+    max_new: int
+    max_len_after: int
+    host: Dict[str, object]
+
+    @property
+    def key(self):
+        return (self.n_seqs, self.n_rows, self.n_want, self.strides)
+
+
+def _table_width(n_pages: int, ring_pages: int) -> int:
+    """Width of a step's page table: the next power of two, so that it (and
+    what is derived from it) changes rarely while sequences grow."""
+    w = 1
+    while w < n_pages:
+        w *= 2
+    return max(1, min(w, ring_pages))
+
+
+def pack_step(cache: Cache, batch: Sequence[SeqInput], vocab_size: int) -> PackedStep:
+    """Check a step's entries, get their pages, and lay the batch out: tokens,
+    row positions, row-to-sequence map, prefix sums, slots, lengths, wanted
+    rows and page tables in one array."""
     if not batch:
         raise StepError("a step needs at least one sequence")
     B = len(batch)
@@ -115,45 +141,76 @@ def build_context(cache: Cache, batch: Sequence[SeqInput], vocab_size: int, dtyp
     want_rows = np.array([cu[b] + w for b, s in enumerate(batch) for w in s.want], dtype=np.int64)
     tables = []
     for g in cache.groups:
-        stride = max(1, max(len(g.pages_of_slot[s.slot]) for s in batch))
+        stride = _table_width(max(len(g.pages_of_slot[s.slot]) for s in batch), g.ring_pages)
         t = np.zeros((B, stride), dtype=np.int64)
         for b, s in enumerate(batch):
             pg = g.pages_of_slot[s.slot]
             t[b, :len(pg)] = pg
         tables.append(t)
-    # one upload for all of it
+    from ..kernels.ops import aligned_columns
+    tile_off, aligned_cols = aligned_columns(len_before, n_new)
     parts = [tokens, row_pos, row_seq, cu, np.array([s.slot for s in batch]), len_before,
-             len_after, want_rows] + [t.reshape(-1) for t in tables]
-    flat = np.concatenate(parts).astype(np.int32)
-    dev = torch.from_numpy(flat).to(device, non_blocking=False)
-    views, off = [], 0
-    for p in parts:
-        views.append(dev[off:off + p.size])
-        off += p.size
-    ctx = StepContext(
-        n_rows=N, n_seqs=B, dtype=dtype, device=device,
-        tokens=views[0], row_pos=views[1], row_seq=views[2], cu_seqlens=views[3], slots=views[4],
-        len_before=views[5], len_after=views[6],
-        tables={gi: views[8 + gi].view(B, tables[gi].shape[1]) for gi in range(len(tables))},
+             len_after, want_rows, np.array(tile_off)] + [t.reshape(-1) for t in tables]
+    return PackedStep(
+        flat=np.concatenate(parts).astype(np.int32), sizes=[p.size for p in parts], n_rows=N, n_seqs=B,
+        n_want=int(want_rows.size), strides=tuple(t.shape[1] for t in tables),
         all_single=bool((n_new == 1).all()), max_new=int(n_new.max()),
-        max_len_after=int(len_after.max()), workspace=workspace, cache=cache,
+        max_len_after=int(len_after.max()),
         host={"n_new": n_new, "len_before": len_before, "len_after": len_after, "cu": cu,
-              "slots": [s.slot for s in batch]})
-    return ctx, (views[7] if want_rows.size else None), int(want_rows.size)
+              "slots": [s.slot for s in batch], "aligned_cols": aligned_cols})
 
+
+def context_from(packed: PackedStep, dev: torch.Tensor, cache: Cache, dtype: torch.dtype, device,
+                 workspace: Workspace) -> Tuple[StepContext, Optional[torch.Tensor], int]:
+    """Views of the uploaded array `dev` as the context that the parts see."""
+    views, off = [], 0
+    for n in packed.sizes:
+        views.append(dev[off:off + n])
+        off += n
+    B = packed.n_seqs
+    ctx = StepContext(
+        n_rows=packed.n_rows, n_seqs=B, dtype=dtype, device=device,
+        tokens=views[0], row_pos=views[1], row_seq=views[2], cu_seqlens=views[3], slots=views[4],
+        len_before=views[5], len_after=views[6], tile_off=views[8],
+        tables={gi: views[9 + gi].view(B, w) for gi, w in enumerate(packed.strides)},
+        all_single=packed.all_single, max_new=packed.max_new, max_len_after=packed.max_len_after,
+        workspace=workspace, cache=cache, host=dict(packed.host))
+    return ctx, (views[7] if packed.n_want else None), packed.n_want
+
+
+def build_context(cache: Cache, batch: Sequence[SeqInput], vocab_size: int, dtype: torch.dtype, device,
+                  workspace: Workspace) -> Tuple[StepContext, Optional[torch.Tensor], int]:
+    """`pack_step`, one upload, `context_from`."""
+    packed = pack_step(cache, batch, vocab_size)
+    dev = torch.from_numpy(packed.flat).to(device, non_blocking=False)
+    return context_from(packed, dev, cache, dtype, device, workspace)
+
+
+@dataclass
+class _Graph:
+    """A captured single-token step: its input array, workspace and logits."""
+    meta: torch.Tensor
+    staging: torch.Tensor
+    workspace: Workspace
+    graph: object = None
+    logits: Optional[torch.Tensor] = None
 
 
 class Engine:
     """A model, its cache and workspace.  `max_tokens` is the most positions
     that live sequences hold at any time, each rounded up to whole pages."""
 
-    def __init__(self, model: Model, max_tokens: int, max_slots: Optional[int] = None):
+    def __init__(self, model: Model, max_tokens: int, max_slots: Optional[int] = None,
+                 use_graphs: bool = True):
         self.model = model
         self.device = model.device
         self.cache: Cache = model.make_cache(max_tokens, max_slots)
         self.runs = model.bind_cache(self.cache)
         self.workspace = Workspace(self.device)
         self.vocab_size = model.spec.vocab_size
+        self.use_graphs = use_graphs
+        self.max_graphs = 32
+        self._graphs: Dict[tuple, _Graph] = {}
 
     # ---- slots -----------------------------------------------------------
     def alloc(self) -> int:
@@ -177,8 +234,48 @@ class Engine:
     def step(self, batch: Sequence[SeqInput]) -> torch.Tensor:
         """Run one step; returns float32 logits [number of wanted rows, V] in
         the order of the entries and of their `want` lists.  The tensor is a
-        view of the engine's workspace: it is overwritten by the next step."""
-        ctx, want_rows, n_want = self.build_context(batch)
-        logits = self.model.forward(ctx, self.runs, want_rows, n_want)
-        self.cache.commit([(s.slot, len(s.tokens)) for s in batch])
+        view of the engine's workspace: it is overwritten by a later step.
+
+        Steps in which every sequence brings one token are launch-bound; the
+        second time a shape of such a step (batch size, page-table widths) is
+        seen it is captured as a HIP graph, and from then on replayed."""
+        packed = pack_step(self.cache, batch, self.vocab_size)
+        growth = [(s.slot, len(s.tokens)) for s in batch]
+        if self.use_graphs and packed.all_single and self.model.graph_safe:
+            logits = self._graph_step(packed)
+        else:
+            dev = torch.from_numpy(packed.flat).to(self.device, non_blocking=False)
+            ctx, want_rows, n_want = context_from(packed, dev, self.cache, self.model.dtype,
+                                                  self.device, self.workspace)
+            logits = self.model.forward(ctx, self.runs, want_rows, n_want)
+        self.cache.commit(growth)
         return logits
+
+    def _graph_step(self, packed: PackedStep) -> torch.Tensor:
+        key = packed.key
+        g = self._graphs.get(key)
+        if g is None:
+            # first sight: run it as it is, in the workspace the graph will own, so that
+            # every buffer exists before the capture
+            if len(self._graphs) >= self.max_graphs:
+                self._graphs.pop(next(iter(self._graphs)))
+            g = _Graph(meta=torch.empty(packed.flat.size, dtype=torch.int32, device=self.device),
+                       staging=torch.empty(packed.flat.size, dtype=torch.int32).pin_memory(),
+                       workspace=Workspace(self.device))
+            self._graphs[key] = g
+        g.staging.numpy()[:] = packed.flat
+        g.meta.copy_(g.staging)
+        if g.graph is None and g.logits is not None:
+            ctx, want_rows, n_want = context_from(packed, g.meta, self.cache, self.model.dtype,
+                                                  self.device, g.workspace)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                g.logits = self.model.forward(ctx, self.runs, want_rows, n_want)
+            g.graph = graph
+        if g.graph is not None:
+            g.graph.replay()
+            return g.logits
+        ctx, want_rows, n_want = context_from(packed, g.meta, self.cache, self.model.dtype, self.device,
+                                              g.workspace)
+        g.logits = self.model.forward(ctx, self.runs, want_rows, n_want)
+        return g.logits

@@ -39,6 +39,7 @@ class Model:
                 raise ValueError(f"schedule entry {i} reads the cache of entry {run.kv_from}, which "
                                  "is not an earlier one")
         self.loaded = False
+        self.graph_safe = all(p.graph_safe for p in [self.embedding, self.final_norm, self.head] + self.blocks)
 
     # ---- weights -----------------------------------------------------------
     def load_weights(self, source) -> None:

@@ -85,9 +85,12 @@ def rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float, out: torch.Tensor) -> 
 
 
 def rope_split(qkv: torch.Tensor, row_pos: torch.Tensor, inv_freq: torch.Tensor, nq: int, nkv: int,
-               d: int, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> None:
+               d: int, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, vt: Optional[torch.Tensor] = None,
+               row_seq=None, tile_off=None, n_cached=None) -> None:
     """Rotate q and k of the fused projection by their rows' positions and
-    write q [n,nq,d], k, v [n,nkv,d]."""
+    write q [n,nq,d], k, v [n,nkv,d].  With `vt` [nkv, d, cols] the values are
+    also written transposed, row n into column tile_off[b] + pos - 64 *
+    (n_cached[b] // 64) of its sequence b = row_seq[n]."""
     n = qkv.shape[0]
     _req(qkv, "rope.qkv", torch.float32, (n, (nq + 2 * nkv) * d))
     _req(row_pos, "rope.row_pos", torch.int32, (n,))
@@ -96,8 +99,18 @@ def rope_split(qkv: torch.Tensor, row_pos: torch.Tensor, inv_freq: torch.Tensor,
     if nkv:
         _req(k, "rope.k", q.dtype, (n, nkv, d))
         _req(v, "rope.v", q.dtype, (n, nkv, d))
+    cols = 0
+    if vt is not None:
+        _req(vt, "rope.vt", q.dtype)
+        if vt.dim() != 3 or tuple(vt.shape[:2]) != (nkv, d):
+            raise KernelError(f"rope.vt: shape {tuple(vt.shape)}, kernel needs [{nkv}, {d}, columns]")
+        cols = vt.shape[2]
+        _req(row_seq, "rope.row_seq", torch.int32, (n,))
+        _req(tile_off, "rope.tile_off", torch.int32)
+        _req(n_cached, "rope.n_cached", torch.int32, tuple(tile_off.shape))
     _check(lib().tl_rope_split(_p(qkv), _p(row_pos), _p(inv_freq), n, nq, nkv, d, _p(q), _p(k), _p(v),
-                               _code(q.dtype), _stream()))
+                               _p(vt), cols, _p(row_seq), _p(tile_off), _p(n_cached), _code(q.dtype),
+                               _stream()))
 
 
 def kv_commit(k: torch.Tensor, v: torch.Tensor, row_seq, row_pos, len_after, table: torch.Tensor,
@@ -189,44 +202,95 @@ def sample(logits: torch.Tensor, temperature: float, top_k: int, top_p: float, s
                            _p(counters), _p(probs), _p(out), _stream()))
 
 
+EPI_STORE, EPI_ACCUMULATE, EPI_SILU_PAIR = 0, 1, 2
+
+
 def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False,
-              variant: Optional[int] = None) -> None:
+              variant: Optional[int] = None, silu_pair: bool = False) -> None:
     """out[M,N] (+)= a[M,K] @ w[N,K]^T on the matrix cores: bfloat16 operands,
-    float32 accumulation.  K must be a multiple of 8.  `variant` (tests only)
-    forces one kernel: 0 tiled, 1..4 the skinny ones."""
+    float32 accumulation.  K must be a multiple of 8.  With `silu_pair`, w's
+    rows come in groups of 64 (32 gate rows and the 32 up rows that belong to
+    them) and out is bfloat16 [M, N/2] = silu(gate) * up.  `variant` (tests
+    and tuning) forces one kernel."""
     M, K = a.shape
     N = w.shape[0]
     _req(a, "gemm.a", torch.bfloat16)
     _req(w, "gemm.w", torch.bfloat16, (N, K))
-    _req(out, "gemm.out", torch.float32, (M, N))
-    if variant is None:
-        _check(lib().tl_gemm_bf16(_p(a), _p(w), _p(out), M, N, K, int(accumulate), _stream()))
+    if silu_pair:
+        if accumulate or N % 64:
+            raise KernelError("gemm: the paired epilogue stores, and needs N to be a multiple of 64")
+        _req(out, "gemm.out", torch.bfloat16, (M, N // 2))
+        epi = EPI_SILU_PAIR
     else:
-        _check(lib().tl_gemm_bf16_variant(_p(a), _p(w), _p(out), M, N, K, int(accumulate), int(variant),
-                                          _stream()))
+        _req(out, "gemm.out", torch.float32, (M, N))
+        epi = EPI_ACCUMULATE if accumulate else EPI_STORE
+    if variant is None:
+        _check(lib().tl_gemm_bf16(_p(a), _p(w), _p(out), M, N, K, epi, _stream()))
+    else:
+        _check(lib().tl_gemm_bf16_variant(_p(a), _p(w), _p(out), M, N, K, epi, int(variant), _stream()))
+
+
+def bf16_gemm_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
+    return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.shape[1] % 8 == 0
+            and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
 
 def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
     """out[M,N] (+)= a[M,K] @ w[N,K]^T with float32 accumulation.  The kernel
     follows from the operand types: bfloat16 x bfloat16 goes to the matrix
     cores, anything with float32 in it to the plain FMA kernel."""
-    if (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.shape[1] % 8 == 0
-            and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0):
+    if bf16_gemm_ok(a, w):
         gemm_bf16(a, w, out, accumulate)
     else:
         gemm_plain(a, w, out, accumulate)
 
 
-def attn_prefill_bf16(q, k_new, v_new, pages, table, ring_pages: int, row_pos, cu_seqlens, n_cached,
-                      n_tiles: int, window: Optional[int], scale: float, out) -> None:
-    """bfloat16 attention for steps with many rows per sequence.  `n_tiles`:
-    sum over the sequences of ceil(rows / 128)."""
+def rope_commit(qkv: torch.Tensor, row_pos, inv_freq, table, ring_pages: int, nq: int, nkv: int, d: int,
+                q: torch.Tensor, pages: torch.Tensor) -> None:
+    """Single-token steps: rotate q and k, write q [n,nq,d] and put k and v of
+    row n straight into sequence n's page for its position."""
+    n = qkv.shape[0]
+    _req(qkv, "rope.qkv", torch.float32, (n, (nq + 2 * nkv) * d))
+    _req(row_pos, "rope.row_pos", torch.int32, (n,))
+    _req(inv_freq, "rope.inv_freq", torch.float32, (d // 2,))
+    _req(q, "rope.q", pages.dtype, (n, nq, d))
+    _req(table, "rope.table", torch.int32)
+    _req(pages, "rope.pages")
+    if pages.dim() != 5 or tuple(pages.shape[1:]) != (2, nkv, 64, d):
+        raise KernelError(f"rope.pages: shape {tuple(pages.shape)}, kernel needs [*, 2, {nkv}, 64, {d}]")
+    if table.dim() != 2 or table.shape[0] != n:
+        raise KernelError("rope.table: needs one row per sequence")
+    _check(lib().tl_rope_commit(_p(qkv), _p(row_pos), _p(inv_freq), _p(table), table.shape[1], ring_pages,
+                                n, nq, nkv, d, _p(q), _p(pages), _code(q.dtype), _stream()))
+
+
+def aligned_columns(n_cached, n_new):
+    """Column offsets (and their total) at which sequences lie when each is
+    given room from the last multiple of 64 below its cached length up to its
+    end, rounded up to 64: positions that are multiples of 64 then lie on
+    columns that are."""
+    off, total = [], 0
+    for c, n in zip(n_cached, n_new):
+        off.append(total)
+        total += -(-((int(c) % 64) + int(n)) // 64) * 64
+    return off, total
+
+
+def attn_prefill_bf16(q, k_new, vt_new, tile_off, pages, table, ring_pages: int, row_pos, cu_seqlens,
+                      n_cached, n_tiles: int, window: Optional[int], scale: float, out) -> None:
+    """bfloat16 attention for steps with many rows per sequence.  `vt_new`:
+    this step's values transposed [nkv, d, cols] at the columns that
+    `aligned_columns` gives (`tile_off`).  `n_tiles`: sum over the sequences
+    of ceil(rows / 128)."""
     n, nq, d = q.shape
     nkv = pages.shape[2]
     B = n_cached.shape[0]
     _req(q, "attn.q", torch.bfloat16)
     _req(k_new, "attn.k_new", torch.bfloat16, (n, nkv, d))
-    _req(v_new, "attn.v_new", torch.bfloat16, (n, nkv, d))
+    _req(vt_new, "attn.vt_new", torch.bfloat16)
+    if vt_new.dim() != 3 or tuple(vt_new.shape[:2]) != (nkv, d) or vt_new.shape[2] % 64:
+        raise KernelError(f"attn.vt_new: shape {tuple(vt_new.shape)}, kernel needs [{nkv}, {d}, 64 k]")
+    _req(tile_off, "attn.tile_off", torch.int32, (B,))
     _req(pages, "attn.pages", torch.bfloat16)
     if pages.dim() != 5 or tuple(pages.shape[1:]) != (2, nkv, 64, d):
         raise KernelError(f"attn.pages: shape {tuple(pages.shape)}, kernel needs [*, 2, nkv, 64, {d}]")
@@ -237,10 +301,10 @@ def attn_prefill_bf16(q, k_new, v_new, pages, table, ring_pages: int, row_pos, c
     _req(out, "attn.out", torch.bfloat16, (n, nq, d))
     if table.dim() != 2 or table.shape[0] != B:
         raise KernelError("attn.table: needs one row per sequence")
-    _check(lib().tl_attn_prefill_bf16(_p(q), _p(k_new), _p(v_new), _p(pages), _p(table), table.shape[1],
-                                      ring_pages, _p(row_pos), _p(cu_seqlens), _p(n_cached), B,
-                                      int(n_tiles), nq, nkv, d, int(window or 0), ctypes.c_float(scale),
-                                      _p(out), _stream()))
+    _check(lib().tl_attn_prefill_bf16(_p(q), _p(k_new), _p(vt_new), vt_new.shape[2], _p(tile_off), _p(pages),
+                                      _p(table), table.shape[1], ring_pages, _p(row_pos), _p(cu_seqlens),
+                                      _p(n_cached), B, int(n_tiles), nq, nkv, d, int(window or 0),
+                                      ctypes.c_float(scale), _p(out), _stream()))
 
 
 def attn_decode_bf16(q, pages, table, ring_pages: int, row_pos, window: Optional[int], scale: float,
@@ -269,32 +333,35 @@ def attn_decode_bf16(q, pages, table, ring_pages: int, row_pos, window: Optional
 
 def decode_splits(B: int, nq: int, nkv: int, max_pages: int) -> int:
     """Into how many parts the keys of a decode step are cut so that the chip
-    has some two workgroups a compute unit to run."""
+    has some four workgroups a compute unit to run."""
     groups = B * nkv * (-(-(nq // nkv) // 16))
-    return max(1, min(max_pages, -(-512 // groups)))
+    return max(1, min(-(-max_pages // 2), -(-1024 // groups), 4096))
+
+
+def uses_transposed_values(dtype: torch.dtype, d: int, all_single: bool) -> bool:
+    """Does `attention` take this step's values transposed (`vt_new`)?"""
+    return dtype == torch.bfloat16 and d % 16 == 0 and 16 <= d <= 256 and not all_single
 
 
 def attention(q, k_new, v_new, pages, table, ring_pages: int, ctx, n_cached, window, scale: float,
-              out) -> None:
+              out, vt_new=None) -> None:
     """Attention of a step's rows: keys j < n_cached[b] from the pages, later
     ones from this step's rows (`k_new`/`v_new`; None when everything is in
     the pages).  bfloat16 with head sizes in steps of 16 runs on the matrix
     cores, single-token steps and steps with longer rows each in their own
-    kernel; everything else runs in the plain kernel."""
+    kernel (the latter takes the values transposed, `vt_new`, see
+    `rope_split`); everything else runs in the plain kernel."""
     n, nq, d = q.shape
     fast = q.dtype == torch.bfloat16 and d % 16 == 0 and 16 <= d <= 256
     if fast and k_new is None and ctx.all_single:
         nkv = pages.shape[2]
-        max_pages = min(-(-ctx.max_len_after // 64), ring_pages)
-        if window:
-            max_pages = min(max_pages, -(-window // 64) + 1)
-        splits = decode_splits(n, nq, nkv, max_pages)
+        splits = decode_splits(n, nq, nkv, table.shape[1])      # by the table's width: fixed while a graph lives
         part = ctx.workspace.get("attn_part", (n * nq * splits * (d + 2),), torch.float32)
         attn_decode_bf16(q, pages, table, ring_pages, ctx.row_pos, window, scale, splits, part, out)
-    elif fast and k_new is not None:
+    elif fast and k_new is not None and vt_new is not None:
         n_tiles = int(sum(-(-int(x) // 128) for x in ctx.host["n_new"]))
-        attn_prefill_bf16(q, k_new, v_new, pages, table, ring_pages, ctx.row_pos, ctx.cu_seqlens,
-                          n_cached, n_tiles, window, scale, out)
+        attn_prefill_bf16(q, k_new, vt_new, ctx.tile_off, pages, table, ring_pages, ctx.row_pos,
+                          ctx.cu_seqlens, n_cached, n_tiles, window, scale, out)
     else:
-        attn_plain(q, k_new, v_new, pages, table, ring_pages, ctx.row_seq,
-                   ctx.row_pos, ctx.cu_seqlens, n_cached, window, scale, out)
+        attn_plain(q, k_new, v_new, pages, table, ring_pages, ctx.row_seq, ctx.row_pos, ctx.cu_seqlens,
+                   n_cached, window, scale, out)

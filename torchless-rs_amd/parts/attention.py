@@ -29,6 +29,8 @@ from .linear import Linear
 
 
 class AttentionMixer(Mixer):
+    graph_safe = True
+
     def __init__(self, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int,
                  position: PartSpec, window: Optional[int] = None, own_kv: bool = True,
                  prefix: str = "self_attn."):
@@ -74,20 +76,33 @@ class AttentionMixer(Mixer):
         inv_freq = self.position.inv_freq(y.device)
         q = ws.get("attn_q", (n, nq, d), ctx.dtype)
         out = ws.get("attn_out", (n, nq, d), ctx.dtype)
+        if self.own_kv and ctx.all_single and not run.kv_read_later:
+            # one token a sequence: k and v go straight into the pages, then everything is read there
+            qkv = ws.get("attn_qkv", (n, (nq + 2 * nkv) * d), torch.float32)
+            self.qkv(y, qkv)
+            ops.rope_commit(qkv, ctx.row_pos, inv_freq, table, group.ring_pages, nq, nkv, d, q, pages)
+            ops.attention(q, None, None, pages, table, group.ring_pages, ctx, ctx.len_after,
+                          self.window, self.scale, out)
+            self.o(out.view(n, nq * d), x, accumulate=True)
+            return
         if self.own_kv:
             tag = f"_{run.index}" if run.kv_read_later else ""
             qkv = ws.get("attn_qkv", (n, (nq + 2 * nkv) * d), torch.float32)
             self.qkv(y, qkv)
             k = ws.get("attn_k" + tag, (n, nkv, d), ctx.dtype)
             v = ws.get("attn_v" + tag, (n, nkv, d), ctx.dtype)
-            ops.rope_split(qkv, ctx.row_pos, inv_freq, nq, nkv, d, q, k, v)
+            vt = None
+            if ops.uses_transposed_values(ctx.dtype, d, ctx.all_single):
+                vt = ws.get("attn_vt" + tag, (nkv, d, ctx.host["aligned_cols"]), ctx.dtype)
+            ops.rope_split(qkv, ctx.row_pos, inv_freq, nq, nkv, d, q, k, v, vt, ctx.row_seq, ctx.tile_off,
+                           ctx.len_before)
             if run.kv_read_later:
-                ctx.host[f"kv_new_{run.index}"] = (k, v)
+                ctx.host[f"kv_new_{run.index}"] = (k, v, vt)
         else:
             qf = ws.get("attn_qkv", (n, nq * d), torch.float32)
             self.qkv(y, qf)
             ops.rope_split(qf, ctx.row_pos, inv_freq, nq, 0, d, q, None, None)
-            k, v = ctx.host[f"kv_new_{run.kv_source}"]
+            k, v, vt = ctx.host[f"kv_new_{run.kv_source}"]
         if ctx.all_single and not self.own_kv:
             ops.attention(q, None, None, pages, table, group.ring_pages, ctx, ctx.len_after,
                           self.window, self.scale, out)
@@ -97,7 +112,7 @@ class AttentionMixer(Mixer):
                           self.window, self.scale, out)
         else:
             ops.attention(q, k, v, pages, table, group.ring_pages, ctx, ctx.len_before,
-                          self.window, self.scale, out)
+                          self.window, self.scale, out, vt_new=vt)
             if self.own_kv:
                 def commit():
                     ops.kv_commit(k, v, ctx.row_seq, ctx.row_pos, ctx.len_after, table,

@@ -109,6 +109,11 @@ class Part:
     names); `load` receives them, already resident on the device in their
     stored width, and `compute_dtype` (float32 or bfloat16)."""
 
+    # True if `forward` of a single-token step launches the same kernels with the same
+    # arguments whatever the step's values are (everything that varies is read on the
+    # device): such a step can be captured once as a HIP graph and replayed.
+    graph_safe = False
+
     def weight_specs(self) -> Dict[str, WeightSpec]:
         return {}
 
@@ -200,6 +205,8 @@ class StepContext:
     slots: torch.Tensor                   # int32 [B]
     len_before: torch.Tensor              # int32 [B]
     len_after: torch.Tensor               # int32 [B]
+    tile_off: torch.Tensor                # int32 [B]  column of each sequence in buffers laid out by
+                                          #   `ops.aligned_columns` (host["aligned_cols"] in all)
     tables: Dict[int, torch.Tensor]       # group index -> int32 [B, stride] page ids
     all_single: bool                      # every sequence brings exactly one token
     max_new: int

@@ -19,6 +19,7 @@ class PreNormBlock(Part):
         self.mixer_norm = make_part("norm", layer.mixer_norm)
         self.ffn_norm = make_part("norm", layer.ffn_norm)
         self.n1, self.n2 = mixer_norm_name, ffn_norm_name
+        self.graph_safe = all(p.graph_safe for p in (self.mixer, self.ffn, self.mixer_norm, self.ffn_norm))
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
         out: Dict[str, WeightSpec] = {}

@@ -14,6 +14,8 @@ from .linear import Linear
 
 
 class TokenEmbedding(Part):
+    graph_safe = True
+
     def __init__(self, vocab_size: int, hidden_size: int, name: str = "embed_tokens.weight"):
         self.V, self.H, self.name = int(vocab_size), int(hidden_size), name
         self.table = None
@@ -30,6 +32,8 @@ class TokenEmbedding(Part):
 
 class LMHead(Part):
     """`tied`: use the embedding table instead of a tensor of its own."""
+    graph_safe = True
+
 
     def __init__(self, vocab_size: int, hidden_size: int, tied: bool = False, name: str = "weight"):
         self.V, self.H, self.tied, self.name = int(vocab_size), int(hidden_size), bool(tied), name

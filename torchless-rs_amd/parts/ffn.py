@@ -11,10 +11,12 @@ import torch
 from ..kernels import ops
 from ..weights.binding import WeightSpec
 from .base import FeedForward, register_part
-from .linear import Linear
+from .linear import Linear, interleave_pairs
 
 
 class SwiGLU(FeedForward):
+    graph_safe = True
+
     def __init__(self, hidden_size: int, intermediate_size: int, prefix: str = "mlp."):
         self.H = int(hidden_size)
         self.I = int(intermediate_size)
@@ -33,15 +35,22 @@ class SwiGLU(FeedForward):
         g, u = tensors[p + "gate_proj.weight"], tensors[p + "up_proj.weight"]
         if g.dtype != u.dtype:
             g, u = g.to(torch.float32), u.to(torch.float32)
-        self.gate_up = Linear(torch.cat([g, u], dim=0))
+        # bfloat16 on the matrix cores: gate and up rows interleaved so that the product's
+        # epilogue applies silu(gate) * up itself and writes bfloat16
+        self.paired = (compute_dtype == torch.bfloat16 and g.dtype == torch.bfloat16 and self.I % 32 == 0
+                       and self.H % 8 == 0)
+        self.gate_up = Linear(interleave_pairs(g, u) if self.paired else torch.cat([g, u], dim=0))
         self.down = Linear(tensors[p + "down_proj.weight"])
 
     def forward(self, ctx, y: torch.Tensor, x: torch.Tensor) -> None:
         n = y.shape[0]
-        gu = ctx.workspace.get("ffn_gu", (n, 2 * self.I), torch.float32)
-        self.gate_up(y, gu)
         h = ctx.workspace.get("ffn_h", (n, self.I), ctx.dtype)
-        ops.silu_mul(gu, h)
+        if self.paired and ops.bf16_gemm_ok(y, self.gate_up.weight):
+            ops.gemm_bf16(y, self.gate_up.weight, h, silu_pair=True)
+        else:
+            gu = ctx.workspace.get("ffn_gu", (n, 2 * self.I), torch.float32)
+            self.gate_up(y, gu)
+            ops.silu_mul(gu, h)
         self.down(h, x, accumulate=True)
 
 

@@ -20,3 +20,12 @@ class Linear:
     def __call__(self, a: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
         """out[M, N] (+)= a[M, K] @ W^T; out is float32."""
         ops.gemm(a, self.weight, out, accumulate)
+
+
+def interleave_pairs(gate: torch.Tensor, up: torch.Tensor, block: int = 32) -> torch.Tensor:
+    """Rows in groups of 2*block: `block` rows of gate, then the `block` rows of
+    up that belong to them: the layout of the products' paired epilogue."""
+    I, K = gate.shape
+    g = gate.view(I // block, block, K)
+    u = up.view(I // block, block, K)
+    return torch.stack([g, u], dim=1).reshape(2 * I, K).contiguous()
