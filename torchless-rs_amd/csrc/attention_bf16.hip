@@ -35,7 +35,7 @@ __device__ __forceinline__ bf16x8 z8() {
 constexpr int PF_BM = 128, PF_BN = 64, PF_VLD = PF_BN + 4;
 
 template <int DPAD>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256, DPAD <= 128 ? 2 : 1)
 attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
                     const bf16* __restrict__ vt_new, int vt_cols, const int* __restrict__ tile_off,
                     const bf16* __restrict__ pages, const int* __restrict__ table, int table_stride,
@@ -91,7 +91,38 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
 
   bf16x8 kfetch[PT], vfetch[PT];
   // tile j0 -> registers: keys as rows [key][d], values as rows [dv][key]
+  const int seq_end = p_first + n_new;               // one past the sequence's last position
   auto fetch = [&](int j0) {
+    if (j0 + PF_BN <= cached) {
+      // a cached page: keys [64][d], values [d][64]
+      const int page = table[(size_t)b * table_stride + (j0 / PAGE) % ring_pages];
+      const bf16* kpage = pages + (size_t)page * page_elems + (size_t)kvh * head_elems;
+      const bf16* vpage = kpage + (size_t)nkv * head_elems;
+#pragma unroll
+      for (int i = 0; i < PT; ++i) {
+        const int c = tid + 256 * i;
+        const int row = c / CH, col = (c % CH) * 8;
+        kfetch[i] = (col < d) ? ld8(kpage + (size_t)row * d + col) : z8();
+        const int dv = c / (PF_BN / 8), kc = (c % (PF_BN / 8)) * 8;
+        vfetch[i] = (dv < d) ? ld8(vpage + (size_t)dv * PAGE + kc) : z8();
+      }
+      return;
+    }
+    if (j0 >= cached && j0 + PF_BN <= seq_end) {
+      // rows of this step, all of them written
+      const bf16* krows = k_new + ((size_t)(row0 + j0 - cached) * nkv + kvh) * d;
+      const bf16* vcols = vt_head + (j0 - j_base);
+#pragma unroll
+      for (int i = 0; i < PT; ++i) {
+        const int c = tid + 256 * i;
+        const int row = c / CH, col = (c % CH) * 8;
+        kfetch[i] = (col < d) ? ld8(krows + (size_t)row * nkv * d + col) : z8();
+        const int dv = c / (PF_BN / 8), kc = (c % (PF_BN / 8)) * 8;
+        vfetch[i] = (dv < d) ? ld8(vcols + (size_t)dv * vt_cols + kc) : z8();
+      }
+      return;
+    }
+    // the tile that holds the boundary between cached and new rows, or the sequence's end
     const bool has_cached = j0 < cached, has_new = j0 + PF_BN > cached;
     const bf16* kpage = nullptr;
     if (has_cached) {
@@ -104,13 +135,13 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
       {   // keys: chunk c = (row, 8 columns)
         const int row = c / CH, col = (c % CH) * 8, j = j0 + row;
         bf16x8 kv = z8();
-        if (col < d && j <= p_hi) {
+        if (col < d && j < seq_end) {
           if (j < cached) kv = ld8(kpage + (size_t)row * d + col);
           else kv = ld8(k_new + ((size_t)(row0 + j - cached) * nkv + kvh) * d + col);
         }
         kfetch[i] = kv;
       }
-      {   // values: chunk c = (dv, 8 keys)
+      {   // values: chunk c = (dv, 8 keys); columns past the sequence's end were never written
         const int dv = c / (PF_BN / 8), kc = (c % (PF_BN / 8)) * 8;
         bf16x8 vv = z8();
         if (dv < d) {
@@ -120,7 +151,7 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
             const int j = j0 + kc + e;
-            vv[e] = (j < cached) ? cv[e] : ((j <= p_hi) ? nv[e] : (bf16)0.f);
+            vv[e] = (j < cached) ? cv[e] : ((j < seq_end) ? nv[e] : (bf16)0.f);
           }
         }
         vfetch[i] = vv;
@@ -168,39 +199,53 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
         const bf16x8 a = *reinterpret_cast<const bf16x8*>(&Ks[(nb * 32 + l32) * KLD + kb * 16 + 8 * half]);
         s[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[kb], s[nb], 0, 0, 0);
       }
-    // s[nb][r] = score of key j0 + 32 nb + 8 (r/4) + 4 half + r%4 with this lane's query
+    // s[nb][r] = k.q of key j0 + 32 nb + 8 (r/4) + 4 half + r%4 with this lane's query.
+    // Only tiles that cross the wave's causal edge, the window's edge or the rows' end need masks.
+    const bool edge = j0 + PF_BN - 1 > pw_lo || (window > 0 && j0 <= pw_hi - window) ||
+                      pw_lo + 31 > pw_hi;
+    if (edge) {
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int j = j0 + nb * 32 + 8 * (r / 4) + 4 * half + (r % 4);
+          const bool ok = q_ok && j <= p_me && (window == 0 || j > p_me - window);
+          s[nb][r] = ok ? s[nb][r] : -INFINITY;
+        }
+    }
     float tmax = -INFINITY;
 #pragma unroll
     for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int j = j0 + nb * 32 + 8 * (r / 4) + 4 * half + (r % 4);
-        const bool ok = q_ok && j <= p_me && (window == 0 || j > p_me - window);
-        const float v = ok ? s[nb][r] * scale : -INFINITY;
-        s[nb][r] = v;
-        tmax = fmaxf(tmax, v);
-      }
+      for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, s[nb][r]);
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
-    const float m_new = fmaxf(m, tmax);
+    const float m_new = fmaxf(m, tmax * scale);          // scale > 0: the maximum of the scaled scores
     const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-    const float alpha = __expf(m - m_use);
+    if (__ballot(m_new != m) != 0ull) {                  // the running maximum moved in some lane
+      const float alpha = __expf(m - m_use);
+      l *= alpha;
+#pragma unroll
+      for (int vb = 0; vb < VB; ++vb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[vb][r] *= alpha;
+      m = m_new;
+    }
+    // p = exp(s * scale - m) = 2^(s * c1 + c0)
+    const float c1 = scale * 1.44269504088896f, c0 = -m_use * 1.44269504088896f;
     float psum = 0.f;
     bf16x8 pb[2][2];
 #pragma unroll
     for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const float pv = __expf(s[nb][r] - m_use);
+        const float pv = __builtin_amdgcn_exp2f(fmaf(s[nb][r], c1, c0));
         psum += pv;
         pb[nb][r / 8][r % 8] = (bf16)pv;
       }
     psum += __shfl_xor(psum, 32, WAVE);
-    l = l * alpha + psum;
-    m = m_new;
+    l += psum;
 #pragma unroll
     for (int vb = 0; vb < VB; ++vb) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) o[vb][r] *= alpha;
 #pragma unroll
       for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
