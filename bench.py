@@ -37,6 +37,8 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=SHAPE["num_hidden_layers"])
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64")
+    ap.add_argument("--only", choices=["prefill", "decode"], default=None,
+                    help="measure one phase only and print its line to stderr (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not served")
@@ -102,6 +104,12 @@ def main() -> int:
             eng.free(s)
         return dt / steps, ctx_mid
 
+    if args.only == "decode":
+        sec, _ = run_decode(args.batch, args.context, args.steps, args.warmup)
+        print(f"[bench] decode b{args.batch}: {args.batch / sec:.1f} tok/s, {sec * 1e3:.3f} ms/step",
+              file=sys.stderr, flush=True)
+        return 0
+
     # prefill of one prompt
     T = args.prefill_tokens
     eng = Engine(model, max_tokens=T + 64, max_slots=1)
@@ -122,6 +130,8 @@ def main() -> int:
     prefill = {"value": round(T / (pre / 1e3), 1), "tokens": T, "ms": round(pre, 3),
                "frac": round(pre_flops / (pre / 1e3) / (PEAK_TFLOPS["bf16"] * 1e12), 4)}
     print(f"[bench] prefill {prefill}", file=sys.stderr, flush=True)
+    if args.only == "prefill":
+        return 0
 
     sec, ctx_mid = run_decode(args.batch, args.context, args.steps, args.warmup)
     held = min(ctx_mid, W) if W else ctx_mid
