@@ -283,7 +283,8 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
 // the split's pages in turn, each page as two groups of 32 keys read straight
 // from global memory into MFMA operands.  Per wave: running (max, sum, O^T);
 // the waves meet in LDS and the workgroup writes one partial per head:
-// part[(b, h, split)] = (max, sum, O[d]).  dec_combine merges the splits.
+// part[(b, h, split)] = (max, sum, O[d]), merged by attn_decode_combine; with one split the
+// result is written at once.
 constexpr int DC_WAVES = 4;
 
 template <int DPAD>   // multiple of 32
@@ -291,7 +292,7 @@ __global__ void __launch_bounds__(DC_WAVES * 64)
 attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
                    const int* __restrict__ table, int table_stride, int ring_pages,
                    const int* __restrict__ row_pos, int nq, int nkv, int d, int window, float scale,
-                   int n_splits, int head_groups, float* __restrict__ part) {
+                   int n_splits, int head_groups, float* __restrict__ part, bf16* __restrict__ out) {
   constexpr int KB = DPAD / 32, VB = DPAD / 16;
   __shared__ float red_o[VB * 4 * 64];
   __shared__ float red_ml[DC_WAVES][2][16];
@@ -436,7 +437,12 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
       ll += (mw == -INFINITY) ? 0.f : red_ml[w][1][hd] * __expf(mw - mh);
     }
     const int idx = ((dv / 16) * 4 + (dv % 4)) * 64 + ((dv % 16) / 4) * 16 + hd;
-    float* dst = part + (((size_t)b * nq + kvh * g + hg * 16 + hd) * n_splits + split) * (d + 2);
+    const size_t bh = (size_t)b * nq + kvh * g + hg * 16 + hd;
+    if (n_splits == 1) {                                // nothing to merge with
+      out[bh * d + dv] = (bf16)(red_o[idx] / ll);
+      continue;
+    }
+    float* dst = part + (bh * n_splits + split) * (d + 2);
     dst[2 + dv] = red_o[idx];
     if (dv == 0) {
       dst[0] = mh;
@@ -445,6 +451,9 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
   }
 }
 
+// Merge the splits of one (sequence, head): common maximum, weighted sums, in the order of the
+// splits.  (A second kernel and not the last workgroup of the first: what other XCDs wrote is
+// only sure to be seen across a kernel boundary without flushing L2 from inside the kernel.)
 __global__ void __launch_bounds__(64)
 attn_decode_combine_kernel(const float* __restrict__ part, int n_splits, int d, bf16* __restrict__ out) {
   extern __shared__ float fac[];                       // [n_splits] weight of each split
@@ -465,10 +474,8 @@ attn_decode_combine_kernel(const float* __restrict__ part, int n_splits, int d, 
   __syncthreads();
   for (int dv = lane; dv < d; dv += 64) {
     float acc = 0.f;
-    for (int s = 0; s < n_splits; ++s) {
-      const float f = fac[s];
-      if (f != 0.f) acc += src[(size_t)s * (d + 2) + 2 + dv] * f;
-    }
+#pragma unroll 4
+    for (int s = 0; s < n_splits; ++s) acc += src[(size_t)s * (d + 2) + 2 + dv] * fac[s];
     out[bh * d + dv] = (bf16)(acc / ll);
   }
 }
@@ -507,10 +514,12 @@ static int launch_decode(const bf16* q, const bf16* pages, const int* table, int
   dim3 grid(B * nkv * head_groups, n_splits);
   attn_decode_kernel<DPAD><<<grid, DC_WAVES * 64, 0, st>>>(q, pages, table, table_stride, ring_pages,
                                                             row_pos, nq, nkv, d, window, scale, n_splits,
-                                                            head_groups, part);
+                                                            head_groups, part, out);
   TL_LAUNCH_CHECK("attn_decode");
-  attn_decode_combine_kernel<<<B * nq, 64, n_splits * sizeof(float), st>>>(part, n_splits, d, out);
-  TL_LAUNCH_CHECK("attn_decode_combine");
+  if (n_splits > 1) {
+    attn_decode_combine_kernel<<<B * nq, 64, n_splits * sizeof(float), st>>>(part, n_splits, d, out);
+    TL_LAUNCH_CHECK("attn_decode_combine");
+  }
   return 0;
 }
 
@@ -553,7 +562,7 @@ extern "C" int tl_attn_prefill_bf16(const void* q, const void* k_new, const void
   return 1;
 }
 
-// part: float scratch of B * nq * n_splits * (d + 2) elements
+// part: float scratch of B * nq * n_splits * (d + 2) elements (not touched when n_splits is 1)
 extern "C" int tl_attn_decode_bf16(const void* q, const void* pages, const int* table, int table_stride,
                                    int ring_pages, const int* row_pos, int B, int nq, int nkv, int d,
                                    int window, float scale, int n_splits, float* part, void* out,

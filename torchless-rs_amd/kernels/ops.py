@@ -331,11 +331,21 @@ def attn_decode_bf16(q, pages, table, ring_pages: int, row_pos, window: Optional
                                      int(n_splits), _p(part), _p(out), _stream()))
 
 
+def decode_groups(B: int, nq: int, nkv: int) -> int:
+    """Workgroups of a decode step's attention before splitting: one per
+    (sequence, KV head, 16 query heads of its group)."""
+    return B * nkv * (-(-(nq // nkv) // 16))
+
+
+SPLIT_TARGET = 512          # workgroups a decode step's attention aims at
+
+
 def decode_splits(B: int, nq: int, nkv: int, max_pages: int) -> int:
     """Into how many parts the keys of a decode step are cut so that the chip
-    has some four workgroups a compute unit to run."""
-    groups = B * nkv * (-(-(nq // nkv) // 16))
-    return max(1, min(-(-max_pages // 2), -(-1024 // groups), 4096))
+    has some two workgroups a compute unit to run, each with at least
+    four pages (measured: more parts cost more in the merge than they gain)."""
+    groups = decode_groups(B, nq, nkv)
+    return max(1, min(-(-max_pages // 4), -(-SPLIT_TARGET // groups), 4096))
 
 
 def uses_transposed_values(dtype: torch.dtype, d: int, all_single: bool) -> bool:

@@ -175,14 +175,17 @@ class Workspace:
         self.device = device
         self._bufs: Dict[str, torch.Tensor] = {}
 
-    def get(self, name: str, shape: Tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
+    def get(self, name: str, shape: Tuple[int, ...], dtype: torch.dtype, zero: bool = False) -> torch.Tensor:
+        """`zero`: the buffer is zero when it is first made (not on later calls:
+        for counters that their kernels leave at zero)."""
         n = 1
         for s in shape:
             n *= int(s)
         key = f"{name}:{dtype}"
         buf = self._bufs.get(key)
         if buf is None or buf.numel() < n:
-            buf = torch.empty(max(n, 1), dtype=dtype, device=self.device)
+            make = torch.zeros if zero else torch.empty
+            buf = make(max(n, 1), dtype=dtype, device=self.device)
             self._bufs[key] = buf
         return buf[:n].view(shape)
 
