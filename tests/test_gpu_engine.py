@@ -385,3 +385,57 @@ def test_graph_replays_equal_eager_steps(zoo, dtype):
     assert replays > 50 and not eng_e._graphs
     want = plain.forward(z["w"], z["cfg"], ids[0][:75])[74:75]
     assert rel_err(outs[0][:1], want) < TOL[dtype]
+
+
+# ---- other storage widths and real layer sizes ------------------------------------------
+
+def test_float32_checkpoint_in_bfloat16_mode(tmp_path):
+    """A tensor stored in 32 bits stays so: activations and cache are bfloat16, the products
+    take float32 weights through the plain kernel."""
+    from torchless_rs_amd.engine import Engine, SeqInput, load_model
+    d = make_model_dir(tmp_path, "B", torch.float32)
+    cfg, w = read_model_dir(d)
+    assert w["lm_head.weight"].dtype == torch.float32
+    model = load_model(d, "bfloat16")
+    assert model.head.proj.weight.dtype == torch.float32 and model.dtype == torch.bfloat16
+    eng = Engine(model, max_tokens=256)
+    ids = prompts(cfg["vocab_size"], [40], seed=3)[0]
+    want = plain.forward(w, cfg, ids)
+    s = eng.alloc()
+    got = [eng.step([SeqInput(s, ids[:30], list(range(30)))]).clone()]
+    got += [eng.step([SeqInput(s, [t], [0])]).clone() for t in ids[30:]]
+    eng.free(s)
+    assert rel_err(torch.cat(got), want) < TOL["bfloat16"]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_layer_sizes_of_the_7b_shape(tmp_path, dtype):
+    """Two layers with the widths of Mistral 7B (4096 wide, 32 heads over 8 KV heads of 128,
+    14336 inner, 32000 words) and a window of 96, so that every kernel runs at its real sizes:
+    whole, in a batch with a shorter request, and with the last tokens one by one."""
+    from torchless_rs_amd import write_random_model
+    from torchless_rs_amd.engine import Engine, SeqInput, load_model
+    cfgd = {"architectures": ["MistralForCausalLM"], "num_hidden_layers": 2, "hidden_size": 4096,
+            "num_attention_heads": 32, "num_key_value_heads": 8, "intermediate_size": 14336,
+            "vocab_size": 32000, "rope_theta": 10000.0, "sliding_window": 96, "rms_norm_eps": 1e-5}
+    d = write_random_model(str(tmp_path / "wide"), cfgd, seed=5, std=0.02, dtype=torch.bfloat16)
+    cfg, w = read_model_dir(d)
+    ids = prompts(32000, [150, 70], seed=6)
+    wants = [plain.forward(w, cfg, p, dtype=torch.float32) for p in ids]
+    eng = Engine(load_model(d, dtype), max_tokens=64 * 8)
+    a, b = eng.alloc(), eng.alloc()
+    lg = eng.step([SeqInput(a, ids[0][:140], [0, 100, 139]), SeqInput(b, ids[1][:65], [64])]).clone()
+    assert rel_err(lg[:3], wants[0][[0, 100, 139]]) < TOL[dtype]
+    assert rel_err(lg[3:], wants[1][[64]]) < TOL[dtype]
+    outs_a, outs_b = [], []
+    for t in range(10):
+        batch = [SeqInput(a, [ids[0][140 + t]], [0])] + ([SeqInput(b, [ids[1][65 + t]], [0])] if t < 5 else [])
+        lg = eng.step(batch).clone()
+        outs_a.append(lg[:1])
+        if t < 5:
+            outs_b.append(lg[1:])
+        if t == 4:
+            eng.free(b)
+    eng.free(a)
+    assert rel_err(torch.cat(outs_a), wants[0][140:150]) < TOL[dtype]
+    assert rel_err(torch.cat(outs_b), wants[1][65:70]) < TOL[dtype]

@@ -506,3 +506,70 @@ def test_rope_commit_equals_rope_split_then_commit(ops, dt, window):
     assert torch.equal(q1, q2)
     assert torch.equal(torch.nan_to_num(pages1.float(), nan=-7.0), torch.nan_to_num(pages2.float(), nan=-7.0))
     assert not torch.equal(torch.nan_to_num(pages2.float(), nan=-7.0), torch.nan_to_num(a["pages"].float(), nan=-7.0))
+
+
+# ---- 17..64 rows: shared activations, K cut into partial sums -----------------------------
+
+@pytest.mark.parametrize("M", [17, 32, 33, 48, 50, 64, 5])
+@pytest.mark.parametrize("N,K,S", [(50, 72, 1), (64, 512, 2), (130, 776, 3), (200, 2000, 7), (384, 96, 1), (96, 4096, 16)])
+def test_gemm_mid_bf16(ops, M, N, K, S):
+    a = rnd(M, K, seed=41, dtype=torch.bfloat16)
+    w = rnd(N, K, seed=42, dtype=torch.bfloat16)
+    want = a.double() @ w.double().t()
+    if S == 1:
+        out = torch.full((M, N), float("nan"), device=DEV)
+        ops.gemm_mid_bf16(a.to(DEV), w.to(DEV), out)
+        assert rel_err(out, want) < 3e-6
+        base = rnd(M, N, seed=43)
+        acc = base.clone().to(DEV)
+        ops.gemm_mid_bf16(a.to(DEV), w.to(DEV), acc, accumulate=True)
+        assert rel_err(acc, want + base.double()) < 3e-6
+        return
+    parts = torch.full((S, M, N), float("nan"), device=DEV)
+    ops.gemm_mid_bf16(a.to(DEV), w.to(DEV), parts, S)
+    assert rel_err(parts.sum(0), want) < 3e-6
+    base = rnd(M, N, seed=44)
+    x = base.clone().to(DEV)
+    ops.add_partials(x, parts)
+    assert rel_err(x, want + base.double()) < 3e-6
+    if N % 4 == 0:
+        x2 = base.clone().to(DEV)
+        g = (1 + 0.1 * rnd(N, seed=45)).to(DEV)
+        y = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+        ops.add_rmsnorm(x2, parts, g, 1e-5, y)
+        assert torch.equal(x2, x)
+        assert rel_err(y, plain.rmsnorm(x.double().cpu(), g.double().cpu(), 1e-5)) < KTOL["bfloat16"]
+
+
+@pytest.mark.parametrize("M", [20, 64])
+def test_gemm_mid_paired_silu_and_row_independence(ops, M):
+    from torchless_rs_amd.parts.linear import interleave_pairs
+    I, K = 160, 200
+    a = rnd(M, K, seed=46, dtype=torch.bfloat16)
+    g = rnd(I, K, seed=47, dtype=torch.bfloat16, scale=0.3)
+    u = rnd(I, K, seed=48, dtype=torch.bfloat16, scale=0.3)
+    out = torch.full((M, I), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.gemm_mid_bf16(a.to(DEV), interleave_pairs(g, u).to(DEV), out, silu_pair=True)
+    want = plain.silu(a.double() @ g.double().t()) * (a.double() @ u.double().t())
+    assert rel_err(out, want) < KTOL["bfloat16"]
+    # a row's result does not depend on the other rows of the batch
+    w = rnd(96, K, seed=49, dtype=torch.bfloat16).to(DEV)
+    full = torch.empty(M, 96, device=DEV)
+    ops.gemm_mid_bf16(a.to(DEV), w, full)
+    few = torch.empty(17, 96, device=DEV)
+    ops.gemm_mid_bf16(a[:17].contiguous().to(DEV), w, few)
+    assert torch.equal(few, full[:17])
+
+
+def test_rope_commit_adds_partial_products(ops):
+    from torchless_rs_amd.parts.position import Rotary
+    nq, nkv, d = 6, 2, 48
+    a = paged_case(ops, "bfloat16", nq, nkv, d, None, lens_cached=[0, 63, 64, 300], lens_new=[1] * 4, seed=7)
+    qkv = rnd(3, 4, (nq + 2 * nkv) * d, seed=8).to(DEV)
+    inv = Rotary(d, 777.0).inv_freq(DEV)
+    q1, q2 = (torch.empty(4, nq, d, dtype=torch.bfloat16, device=DEV) for _ in range(2))
+    p1, p2 = a["pages"].clone(), a["pages"].clone()
+    ops.rope_commit((qkv[0] + qkv[1] + qkv[2]).contiguous(), a["row_pos"], inv, a["table"], a["ring"], nq, nkv, d, q1, p1)
+    ops.rope_commit(qkv, a["row_pos"], inv, a["table"], a["ring"], nq, nkv, d, q2, p2)
+    assert torch.equal(q1, q2)
+    assert torch.equal(torch.nan_to_num(p1.float(), nan=-7.0), torch.nan_to_num(p2.float(), nan=-7.0))

@@ -50,12 +50,14 @@ def test_position_part():
         make_part("position", PartSpec("rotary", {"head_dim": 7, "theta": 1.0}))
 
 
+@pytest.mark.parametrize("n", [7, 40])
 @pytest.mark.parametrize("dt", ["float32", "bfloat16"])
-def test_feed_forward_part(dt):
+def test_feed_forward_part(dt, n):
     from torchless_rs_amd.cache import Cache
     from torchless_rs_amd.engine import SeqInput
     from torchless_rs_amd.parts import PartSpec, make_part
-    H, I, n = 72, 200, 7
+    from torchless_rs_amd.parts.base import flush_pending
+    H, I = 72, 224
     ffn = make_part("ffn", PartSpec("swiglu", {"hidden_size": H, "intermediate_size": I}))
     w = {"mlp.gate_proj.weight": rnd(I, H, seed=3, scale=0.2, dtype=DT[dt]),
          "mlp.up_proj.weight": rnd(I, H, seed=4, scale=0.2, dtype=DT[dt]),
@@ -69,6 +71,7 @@ def test_feed_forward_part(dt):
     x0 = rnd(n, H, seed=7)
     x = x0.clone().to(DEV)
     ffn.forward(ctx, y.to(DEV), x)
+    flush_pending(ctx, x)
     want = x0.double() + plain.swiglu(y.double(), {k: v.double() for k, v in w.items()}, "")
     assert rel_err(x, want) < PTOL[dt]
 
@@ -80,6 +83,7 @@ def test_attention_part_whole_and_in_steps(dt, nq, nkv, d, window):
     from torchless_rs_amd.cache import Cache
     from torchless_rs_amd.engine import SeqInput
     from torchless_rs_amd.parts import PartSpec, RunBinding, make_part
+    from torchless_rs_amd.parts.base import flush_pending
     H, lens = 40, [90, 13]
     mixer = make_part("mixer", PartSpec("attention", {
         "hidden_size": H, "n_heads": nq, "n_kv_heads": nkv, "head_dim": d, "window": window,
@@ -106,6 +110,7 @@ def test_attention_part_whole_and_in_steps(dt, nq, nkv, d, window):
     ctx = context(cache, batch, DT[dt])
     x = torch.zeros(sum(lens), H, device=DEV)
     mixer.forward(ctx, run, torch.cat(ys).to(DEV), x)
+    flush_pending(ctx, x)               # a part may leave partial products for the next reader of x
     cache.commit([(s, n) for s, n in zip(slots, lens)])
     assert rel_err(x, want) < PTOL[dt]
     for s in slots:
@@ -117,6 +122,7 @@ def test_attention_part_whole_and_in_steps(dt, nq, nkv, d, window):
     ctx = context(cache, [SeqInput(s, [0] * h, []) for s, h in zip(slots, heads)], DT[dt])
     x = torch.zeros(sum(heads), H, device=DEV)
     mixer.forward(ctx, run, torch.cat([y[:h] for y, h in zip(ys, heads)]).to(DEV), x)
+    flush_pending(ctx, x)
     cache.commit(list(zip(slots, heads)))
     got[0].append(x[:50].clone()); got[1].append(x[50:].clone())
     fed = list(heads)
@@ -125,6 +131,7 @@ def test_attention_part_whole_and_in_steps(dt, nq, nkv, d, window):
         ctx = context(cache, [SeqInput(slots[i], [0], []) for i in live], DT[dt])
         x = torch.zeros(len(live), H, device=DEV)
         mixer.forward(ctx, run, torch.stack([ys[i][fed[i]] for i in live]).to(DEV), x)
+        flush_pending(ctx, x)
         cache.commit([(slots[i], 1) for i in live])
         for r, i in enumerate(live):
             got[i].append(x[r:r + 1].clone())

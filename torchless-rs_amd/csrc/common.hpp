@@ -64,6 +64,14 @@ template <int NT> __device__ __forceinline__ float block_max(float v, float* sh)
   return r;
 }
 
+// Rotation of a pair by (c, s), each product and the sum rounded on its own (no fused
+// multiply-add), so that every kernel that rotates gives the same bits:
+// a' = a c - b s ; b' = a s + b c   (src/kernels/mod.rs:603-605 of the reference)
+__device__ __forceinline__ void rotate_pair(float a, float b, float c, float s, float& ra, float& rb) {
+  ra = __fsub_rn(__fmul_rn(a, c), __fmul_rn(b, s));
+  rb = __fadd_rn(__fmul_rn(a, s), __fmul_rn(b, c));
+}
+
 // ---- error channel -------------------------------------------------------
 void set_error(const char* fmt, ...);
 

@@ -82,6 +82,57 @@ __global__ void __launch_bounds__(256) rmsnorm_reg_kernel(const float* __restric
   }
 }
 
+// x += sum of the partial products P[s][n][H] (in the order of s), then the norm of the new x.
+template <typename TO, int IT>
+__global__ void __launch_bounds__(256)
+add_rmsnorm_reg_kernel(float* __restrict__ x, const float* __restrict__ parts, int n_parts, size_t part_stride,
+                       const float* __restrict__ w, float eps, TO* __restrict__ out, int H) {
+  __shared__ float sh[4];
+  const int n = blockIdx.x;
+  float4* xr = reinterpret_cast<float4*>(x + (size_t)n * H);
+  const float4* wr = reinterpret_cast<const float4*>(w);
+  const int nv = H / 4;
+  float4 v[IT], g[IT];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < IT; ++i) {
+    const int c = threadIdx.x + 256 * i;
+    if (c < nv) {
+      float4 a = xr[c];
+      for (int s = 0; s < n_parts; ++s) {
+        const float4 p = reinterpret_cast<const float4*>(parts + s * part_stride + (size_t)n * H)[c];
+        a.x += p.x; a.y += p.y; a.z += p.z; a.w += p.w;
+      }
+      xr[c] = a;
+      v[i] = a;
+      g[i] = wr[c];
+      ss += a.x * a.x + a.y * a.y + a.z * a.z + a.w * a.w;
+    }
+  }
+  ss = block_sum<256>(ss, sh);
+  const float rms = sqrtf(ss / (float)H + eps);
+  TO* o = out + (size_t)n * H;
+#pragma unroll
+  for (int i = 0; i < IT; ++i) {
+    const int c = threadIdx.x + 256 * i;
+    if (c < nv) {
+      o[4 * c + 0] = from_f32<TO>((v[i].x / rms) * g[i].x);
+      o[4 * c + 1] = from_f32<TO>((v[i].y / rms) * g[i].y);
+      o[4 * c + 2] = from_f32<TO>((v[i].z / rms) * g[i].z);
+      o[4 * c + 3] = from_f32<TO>((v[i].w / rms) * g[i].w);
+    }
+  }
+}
+
+__global__ void add_partials_kernel(float* __restrict__ x, const float* __restrict__ parts, int n_parts,
+                                    size_t part_stride, size_t total) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  float a = x[i];
+  for (int s = 0; s < n_parts; ++s) a += parts[s * part_stride + i];
+  x[i] = a;
+}
+
 // ---- rotation and split ------------------------------------------------------
 // qkv[n, :] = [q (nq*d) | k (nkv*d) | v (nkv*d)] in float.  q and k are rotated
 // in pairs (i, i + d/2) by the angle pos * inv_freq[i]; v is copied.
@@ -110,7 +161,8 @@ __global__ void rope_split_kernel(const float* __restrict__ qkv, const int* __re
     const int h = t / half, i = t % half;
     const float c = cs[i], s = sn[i];
     const float a = src[h * d + i], b = src[h * d + i + half];
-    const float ra = a * c - b * s, rb = a * s + b * c;
+    float ra, rb;
+    rotate_pair(a, b, c, s, ra, rb);
     TO* dst = (h < nq) ? q + ((size_t)n * nq + h) * d : k + ((size_t)n * nkv + (h - nq)) * d;
     dst[i] = from_f32<TO>(ra);
     dst[i + half] = from_f32<TO>(rb);
@@ -156,8 +208,10 @@ __global__ void kv_commit_kernel(const T* __restrict__ k, const T* __restrict__ 
 
 // ---- single-token steps: rotate, and put k and v straight into the pages ------
 // Row n is the one new token of sequence n (position row_pos[n]).
+// qkv may come as n_parts partial products (part_stride elements apart) that are added up here.
 template <typename T>
-__global__ void rope_commit_kernel(const float* __restrict__ qkv, const int* __restrict__ row_pos,
+__global__ void rope_commit_kernel(const float* __restrict__ qkv, int n_parts, size_t part_stride,
+                                   const int* __restrict__ row_pos,
                                    const float* __restrict__ inv_freq, const int* __restrict__ table,
                                    int table_stride, int ring_pages, int nq, int nkv, int d,
                                    T* __restrict__ q, T* __restrict__ pages) {
@@ -181,14 +235,23 @@ __global__ void rope_commit_kernel(const float* __restrict__ qkv, const int* __r
   for (int t = threadIdx.x; t < n_rot; t += blockDim.x) {
     const int h = t / half, i = t % half;
     const float c = cs[i], s = sn[i];
-    const float a = src[h * d + i], b = src[h * d + i + half];
-    const float ra = a * c - b * s, rb = a * s + b * c;
+    float a = src[h * d + i], b = src[h * d + i + half];
+    for (int sp = 1; sp < n_parts; ++sp) {
+      a += src[sp * part_stride + h * d + i];
+      b += src[sp * part_stride + h * d + i + half];
+    }
+    float ra, rb;
+    rotate_pair(a, b, c, s, ra, rb);
     T* dst = (h < nq) ? q + ((size_t)n * nq + h) * d : kd + ((size_t)(h - nq) * PAGE + r) * d;
     dst[i] = from_f32<T>(ra);
     dst[i + half] = from_f32<T>(rb);
   }
   const float* vs = src + (size_t)(nq + nkv) * d;
-  for (int t = threadIdx.x; t < nkv * d; t += blockDim.x) vd[(size_t)t * PAGE + r] = from_f32<T>(vs[t]);
+  for (int t = threadIdx.x; t < nkv * d; t += blockDim.x) {
+    float a = vs[t];
+    for (int sp = 1; sp < n_parts; ++sp) a += vs[sp * part_stride + t];
+    vd[(size_t)t * PAGE + r] = from_f32<T>(a);
+  }
 }
 
 // ---- h = silu(gate) * up, silu(g) = g / (1 + exp(-g)) ------------------------
@@ -260,6 +323,39 @@ int tl_rmsnorm(const float* x, const float* w, float eps, void* out, int out_dt,
 
 // vt (may be null): values also transposed, [nkv][d][vt_cols], row n in column
 // tile_off[row_seq[n]] + row_pos[n] - 64 * (n_cached[row_seq[n]] / 64)
+// x[n, H] += parts[0..n_parts)[n, H]; out = rmsnorm(x)
+int tl_add_rmsnorm(float* x, const float* parts, int n_parts, const float* w, float eps, void* out, int out_dt,
+                   int n, int H, hipStream_t st) {
+  TL_REQUIRE(n >= 0 && H > 0 && n_parts >= 0, "add_rmsnorm: bad sizes n=%d H=%d parts=%d", n, H, n_parts);
+  TL_REQUIRE(out_dt == DT_F32 || out_dt == DT_BF16, "add_rmsnorm: unknown dtype code %d", out_dt);
+  TL_REQUIRE(H % 4 == 0 && H <= 8192 && ((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0) &&
+             ((uintptr_t)parts % 16 == 0), "add_rmsnorm: H=%d must be a multiple of 4, at most 8192, rows 16-byte aligned", H);
+  if (n == 0) return 0;
+  const size_t stride = (size_t)n * H;
+#define TL_ARMS(IT)                                                                                        \
+  do {                                                                                                     \
+    if (out_dt == DT_F32) add_rmsnorm_reg_kernel<float, IT><<<n, 256, 0, st>>>(x, parts, n_parts, stride, w, eps, (float*)out, H); \
+    else add_rmsnorm_reg_kernel<bf16, IT><<<n, 256, 0, st>>>(x, parts, n_parts, stride, w, eps, (bf16*)out, H);                   \
+  } while (0)
+  if (H <= 1024) TL_ARMS(1);
+  else if (H <= 2048) TL_ARMS(2);
+  else if (H <= 4096) TL_ARMS(4);
+  else TL_ARMS(8);
+#undef TL_ARMS
+  TL_LAUNCH_CHECK("add_rmsnorm");
+  return 0;
+}
+
+// x[n, H] += parts[0..n_parts)[n, H]
+int tl_add_partials(float* x, const float* parts, int n_parts, int n, int H, hipStream_t st) {
+  TL_REQUIRE(n >= 0 && H > 0 && n_parts >= 0, "add_partials: bad sizes n=%d H=%d parts=%d", n, H, n_parts);
+  if (n == 0 || n_parts == 0) return 0;
+  const size_t total = (size_t)n * H;
+  add_partials_kernel<<<(unsigned)((total + 255) / 256), 256, 0, st>>>(x, parts, n_parts, total, total);
+  TL_LAUNCH_CHECK("add_partials");
+  return 0;
+}
+
 int tl_rope_split(const float* qkv, const int* row_pos, const float* inv_freq, int n, int nq,
                   int nkv, int d, void* q, void* k, void* v, void* vt, int vt_cols, const int* row_seq,
                   const int* tile_off, const int* n_cached, int out_dt, hipStream_t st) {
@@ -303,20 +399,23 @@ int tl_kv_commit(const void* k, const void* v, int dt, const int* row_seq, const
   return 0;
 }
 
-int tl_rope_commit(const float* qkv, const int* row_pos, const float* inv_freq, const int* table,
+// n_parts >= 1: qkv is [n_parts][n][(nq + 2 nkv) d], summed on the way in
+int tl_rope_commit(const float* qkv, int n_parts, const int* row_pos, const float* inv_freq, const int* table,
                    int table_stride, int ring_pages, int n, int nq, int nkv, int d, void* q, void* pages,
                    int dt, hipStream_t st) {
   TL_REQUIRE(n >= 0 && nq > 0 && nkv > 0 && d > 0 && d % 2 == 0 && ring_pages > 0 && table_stride > 0,
              "rope_commit: bad sizes n=%d nq=%d nkv=%d d=%d ring_pages=%d table_stride=%d", n, nq, nkv, d,
              ring_pages, table_stride);
   TL_REQUIRE(d <= 2 * ROPE_MAX_HALF, "rope_commit: head size %d is not served (at most %d)", d, 2 * ROPE_MAX_HALF);
+  TL_REQUIRE(n_parts >= 1, "rope_commit: n_parts=%d", n_parts);
   if (n == 0) return 0;
+  const size_t stride = (size_t)n * (nq + 2 * nkv) * d;
   if (dt == DT_F32)
-    rope_commit_kernel<float><<<n, 256, 0, st>>>(qkv, row_pos, inv_freq, table, table_stride, ring_pages,
-                                                  nq, nkv, d, (float*)q, (float*)pages);
+    rope_commit_kernel<float><<<n, 256, 0, st>>>(qkv, n_parts, stride, row_pos, inv_freq, table, table_stride,
+                                                  ring_pages, nq, nkv, d, (float*)q, (float*)pages);
   else if (dt == DT_BF16)
-    rope_commit_kernel<bf16><<<n, 256, 0, st>>>(qkv, row_pos, inv_freq, table, table_stride, ring_pages, nq,
-                                                 nkv, d, (bf16*)q, (bf16*)pages);
+    rope_commit_kernel<bf16><<<n, 256, 0, st>>>(qkv, n_parts, stride, row_pos, inv_freq, table, table_stride,
+                                                 ring_pages, nq, nkv, d, (bf16*)q, (bf16*)pages);
   else
     TL_REQUIRE(false, "rope_commit: unknown dtype code %d", dt);
   TL_LAUNCH_CHECK("rope_commit");

@@ -147,6 +147,142 @@ static int launch_skinny(const bf16* A, const bf16* W, float* C, int M, int N, i
   return 0;
 }
 
+// ------------------------------------------------------------------- mid ----
+// 17..64 rows (decode at larger batches).  Per byte of W there are now enough
+// MFMAs that the activations must be shared: a workgroup owns 64 output
+// channels (one 16-channel tile per wave) and a slice of K; the activations of
+// a k-step go through LDS once for the four waves, W streams from global
+// memory into registers.  With n_split > 1 the slices of K go to different
+// workgroups, which write partial sums P[split][M][N]; the kernel that reads
+// them next adds them up (always in the order of the splits).
+template <int MT, int KS>      // KS: k per step (a multiple of 64); everything of a step is in flight at once
+__global__ void __launch_bounds__(256)
+gemm_mid_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float* __restrict__ C, int M,
+                int N, int K, int steps_per_split, int epilogue) {
+  constexpr int ROWS = MT * 16, LD = KS + 8, SUB = KS / 64;
+  __shared__ __attribute__((aligned(16))) bf16 As[ROWS * LD];
+  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64, li = lane % 16, kg = lane / 16;
+  const int n0 = blockIdx.x * 64 + wave * 16;
+  const bf16* wrow = W + (size_t)min(n0 + li, N - 1) * K;
+  const int steps = (K + KS - 1) / KS;
+  const int s_begin = blockIdx.y * steps_per_split, s_end = min(steps, s_begin + steps_per_split);
+
+  // activations: ROWS x KS/8 chunks of 8 per step, shared out over the 256 threads
+  constexpr int CPR = KS / 8, CHUNKS = ROWS * CPR, PER = (CHUNKS + 255) / 256;
+  bf16x8 areg[PER];
+  auto fetch_a = [&](int s) {
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int c = tid + 256 * i;
+      const int row = c / CPR, k = s * KS + (c % CPR) * 8;
+      areg[i] = (c < CHUNKS && k + 8 <= K) ? load8(A + (size_t)min(row, M - 1) * K + k) : zero8();
+    }
+  };
+  auto stash_a = [&]() {
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int c = tid + 256 * i;
+      if (c < CHUNKS) *reinterpret_cast<bf16x8*>(&As[(c / CPR) * LD + (c % CPR) * 8]) = areg[i];
+    }
+  };
+  bf16x8 wreg[SUB][2], wnext[SUB][2];
+  auto fetch_w = [&](int s, bf16x8 (&w)[SUB][2]) {
+#pragma unroll
+    for (int j = 0; j < SUB; ++j) {
+      const int k = s * KS + j * 64 + kg * 16;
+      w[j][0] = (k + 8 <= K) ? load8(wrow + k) : zero8();
+      w[j][1] = (k + 16 <= K) ? load8(wrow + k + 8) : zero8();
+    }
+  };
+
+  f32x4 acc[MT];
+#pragma unroll
+  for (int u = 0; u < MT; ++u) acc[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  if (s_begin < s_end) {
+    fetch_a(s_begin);
+    fetch_w(s_begin, wreg);
+  }
+  for (int s = s_begin; s < s_end; ++s) {
+    __syncthreads();                 // the previous step's activations have been read
+    stash_a();
+    __syncthreads();
+    if (s + 1 < s_end) {
+      fetch_a(s + 1);
+      fetch_w(s + 1, wnext);
+    }
+#pragma unroll
+    for (int j = 0; j < SUB; ++j)
+#pragma unroll
+      for (int u = 0; u < MT; ++u) {
+        const bf16* ar = &As[(u * 16 + li) * LD + j * 64 + kg * 16];
+        const bf16x8 a0 = *reinterpret_cast<const bf16x8*>(ar), a1 = *reinterpret_cast<const bf16x8*>(ar + 8);
+        acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, wreg[j][0], acc[u], 0, 0, 0);
+        acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, wreg[j][1], acc[u], 0, 0, 0);
+      }
+#pragma unroll
+    for (int j = 0; j < SUB; ++j) {
+      wreg[j][0] = wnext[j][0];
+      wreg[j][1] = wnext[j][1];
+    }
+  }
+  // acc[u][r] = D[m = 16 u + 4 kg + r][n = n0 + li]
+  if (epilogue == EPI_SILU_PAIR) {
+    // the workgroup's 64 rows are one group: waves 0,1 hold gate rows, waves 2,3 their up rows
+    __syncthreads();
+    float* ex = reinterpret_cast<float*>(&As[0]);           // [2 waves][MT][4][64] floats <= 8 KB
+    if (wave >= 2) {
+#pragma unroll
+      for (int u = 0; u < MT; ++u)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) ex[(((wave - 2) * MT + u) * 4 + r) * 64 + lane] = acc[u][r];
+    }
+    __syncthreads();
+    if (wave < 2) {
+      bf16* H = reinterpret_cast<bf16*>(C);
+      const int NH = N / 2;
+      const int n = blockIdx.x * 32 + wave * 16 + li;
+#pragma unroll
+      for (int u = 0; u < MT; ++u)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int m = 16 * u + 4 * kg + r;
+          if (m < M && n < NH) {
+            const float g = acc[u][r], up = ex[((wave * MT + u) * 4 + r) * 64 + lane];
+            H[(size_t)m * NH + n] = (bf16)((g / (1.0f + expf(-g))) * up);
+          }
+        }
+    }
+    return;
+  }
+  float* dst = C + (size_t)blockIdx.y * M * N;              // the split's own partial (split 0: C itself)
+  const int n = n0 + li;
+  if (n < N) {
+#pragma unroll
+    for (int u = 0; u < MT; ++u)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int m = 16 * u + 4 * kg + r;
+        if (m < M) {
+          float* c = dst + (size_t)m * N + n;
+          *c = (epilogue == EPI_ACCUMULATE) ? *c + acc[u][r] : acc[u][r];
+        }
+      }
+  }
+}
+
+constexpr int MID_KS = 256;
+
+template <int MT>
+static int launch_mid(const bf16* A, const bf16* W, float* C, int M, int N, int K, int n_split, int epilogue,
+                      hipStream_t st) {
+  const int steps = (K + MID_KS - 1) / MID_KS, per = (steps + n_split - 1) / n_split;
+  dim3 grid((N + 63) / 64, n_split);
+  gemm_mid_kernel<MT, MID_KS><<<grid, 256, 0, st>>>(A, W, C, M, N, K, per, epilogue);
+  TL_LAUNCH_CHECK("gemm_mid");
+  return 0;
+}
+
 // ----------------------------------------------------------------- tiled ----
 constexpr int TM = 128, TN = 128, TK = 64, TPAD = 8, TLD = TK + TPAD;
 
@@ -458,4 +594,27 @@ extern "C" int tl_gemm_bf16_variant(const void* A, const void* W, void* C, int M
     case 142: return launch_skinny<1, 4, 8>(a, w, c, M, N, K, epilogue, st);
   }
   TL_REQUIRE(false, "gemm_bf16: unknown variant %d", variant);
+}
+
+// 17..64 rows.  n_split == 1: C as in tl_gemm_bf16 (all three epilogues).  n_split > 1: C is
+// float [n_split][M][N] and receives partial sums (epilogue must be 0); every split gets at
+// least one k-step of 256.
+extern "C" int tl_gemm_mid_bf16(const void* A, const void* W, void* C, int M, int N, int K, int n_split,
+                                int epilogue, hipStream_t st) {
+  TL_REQUIRE(M > 0 && M <= 64 && N > 0 && K > 0 && K % 8 == 0, "gemm_mid: bad sizes M=%d N=%d K=%d (M at most 64, "
+             "K a multiple of 8)", M, N, K);
+  TL_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "gemm_mid: operands must be 16-byte aligned");
+  TL_REQUIRE(n_split >= 1 && n_split <= (K + MID_KS - 1) / MID_KS && n_split <= 65535,
+             "gemm_mid: %d splits do not fit K=%d (one step of %d at least each)", n_split, K, MID_KS);
+  TL_REQUIRE(epilogue >= 0 && epilogue <= 2 && (n_split == 1 || epilogue == EPI_STORE),
+             "gemm_mid: epilogue %d cannot go with %d splits", epilogue, n_split);
+  TL_REQUIRE(epilogue != EPI_SILU_PAIR || N % 64 == 0, "gemm_mid: the paired epilogue needs N=%d to be a "
+             "multiple of 64", N);
+  const bf16* a = (const bf16*)A;
+  const bf16* w = (const bf16*)W;
+  float* c = (float*)C;
+  if (M <= 16) return launch_mid<1>(a, w, c, M, N, K, n_split, epilogue, st);
+  if (M <= 32) return launch_mid<2>(a, w, c, M, N, K, n_split, epilogue, st);
+  if (M <= 48) return launch_mid<3>(a, w, c, M, N, K, n_split, epilogue, st);
+  return launch_mid<4>(a, w, c, M, N, K, n_split, epilogue, st);
 }

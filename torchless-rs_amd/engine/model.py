@@ -14,7 +14,7 @@ import torch
 
 from ..cache.cache import Cache, KVRequest, StateRequest
 from ..config.base import ModelConfig
-from ..parts.base import ModelSpec, PartSpec, RunBinding, StepContext, make_part
+from ..parts.base import ModelSpec, PartSpec, RunBinding, StepContext, flush_pending, make_part
 from ..weights.binding import bind_weights
 
 
@@ -110,6 +110,7 @@ class Model:
             self.blocks[run.layer].forward(ctx, binding, x)
         for commit in ctx.host.pop("deferred", []):
             commit()
+        flush_pending(ctx, x)
         logits = ws.get("logits", (n_want, V), torch.float32)
         if n_want:
             xs = ws.get("head_x", (n_want, H), torch.float32)

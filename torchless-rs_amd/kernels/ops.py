@@ -230,6 +230,61 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: b
         _check(lib().tl_gemm_bf16_variant(_p(a), _p(w), _p(out), M, N, K, epi, int(variant), _stream()))
 
 
+def mid_splits(M: int, N: int, K: int) -> int:
+    """For 17..64 rows: into how many slices K is cut so that some 400
+    workgroups (64 output channels each) are at work; 1 where N alone gives
+    them."""
+    blocks = -(-N // 64)
+    steps = -(-K // 256)
+    return max(1, min(-(-400 // blocks), steps, 16))
+
+
+def gemm_mid_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, n_split: int = 1,
+                  accumulate: bool = False, silu_pair: bool = False) -> None:
+    """The product for 17..64 rows.  n_split == 1: out as in `gemm_bf16`.
+    n_split > 1: out is float32 [n_split, M, N] and receives partial sums that
+    the next kernel adds up (`add_rmsnorm`, `add_partials`, `rope_commit`)."""
+    M, K = a.shape
+    N = w.shape[0]
+    _req(a, "gemm.a", torch.bfloat16)
+    _req(w, "gemm.w", torch.bfloat16, (N, K))
+    if n_split > 1:
+        if accumulate or silu_pair:
+            raise KernelError("gemm_mid: partial sums cannot be accumulated or paired")
+        _req(out, "gemm.out", torch.float32, (n_split, M, N))
+        epi = EPI_STORE
+    elif silu_pair:
+        _req(out, "gemm.out", torch.bfloat16, (M, N // 2))
+        epi = EPI_SILU_PAIR
+    else:
+        _req(out, "gemm.out", torch.float32, (M, N))
+        epi = EPI_ACCUMULATE if accumulate else EPI_STORE
+    _check(lib().tl_gemm_mid_bf16(_p(a), _p(w), _p(out), M, N, K, int(n_split), epi, _stream()))
+
+
+def add_rmsnorm(x: torch.Tensor, parts: torch.Tensor, w: torch.Tensor, eps: float, out: torch.Tensor) -> None:
+    """x += parts[0] + parts[1] + ... (float32 [S, n, H]); out = rmsnorm(x)."""
+    n, H = x.shape
+    _req(x, "add_rmsnorm.x", torch.float32)
+    _req(parts, "add_rmsnorm.parts", torch.float32)
+    if parts.dim() != 3 or tuple(parts.shape[1:]) != (n, H):
+        raise KernelError(f"add_rmsnorm.parts: shape {tuple(parts.shape)}, kernel needs [S, {n}, {H}]")
+    _req(w, "add_rmsnorm.w", torch.float32, (H,))
+    _req(out, "add_rmsnorm.out", None, (n, H))
+    _check(lib().tl_add_rmsnorm(_p(x), _p(parts), parts.shape[0], _p(w), ctypes.c_float(eps), _p(out),
+                                _code(out.dtype), n, H, _stream()))
+
+
+def add_partials(x: torch.Tensor, parts: torch.Tensor) -> None:
+    """x += parts[0] + parts[1] + ... (float32 [S, n, H])."""
+    n, H = x.shape
+    _req(x, "add_partials.x", torch.float32)
+    _req(parts, "add_partials.parts", torch.float32)
+    if parts.dim() != 3 or tuple(parts.shape[1:]) != (n, H):
+        raise KernelError(f"add_partials.parts: shape {tuple(parts.shape)}, kernel needs [S, {n}, {H}]")
+    _check(lib().tl_add_partials(_p(x), _p(parts), parts.shape[0], n, H, _stream()))
+
+
 def bf16_gemm_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
     return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.shape[1] % 8 == 0
             and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
@@ -248,9 +303,11 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
 def rope_commit(qkv: torch.Tensor, row_pos, inv_freq, table, ring_pages: int, nq: int, nkv: int, d: int,
                 q: torch.Tensor, pages: torch.Tensor) -> None:
     """Single-token steps: rotate q and k, write q [n,nq,d] and put k and v of
-    row n straight into sequence n's page for its position."""
-    n = qkv.shape[0]
-    _req(qkv, "rope.qkv", torch.float32, (n, (nq + 2 * nkv) * d))
+    row n straight into sequence n's page for its position.  qkv may be
+    [S, n, width]: partial products that are added up on the way in."""
+    n_parts = qkv.shape[0] if qkv.dim() == 3 else 1
+    n = qkv.shape[-2]
+    _req(qkv, "rope.qkv", torch.float32, ((n_parts,) if qkv.dim() == 3 else ()) + (n, (nq + 2 * nkv) * d))
     _req(row_pos, "rope.row_pos", torch.int32, (n,))
     _req(inv_freq, "rope.inv_freq", torch.float32, (d // 2,))
     _req(q, "rope.q", pages.dtype, (n, nq, d))
@@ -260,7 +317,7 @@ def rope_commit(qkv: torch.Tensor, row_pos, inv_freq, table, ring_pages: int, nq
         raise KernelError(f"rope.pages: shape {tuple(pages.shape)}, kernel needs [*, 2, {nkv}, 64, {d}]")
     if table.dim() != 2 or table.shape[0] != n:
         raise KernelError("rope.table: needs one row per sequence")
-    _check(lib().tl_rope_commit(_p(qkv), _p(row_pos), _p(inv_freq), _p(table), table.shape[1], ring_pages,
+    _check(lib().tl_rope_commit(_p(qkv), n_parts, _p(row_pos), _p(inv_freq), _p(table), table.shape[1], ring_pages,
                                 n, nq, nkv, d, _p(q), _p(pages), _code(q.dtype), _stream()))
 
 

@@ -166,6 +166,14 @@ class RunBinding:
     state: Optional[torch.Tensor] = None      # [max_slots, *shape]
 
 
+def flush_pending(ctx: "StepContext", x: torch.Tensor) -> None:
+    """Add partial products that a part left in `ctx.pending` to the stream."""
+    if ctx.pending is not None:
+        from ..kernels import ops
+        ops.add_partials(x, ctx.pending)
+        ctx.pending = None
+
+
 class Workspace:
     """Scratch tensors by name, kept between steps so that a step allocates
     nothing once sizes have been seen (and a captured graph keeps its
@@ -216,4 +224,8 @@ class StepContext:
     max_len_after: int
     workspace: Workspace
     cache: Any
+    # partial products [S, n, H] (float32) that still have to be added to the residual stream:
+    # a product may leave them here instead of adding them itself; whoever reads the stream
+    # next (a norm that can, else `flush`) adds them up
+    pending: Optional[torch.Tensor] = None
     host: Dict[str, Any] = field(default_factory=dict)     # the same data on the host

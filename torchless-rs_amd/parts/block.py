@@ -8,7 +8,7 @@ from typing import Dict
 import torch
 
 from ..weights.binding import WeightSpec
-from .base import LayerSpec, Part, make_part, register_part
+from .base import LayerSpec, Part, flush_pending, make_part, register_part
 
 
 class PreNormBlock(Part):
@@ -41,10 +41,18 @@ class PreNormBlock(Part):
 
     def forward(self, ctx, run, x: torch.Tensor) -> None:
         y = ctx.workspace.get("block_y", tuple(x.shape), ctx.dtype)
-        self.mixer_norm.forward(ctx, x, y)
+        self._norm(self.mixer_norm, ctx, x, y)
         self.mixer.forward(ctx, run, y, x)
-        self.ffn_norm.forward(ctx, x, y)
+        self._norm(self.ffn_norm, ctx, x, y)
         self.ffn.forward(ctx, y, x)
+
+    @staticmethod
+    def _norm(norm, ctx, x, y) -> None:
+        """A norm reads the stream: partial products that a part left pending are
+        added first, by the norm itself if it can (`takes_pending`)."""
+        if not getattr(norm, "takes_pending", False):
+            flush_pending(ctx, x)
+        norm.forward(ctx, x, y)
 
 
 register_part("block", "pre_norm", PreNormBlock)

@@ -45,13 +45,15 @@ class SwiGLU(FeedForward):
     def forward(self, ctx, y: torch.Tensor, x: torch.Tensor) -> None:
         n = y.shape[0]
         h = ctx.workspace.get("ffn_h", (n, self.I), ctx.dtype)
-        if self.paired and ops.bf16_gemm_ok(y, self.gate_up.weight):
+        if self.paired and self.gate_up.mid(y):
+            ops.gemm_mid_bf16(y, self.gate_up.weight, h, 1, silu_pair=True)
+        elif self.paired and ops.bf16_gemm_ok(y, self.gate_up.weight):
             ops.gemm_bf16(y, self.gate_up.weight, h, silu_pair=True)
         else:
             gu = ctx.workspace.get("ffn_gu", (n, 2 * self.I), torch.float32)
             self.gate_up(y, gu)
             ops.silu_mul(gu, h)
-        self.down(h, x, accumulate=True)
+        self.down.add_into(h, x, ctx, "ffn_down_parts")
 
 
 register_part("ffn", "swiglu", SwiGLU)

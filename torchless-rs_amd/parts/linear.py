@@ -19,7 +19,36 @@ class Linear:
 
     def __call__(self, a: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
         """out[M, N] (+)= a[M, K] @ W^T; out is float32."""
-        ops.gemm(a, self.weight, out, accumulate)
+        if self.mid(a):
+            ops.gemm_mid_bf16(a, self.weight, out, 1, accumulate)
+        else:
+            ops.gemm(a, self.weight, out, accumulate)
+
+    def mid(self, a: torch.Tensor) -> bool:
+        """17..64 rows of bfloat16: the kernel that shares the activations."""
+        return 16 < a.shape[0] <= 64 and ops.bf16_gemm_ok(a, self.weight)
+
+    def partial(self, a: torch.Tensor, ctx, name: str):
+        """The product as partial sums [S, M, N] (float32) for a reader that adds
+        them up, where that pays (17..64 rows and K worth cutting); else None."""
+        if not self.mid(a):
+            return None
+        S = ops.mid_splits(a.shape[0], self.out_features, self.in_features)
+        if S == 1:
+            return None
+        parts = ctx.workspace.get(name, (S, a.shape[0], self.out_features), torch.float32)
+        ops.gemm_mid_bf16(a, self.weight, parts, S)
+        return parts
+
+    def add_into(self, a: torch.Tensor, x: torch.Tensor, ctx, name: str) -> None:
+        """x += a @ W^T, now or as partial sums left in `ctx.pending`."""
+        from .base import flush_pending
+        flush_pending(ctx, x)
+        parts = self.partial(a, ctx, name)
+        if parts is None:
+            self(a, x, accumulate=True)
+        else:
+            ctx.pending = parts
 
 
 def interleave_pairs(gate: torch.Tensor, up: torch.Tensor, block: int = 32) -> torch.Tensor:

@@ -13,6 +13,7 @@ from .base import Norm, register_part
 
 class RMSNorm(Norm):
     graph_safe = True
+    takes_pending = True        # adds partial products left in ctx.pending while it reads the stream
 
     def __init__(self, size: int, eps: float):
         self.size = int(size)
@@ -26,6 +27,15 @@ class RMSNorm(Norm):
         self.weight = tensors["weight"].to(torch.float32).contiguous()
 
     def forward(self, ctx, x: torch.Tensor, out: torch.Tensor) -> None:
+        """Partial products waiting in `ctx.pending` are added to x on the way."""
+        pend = getattr(ctx, "pending", None)
+        if pend is not None and self.size % 4 == 0 and self.size <= 8192:
+            ops.add_rmsnorm(x, pend, self.weight, self.eps, out)
+            ctx.pending = None
+            return
+        if pend is not None:
+            ops.add_partials(x, pend)
+            ctx.pending = None
         ops.rmsnorm(x, self.weight, self.eps, out)
 
 
