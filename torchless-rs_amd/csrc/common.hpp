@@ -68,8 +68,10 @@ template <int NT> __device__ __forceinline__ float block_max(float v, float* sh)
 // multiply-add), so that every kernel that rotates gives the same bits:
 // a' = a c - b s ; b' = a s + b c   (src/kernels/mod.rs:603-605 of the reference)
 __device__ __forceinline__ void rotate_pair(float a, float b, float c, float s, float& ra, float& rb) {
-  ra = __fsub_rn(__fmul_rn(a, c), __fmul_rn(b, s));
-  rb = __fadd_rn(__fmul_rn(a, s), __fmul_rn(b, c));
+#pragma clang fp contract(off)
+  const float ac = a * c, bs = b * s, as = a * s, bc = b * c;
+  ra = ac - bs;
+  rb = as + bc;
 }
 
 // ---- error channel -------------------------------------------------------

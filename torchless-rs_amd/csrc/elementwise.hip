@@ -99,6 +99,7 @@ add_rmsnorm_reg_kernel(float* __restrict__ x, const float* __restrict__ parts, i
     const int c = threadIdx.x + 256 * i;
     if (c < nv) {
       float4 a = xr[c];
+#pragma unroll 4
       for (int s = 0; s < n_parts; ++s) {
         const float4 p = reinterpret_cast<const float4*>(parts + s * part_stride + (size_t)n * H)[c];
         a.x += p.x; a.y += p.y; a.z += p.z; a.w += p.w;
@@ -151,8 +152,7 @@ __global__ void rope_split_kernel(const float* __restrict__ qkv, const int* __re
   const float pos = (float)row_pos[n];
   for (int i = threadIdx.x; i < half; i += blockDim.x) {     // the row's angles, once
     const float ang = inv_freq[i] * pos;
-    cs[i] = cosf(ang);
-    sn[i] = sinf(ang);
+    sincosf(ang, &sn[i], &cs[i]);          // one routine for both, the same in every kernel that rotates
   }
   __syncthreads();
   const float* src = qkv + (size_t)n * (nq + 2 * nkv) * d;
@@ -215,6 +215,8 @@ __global__ void rope_commit_kernel(const float* __restrict__ qkv, int n_parts, s
                                    const float* __restrict__ inv_freq, const int* __restrict__ table,
                                    int table_stride, int ring_pages, int nq, int nkv, int d,
                                    T* __restrict__ q, T* __restrict__ pages) {
+  // blockIdx.y of gridDim.y takes its share of the (q and k) heads and of the values
+  __shared__ float cs[ROPE_MAX_HALF], sn[ROPE_MAX_HALF];
   const int n = blockIdx.x;
   const int half = d / 2;
   const int p = row_pos[n];
@@ -224,18 +226,18 @@ __global__ void rope_commit_kernel(const float* __restrict__ qkv, int n_parts, s
   const int r = p % PAGE;
   T* kd = pages + (size_t)page * 2 * nkv * PAGE * d;
   T* vd = kd + (size_t)nkv * PAGE * d;
-  __shared__ float cs[ROPE_MAX_HALF], sn[ROPE_MAX_HALF];
   for (int i = threadIdx.x; i < half; i += blockDim.x) {
     const float ang = inv_freq[i] * pos;
-    cs[i] = cosf(ang);
-    sn[i] = sinf(ang);
+    sincosf(ang, &sn[i], &cs[i]);          // one routine for both, the same in every kernel that rotates
   }
   __syncthreads();
-  const int n_rot = (nq + nkv) * half;
-  for (int t = threadIdx.x; t < n_rot; t += blockDim.x) {
+  const int heads = nq + nkv;
+  const int h_lo = (int)((long long)heads * blockIdx.y / gridDim.y), h_hi = (int)((long long)heads * (blockIdx.y + 1) / gridDim.y);
+  for (int t = h_lo * half + threadIdx.x; t < h_hi * half; t += blockDim.x) {
     const int h = t / half, i = t % half;
     const float c = cs[i], s = sn[i];
     float a = src[h * d + i], b = src[h * d + i + half];
+#pragma unroll 4
     for (int sp = 1; sp < n_parts; ++sp) {
       a += src[sp * part_stride + h * d + i];
       b += src[sp * part_stride + h * d + i + half];
@@ -247,8 +249,10 @@ __global__ void rope_commit_kernel(const float* __restrict__ qkv, int n_parts, s
     dst[i + half] = from_f32<T>(rb);
   }
   const float* vs = src + (size_t)(nq + nkv) * d;
-  for (int t = threadIdx.x; t < nkv * d; t += blockDim.x) {
+  const int v_lo = (int)((long long)nkv * d * blockIdx.y / gridDim.y), v_hi = (int)((long long)nkv * d * (blockIdx.y + 1) / gridDim.y);
+  for (int t = v_lo + threadIdx.x; t < v_hi; t += blockDim.x) {
     float a = vs[t];
+#pragma unroll 4
     for (int sp = 1; sp < n_parts; ++sp) a += vs[sp * part_stride + t];
     vd[(size_t)t * PAGE + r] = from_f32<T>(a);
   }
@@ -410,11 +414,12 @@ int tl_rope_commit(const float* qkv, int n_parts, const int* row_pos, const floa
   TL_REQUIRE(n_parts >= 1, "rope_commit: n_parts=%d", n_parts);
   if (n == 0) return 0;
   const size_t stride = (size_t)n * (nq + 2 * nkv) * d;
+  const dim3 grid(n, n >= 128 ? 1 : (n >= 32 ? 4 : 8));       // few rows: cut the heads over more workgroups
   if (dt == DT_F32)
-    rope_commit_kernel<float><<<n, 256, 0, st>>>(qkv, n_parts, stride, row_pos, inv_freq, table, table_stride,
+    rope_commit_kernel<float><<<grid, 256, 0, st>>>(qkv, n_parts, stride, row_pos, inv_freq, table, table_stride,
                                                   ring_pages, nq, nkv, d, (float*)q, (float*)pages);
   else if (dt == DT_BF16)
-    rope_commit_kernel<bf16><<<n, 256, 0, st>>>(qkv, n_parts, stride, row_pos, inv_freq, table, table_stride,
+    rope_commit_kernel<bf16><<<grid, 256, 0, st>>>(qkv, n_parts, stride, row_pos, inv_freq, table, table_stride,
                                                  ring_pages, nq, nkv, d, (bf16*)q, (bf16*)pages);
   else
     TL_REQUIRE(false, "rope_commit: unknown dtype code %d", dt);
