@@ -321,3 +321,176 @@ def test_a_toy_mixer_with_state_registers_builds_and_steps():
     finally:
         unregister_part("mixer", "running_sum")
         unregister_architecture("ToyForCausalLM")
+
+
+# ---- toy parts of other kinds, registered from here ---------------------------------------
+
+def _toy_model(spec_layers, H, V, eps=1e-5):
+    from torchless_rs_amd.parts import ModelSpec, PartSpec, Run
+    norm = PartSpec("rmsnorm", {"size": H, "eps": eps})
+    return ModelSpec(hidden_size=H, vocab_size=V,
+                     embedding=PartSpec("tokens", {"vocab_size": V, "hidden_size": H}), embedding_prefix="model.",
+                     layers=spec_layers, schedule=[Run(i) for i in range(len(spec_layers))],
+                     final_norm=norm, final_norm_prefix="model.norm.",
+                     head=PartSpec("linear", {"vocab_size": V, "hidden_size": H}), head_prefix="lm_head.")
+
+
+def test_a_toy_feed_forward_with_routing():
+    """Two experts, each row goes to the one its router prefers (top-1, weight 1): a feed-forward
+    with a dispatch stage of its own, built on the framework's products.  It decides on the host,
+    so it is not `graph_safe` and its steps are never captured."""
+    from torchless_rs_amd.engine import Engine, SeqInput
+    from torchless_rs_amd.engine.model import Model
+    from torchless_rs_amd.kernels import ops
+    from torchless_rs_amd.parts import FeedForward, LayerSpec, PartSpec, register_part, unregister_part
+    from torchless_rs_amd.weights import TensorDict, WeightSpec, random_tensors
+    H, V, I, E, nq, nkv, d = 48, 60, 64, 2, 3, 1, 16
+
+    class Top1Experts(FeedForward):
+        def __init__(self, hidden_size, inner, experts):
+            self.H, self.I, self.E = hidden_size, inner, experts
+
+        def weight_specs(self):
+            out = {"moe.router.weight": WeightSpec((self.E, self.H))}
+            for e in range(self.E):
+                out[f"moe.experts.{e}.gate_up.weight"] = WeightSpec((2 * self.I, self.H))
+                out[f"moe.experts.{e}.down.weight"] = WeightSpec((self.H, self.I))
+            return out
+
+        def load(self, tensors, compute_dtype):
+            self.t = tensors
+
+        def forward(self, ctx, y, x):
+            n = y.shape[0]
+            logits = torch.empty(n, self.E, device=y.device)
+            ops.gemm(y, self.t["moe.router.weight"], logits)
+            choice = logits.argmax(-1)
+            for e in range(self.E):
+                rows = (choice == e).nonzero().flatten()
+                if not rows.numel():
+                    continue
+                ye = y[rows].contiguous()
+                gu = torch.empty(rows.numel(), 2 * self.I, device=y.device)
+                ops.gemm(ye, self.t[f"moe.experts.{e}.gate_up.weight"], gu)
+                h = torch.empty(rows.numel(), self.I, dtype=y.dtype, device=y.device)
+                ops.silu_mul(gu, h)
+                out = torch.empty(rows.numel(), self.H, device=y.device)
+                ops.gemm(h, self.t[f"moe.experts.{e}.down.weight"], out)
+                x[rows] += out
+
+    register_part("ffn", "top1_experts", Top1Experts)
+    try:
+        norm = PartSpec("rmsnorm", {"size": H, "eps": 1e-5})
+        layers = [LayerSpec(prefix=f"model.layers.{i}.",
+                            mixer=PartSpec("attention", {"hidden_size": H, "n_heads": nq, "n_kv_heads": nkv, "head_dim": d,
+                                                         "window": None, "position": PartSpec("rotary", {"head_dim": d, "theta": 100.0})}),
+                            ffn=PartSpec("top1_experts", {"hidden_size": H, "inner": I, "experts": E}),
+                            mixer_norm=norm, ffn_norm=norm) for i in range(2)]
+        spec = _toy_model(layers, H, V)
+        w = random_tensors(spec.weight_specs(), seed=4, std=0.2, dtype=torch.float32)
+        model = Model(spec, None, torch.float32, DEV)
+        model.load_weights(TensorDict(w))
+        assert not model.graph_safe
+        eng = Engine(model, max_tokens=256)
+
+        def plain_forward(ids):
+            wd = {k: v.double() for k, v in w.items()}
+            T = len(ids)
+            pos = torch.arange(T)
+            cfg = {"num_attention_heads": nq, "num_key_value_heads": nkv, "head_dim": d, "hidden_size": H, "rope_theta": 100.0}
+            x = wd["model.embed_tokens.weight"][ids]
+            for i in range(2):
+                p = f"model.layers.{i}."
+                x = x + plain.attention(plain.rmsnorm(x, wd[p + "input_layernorm.weight"], 1e-5), wd, p, cfg, pos)
+                y = plain.rmsnorm(x, wd[p + "post_attention_layernorm.weight"], 1e-5)
+                choice = (y @ wd[p + "moe.router.weight"].t()).argmax(-1)
+                add = torch.zeros_like(x)
+                for t in range(T):
+                    e = int(choice[t])
+                    gu = wd[p + f"moe.experts.{e}.gate_up.weight"] @ y[t]
+                    add[t] = wd[p + f"moe.experts.{e}.down.weight"] @ (plain.silu(gu[:I]) * gu[I:])
+                x = x + add
+            return plain.rmsnorm(x, wd["model.norm.weight"], 1e-5) @ wd["lm_head.weight"].t()
+
+        g = torch.Generator().manual_seed(3)
+        ids = torch.randint(0, V, (30,), generator=g).tolist()
+        want = plain_forward(ids)
+        s = eng.alloc()
+        outs = [eng.step([SeqInput(s, ids[:20], list(range(20)))]).clone()]
+        outs += [eng.step([SeqInput(s, [t], [0])]).clone() for t in ids[20:]]
+        eng.free(s)
+        assert not eng._graphs
+        assert rel_err(torch.cat(outs), want) < 1e-5
+    finally:
+        unregister_part("ffn", "top1_experts")
+
+
+def test_a_toy_position_encoding():
+    """Rotation with every frequency divided by a factor (positions stretched): another position
+    encoding, a part of its own kind that the attention mixer takes by name."""
+    from torchless_rs_amd.engine import Engine, SeqInput
+    from torchless_rs_amd.engine.model import Model
+    from torchless_rs_amd.parts import LayerSpec, PartSpec, register_part, unregister_part
+    from torchless_rs_amd.parts.position import Rotary
+    from torchless_rs_amd.weights import TensorDict, random_tensors
+    H, V, I, nq, nkv, d, factor = 40, 50, 56, 5, 5, 8, 4.0
+
+    class StretchedRotary(Rotary):
+        def __init__(self, head_dim, theta, factor):
+            super().__init__(head_dim, theta)
+            self.factor = factor
+
+        def inv_freq_host(self):
+            return super().inv_freq_host() / self.factor
+
+    register_part("position", "stretched_rotary", StretchedRotary)
+    try:
+        norm = PartSpec("rmsnorm", {"size": H, "eps": 1e-5})
+        pos_spec = PartSpec("stretched_rotary", {"head_dim": d, "theta": 50.0, "factor": factor})
+        layers = [LayerSpec(prefix="model.layers.0.",
+                            mixer=PartSpec("attention", {"hidden_size": H, "n_heads": nq, "n_kv_heads": nkv, "head_dim": d,
+                                                         "window": 5, "position": pos_spec}),
+                            ffn=PartSpec("swiglu", {"hidden_size": H, "intermediate_size": I}),
+                            mixer_norm=norm, ffn_norm=norm)]
+        spec = _toy_model(layers, H, V)
+        w = random_tensors(spec.weight_specs(), seed=6, std=0.3, dtype=torch.float32)
+        model = Model(spec, None, torch.float32, DEV)
+        model.load_weights(TensorDict(w))
+        eng = Engine(model, max_tokens=128)
+
+        def stretched(x, positions):
+            # plain.rope at positions / factor is the same angle
+            half = d // 2
+            inv = plain.rope_inv_freq(d, 50.0, x.dtype) / factor
+            ang = positions.to(x.dtype)[:, None] * inv[None, :]
+            c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+            a, b = x[..., :half], x[..., half:]
+            return torch.cat([a * c - b * s, a * s + b * c], -1)
+
+        def plain_forward(ids):
+            wd = {k: v.double() for k, v in w.items()}
+            T, p = len(ids), "model.layers.0."
+            pos = torch.arange(T)
+            x = wd["model.embed_tokens.weight"][ids]
+            y = plain.rmsnorm(x, wd[p + "input_layernorm.weight"], 1e-5)
+            q = stretched(plain.linear(y, wd[p + "self_attn.q_proj.weight"]).view(T, nq, d), pos)
+            k = stretched(plain.linear(y, wd[p + "self_attn.k_proj.weight"]).view(T, nkv, d), pos)
+            v = plain.linear(y, wd[p + "self_attn.v_proj.weight"]).view(T, nkv, d)
+            a = plain.attention_core(q, k, v, pos, 5).reshape(T, nq * d)
+            x = x + plain.linear(a, wd[p + "self_attn.o_proj.weight"])
+            x = x + plain.swiglu(plain.rmsnorm(x, wd[p + "post_attention_layernorm.weight"], 1e-5), wd, p)
+            return plain.rmsnorm(x, wd["model.norm.weight"], 1e-5) @ wd["lm_head.weight"].t()
+
+        g = torch.Generator().manual_seed(7)
+        ids = torch.randint(0, V, (24,), generator=g).tolist()
+        want = plain_forward(ids)
+        s = eng.alloc()
+        outs = [eng.step([SeqInput(s, ids[:9], list(range(9)))]).clone()]
+        outs += [eng.step([SeqInput(s, [t], [0])]).clone() for t in ids[9:]]
+        eng.free(s)
+        assert rel_err(torch.cat(outs), want) < 1e-5
+        assert rel_err(torch.cat(outs), plain.forward({**w}, {"num_hidden_layers": 1, "hidden_size": H, "num_attention_heads": nq,
+                       "num_key_value_heads": nkv, "head_dim": d, "rope_theta": 50.0, "sliding_window": 5,
+                       "rms_norm_eps": 1e-5}, ids)) > 1e-3           # and it is not the plain rotation
+    finally:
+        unregister_part("position", "stretched_rotary")

@@ -336,19 +336,28 @@ gemm_tiled_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float*
     stash();
     __syncthreads();
     if (k0 + TK < K) fetch(k0 + TK);
+    // operands of the next 16 k are read from LDS while the MFMAs of these 16 run
+    bf16x8 a[2][2], b[2][2];
 #pragma unroll
-    for (int kk = 0; kk < TK; kk += 16) {
-      bf16x8 a[2], b[2];
+    for (int i = 0; i < 2; ++i) {
+      a[0][i] = *reinterpret_cast<const bf16x8*>(&As[(wm + 32 * i + l32) * TLD + 8 * kh]);
+      b[0][i] = *reinterpret_cast<const bf16x8*>(&Ws[(wn + 32 * i + l32) * TLD + 8 * kh]);
+    }
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        a[i] = *reinterpret_cast<const bf16x8*>(&As[(wm + 32 * i + l32) * TLD + kk + 8 * kh]);
-        b[i] = *reinterpret_cast<const bf16x8*>(&Ws[(wn + 32 * i + l32) * TLD + kk + 8 * kh]);
+    for (int ks = 0; ks < TK / 16; ++ks) {
+      const int cur = ks & 1, nxt = cur ^ 1;
+      if (ks + 1 < TK / 16) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          a[nxt][i] = *reinterpret_cast<const bf16x8*>(&As[(wm + 32 * i + l32) * TLD + (ks + 1) * 16 + 8 * kh]);
+          b[nxt][i] = *reinterpret_cast<const bf16x8*>(&Ws[(wn + 32 * i + l32) * TLD + (ks + 1) * 16 + 8 * kh]);
+        }
       }
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[cur][i], b[cur][j], acc[i][j], 0, 0, 0);
     }
   }
   // acc[i][j][r]: row = 8*(r/4) + 4*kh + r%4, column = l32 of the 32x32 block
@@ -452,20 +461,27 @@ gemm_big_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float* _
     stash(0);
     __syncthreads();
     if (kt + 1 < nk) fetch((kt + 1) * GK);
+    bf16x8 a[2][4], b[2][2];
 #pragma unroll
-    for (int kk = 0; kk < GK; kk += 16) {
-      bf16x8 a[4], b[2];
+    for (int i = 0; i < 4; ++i) a[0][i] = *reinterpret_cast<const bf16x8*>(&As[(wm + 32 * i + l32) * GLD + 8 * kh]);
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        a[i] = *reinterpret_cast<const bf16x8*>(&As[(wm + 32 * i + l32) * GLD + kk + 8 * kh]);
+    for (int j = 0; j < 2; ++j) b[0][j] = *reinterpret_cast<const bf16x8*>(&Ws[(wn + 32 * j + l32) * GLD + 8 * kh]);
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
-        b[j] = *reinterpret_cast<const bf16x8*>(&Ws[(wn + 32 * j + l32) * GLD + kk + 8 * kh]);
+    for (int ks = 0; ks < GK / 16; ++ks) {
+      const int cur = ks & 1, nxt = cur ^ 1;
+      if (ks + 1 < GK / 16) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          a[nxt][i] = *reinterpret_cast<const bf16x8*>(&As[(wm + 32 * i + l32) * GLD + (ks + 1) * 16 + 8 * kh]);
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          b[nxt][j] = *reinterpret_cast<const bf16x8*>(&Ws[(wn + 32 * j + l32) * GLD + (ks + 1) * 16 + 8 * kh]);
+      }
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[cur][i], b[cur][j], acc[i][j], 0, 0, 0);
     }
   }
   if (epilogue == EPI_SILU_PAIR) {
