@@ -487,6 +487,45 @@ def test_gemm_bf16_paired_silu_epilogue(ops, variant, M, I, K):
     assert rel_err(out2, want) < KTOL["bfloat16"]
 
 
+@pytest.mark.parametrize("M,N,K", [(129, 50, 72), (300, 130, 264), (200, 384, 96)])
+def test_gemm_library_products(ops, M, N, K):
+    """Above LIBRARY_ROWS rows the dispatcher hands the product to the BLAS library:
+    float32 out (stored or accumulated) and bfloat16 out (stored)."""
+    a = rnd(M, K, seed=41, dtype=torch.bfloat16)
+    w = rnd(N, K, seed=42, dtype=torch.bfloat16)
+    want = a.double() @ w.double().t()
+    assert M > ops.LIBRARY_ROWS
+    out = torch.full((M, N), float("nan"), device=DEV)
+    ops.gemm(a.to(DEV), w.to(DEV), out)
+    assert rel_err(out, want) < 3e-6
+    base = rnd(M, N, seed=43)
+    acc = base.clone().to(DEV)
+    ops.gemm(a.to(DEV), w.to(DEV), acc, accumulate=True)
+    assert rel_err(acc, want + base.double()) < 3e-6
+    ours = torch.empty(M, N, device=DEV)
+    ops.gemm_bf16(a.to(DEV), w.to(DEV), ours)
+    assert rel_err(ours, out) < 1e-6                         # our kernel agrees up to rounding
+    o16 = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    ops.gemm_library(a.to(DEV), w.to(DEV), o16)
+    assert rel_err(o16, want) < KTOL["bfloat16"]
+    with pytest.raises(ops.KernelError, match="accumulate"):
+        ops.gemm_library(a.to(DEV), w.to(DEV), o16, accumulate=True)
+
+
+@pytest.mark.parametrize("n,I", [(1, 32), (5, 96), (131, 480)])
+def test_silu_mul_pairs(ops, n, I):
+    from torchless_rs_amd.parts.linear import interleave_pairs
+    g = rnd(I, n, seed=44, dtype=torch.bfloat16, scale=3.0)
+    u = rnd(I, n, seed=45, dtype=torch.bfloat16, scale=3.0)
+    gu = interleave_pairs(g, u).t().contiguous()            # [n, 2I], columns in groups of 64
+    out = torch.full((n, I), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.silu_mul_pairs(gu.to(DEV), out)
+    assert rel_err(out, (plain.silu(g.double()) * u.double()).t()) < KTOL["bfloat16"]
+    with pytest.raises(ops.KernelError, match="steps of 32"):
+        ops.silu_mul_pairs(torch.zeros(2, 80, dtype=torch.bfloat16, device=DEV),
+                           torch.zeros(2, 40, dtype=torch.bfloat16, device=DEV))
+
+
 @pytest.mark.parametrize("dt", ["float32", "bfloat16"])
 @pytest.mark.parametrize("window", [None, 70])
 def test_rope_commit_equals_rope_split_then_commit(ops, dt, window):

@@ -270,6 +270,27 @@ __global__ void silu_mul_kernel(const float* __restrict__ gu, int I, TO* __restr
   }
 }
 
+// gu[n, 2I] in bfloat16 with columns in groups of 64 (32 of gate, then the 32 of up
+// that belong to them); out[n, I] = silu(gate) * up.  A thread takes 8 pairs.
+__global__ void silu_mul_pairs_kernel(const bf16* __restrict__ gu, long long chunks, int I,
+                                      bf16* __restrict__ out) {
+  const long long c = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= chunks) return;
+  const int per_row = I / 8;
+  const long long n = c / per_row;
+  const int i = (int)(c % per_row), group = i / 4, part = i % 4;
+  const bf16* src = gu + n * 2 * I + group * 64 + part * 8;
+  const bf16x8 g = *reinterpret_cast<const bf16x8*>(src);
+  const bf16x8 u = *reinterpret_cast<const bf16x8*>(src + 32);
+  bf16x8 o;
+#pragma unroll
+  for (int t = 0; t < 8; ++t) {
+    const float gv = (float)g[t];
+    o[t] = (bf16)((gv / (1.0f + expf(-gv))) * (float)u[t]);
+  }
+  *reinterpret_cast<bf16x8*>(out + n * I + group * 32 + part * 8) = o;
+}
+
 __global__ void gather_rows_kernel(const float* __restrict__ x, const int* __restrict__ idx, int H,
                                    float* __restrict__ out) {
   const int m = blockIdx.x;
@@ -438,6 +459,17 @@ int tl_silu_mul(const float* gu, int n, int I, void* out, int out_dt, hipStream_
   else
     TL_REQUIRE(false, "silu_mul: unknown dtype code %d", out_dt);
   TL_LAUNCH_CHECK("silu_mul");
+  return 0;
+}
+
+int tl_silu_mul_pairs(const void* gu, int n, int I, void* out, hipStream_t st) {
+  TL_REQUIRE(n >= 0 && I > 0 && I % 32 == 0, "silu_mul_pairs: bad sizes n=%d I=%d (I in steps of 32)", n, I);
+  TL_REQUIRE((uintptr_t)gu % 16 == 0 && (uintptr_t)out % 16 == 0, "silu_mul_pairs: buffers must be 16-byte aligned");
+  if (n == 0) return 0;
+  const long long chunks = (long long)n * (I / 8);
+  TL_REQUIRE((chunks + 255) / 256 < 2147483647LL, "silu_mul_pairs: too many elements");
+  silu_mul_pairs_kernel<<<(unsigned)((chunks + 255) / 256), 256, 0, st>>>((const bf16*)gu, chunks, I, (bf16*)out);
+  TL_LAUNCH_CHECK("silu_mul_pairs");
   return 0;
 }
 

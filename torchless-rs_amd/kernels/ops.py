@@ -169,6 +169,15 @@ def silu_mul(gu: torch.Tensor, out: torch.Tensor) -> None:
     _check(lib().tl_silu_mul(_p(gu), n, I2 // 2, _p(out), _code(out.dtype), _stream()))
 
 
+def silu_mul_pairs(gu: torch.Tensor, out: torch.Tensor) -> None:
+    """The same on bfloat16 gu whose columns come in groups of 64: 32 of gate,
+    then the 32 of up that belong to them (`interleave_pairs`)."""
+    n, I2 = gu.shape
+    _req(gu, "silu_mul_pairs.gu", torch.bfloat16)
+    _req(out, "silu_mul_pairs.out", torch.bfloat16, (n, I2 // 2))
+    _check(lib().tl_silu_mul_pairs(_p(gu), n, I2 // 2, _p(out), _stream()))
+
+
 def gather_rows(x: torch.Tensor, idx: torch.Tensor, out: torch.Tensor) -> None:
     m, H = idx.shape[0], x.shape[1]
     _req(x, "gather.x", torch.float32)
@@ -285,6 +294,30 @@ def add_partials(x: torch.Tensor, parts: torch.Tensor) -> None:
     _check(lib().tl_add_partials(_p(x), _p(parts), parts.shape[0], n, H, _stream()))
 
 
+LIBRARY_ROWS = 128          # above this many rows the library's product beats ours
+
+
+def gemm_library(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
+    """out[M,N] (+)= a[M,K] @ w[N,K]^T through the BLAS library (hipBLASLt below
+    torch): bfloat16 operands, float32 accumulation; out is float32, or bfloat16
+    when it is only stored.  The reference hands its products to the vendor's
+    library likewise (src/kernels/cuda/mod.rs:462-552, src/kernels/rocm/mod.rs)."""
+    M, K = a.shape
+    N = w.shape[0]
+    _req(a, "gemm.a", torch.bfloat16)
+    _req(w, "gemm.w", torch.bfloat16, (N, K))
+    _req(out, "gemm.out", None, (M, N))
+    if out.dtype == torch.float32:
+        if accumulate:
+            torch.addmm(out, a, w.t(), out_dtype=torch.float32, out=out)
+        else:
+            torch.mm(a, w.t(), out_dtype=torch.float32, out=out)
+    elif out.dtype == torch.bfloat16 and not accumulate:
+        torch.mm(a, w.t(), out=out)
+    else:
+        raise KernelError(f"gemm_library: cannot {'accumulate into' if accumulate else 'store'} {out.dtype}")
+
+
 def bf16_gemm_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
     return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.shape[1] % 8 == 0
             and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
@@ -293,9 +326,13 @@ def bf16_gemm_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
 def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
     """out[M,N] (+)= a[M,K] @ w[N,K]^T with float32 accumulation.  The kernel
     follows from the operand types: bfloat16 x bfloat16 goes to the matrix
-    cores, anything with float32 in it to the plain FMA kernel."""
+    cores (our kernels up to LIBRARY_ROWS rows, the library's above), anything
+    with float32 in it to the plain FMA kernel."""
     if bf16_gemm_ok(a, w):
-        gemm_bf16(a, w, out, accumulate)
+        if a.shape[0] > LIBRARY_ROWS:
+            gemm_library(a, w, out, accumulate)
+        else:
+            gemm_bf16(a, w, out, accumulate)
     else:
         gemm_plain(a, w, out, accumulate)
 

@@ -48,7 +48,12 @@ class SwiGLU(FeedForward):
         if self.paired and self.gate_up.mid(y):
             ops.gemm_mid_bf16(y, self.gate_up.weight, h, 1, silu_pair=True)
         elif self.paired and ops.bf16_gemm_ok(y, self.gate_up.weight):
-            ops.gemm_bf16(y, self.gate_up.weight, h, silu_pair=True)
+            if n > ops.LIBRARY_ROWS:
+                gu = ctx.workspace.get("ffn_gu16", (n, 2 * self.I), torch.bfloat16)
+                ops.gemm_library(y, self.gate_up.weight, gu)
+                ops.silu_mul_pairs(gu, h)
+            else:
+                ops.gemm_bf16(y, self.gate_up.weight, h, silu_pair=True)
         else:
             gu = ctx.workspace.get("ffn_gu", (n, 2 * self.I), torch.float32)
             self.gate_up(y, gu)
