@@ -547,6 +547,40 @@ def test_rope_commit_equals_rope_split_then_commit(ops, dt, window):
     assert not torch.equal(torch.nan_to_num(pages2.float(), nan=-7.0), torch.nan_to_num(a["pages"].float(), nan=-7.0))
 
 
+@pytest.mark.parametrize("nq,nkv,d,K,lens", [(6, 2, 48, 72, [0, 63, 64, 300]), (4, 4, 16, 264, [5]),
+                                             (8, 2, 128, 1000, [9, 64, 127, 128, 640, 2, 3, 4, 5, 6, 7, 8, 70, 71, 72, 73])])
+@pytest.mark.parametrize("window", [None, 70])
+def test_qkv_rope_commit_equals_product_then_rope_commit(ops, nq, nkv, d, K, lens, window):
+    """The fused kernel of single-token steps gives the bits of the product followed by rope_commit."""
+    from torchless_rs_amd.parts.position import Rotary
+    n = len(lens)
+    c = paged_case(ops, "bfloat16", nq, nkv, d, window, lens_cached=lens, lens_new=[1] * n, seed=9, n_pages=60)
+    y = rnd(n, K, seed=10, dtype=torch.bfloat16).to(DEV)
+    w = rnd((nq + 2 * nkv) * d, K, seed=11, dtype=torch.bfloat16, scale=0.2).to(DEV)
+    inv = Rotary(d, 10000.0).inv_freq(DEV)
+    qkv = torch.empty(n, (nq + 2 * nkv) * d, device=DEV)
+    ops.gemm(y, w, qkv)
+    q1 = torch.empty(n, nq, d, dtype=torch.bfloat16, device=DEV)
+    pages1 = c["pages"].clone()
+    ops.rope_commit(qkv, c["row_pos"], inv, c["table"], c["ring"], nq, nkv, d, q1, pages1)
+    q2 = torch.full_like(q1, float("nan"))
+    pages2 = c["pages"].clone()
+    assert ops.qkv_rope_commit_ok(y, w, d, pages2)
+    ops.qkv_rope_commit(y, w, c["row_pos"], inv, c["table"], c["ring"], nq, nkv, d, q2, pages2)
+    assert torch.equal(q1, q2)
+    assert torch.equal(torch.nan_to_num(pages1.float(), nan=-7.0), torch.nan_to_num(pages2.float(), nan=-7.0))
+    # and against the plain rotation of the plain product
+    full = (y.double().cpu() @ w.double().cpu().t()).view(n, nq + 2 * nkv, d)
+    pos = c["row_pos"].cpu().long()
+    want_q = plain.rope(full[:, :nq], pos, 10000.0)
+    assert rel_err(q2, want_q) < KTOL["bfloat16"]
+    assert not ops.qkv_rope_commit_ok(torch.zeros(17, K, dtype=torch.bfloat16, device=DEV), w, d, pages2)
+    with pytest.raises(ops.KernelError, match="steps of 16"):
+        ops.qkv_rope_commit(y, w[: (nq + 2 * nkv) * 8].contiguous(), c["row_pos"], inv[: 4].contiguous(), c["table"],
+                            c["ring"], nq, nkv, 8, torch.empty(n, nq, 8, dtype=torch.bfloat16, device=DEV),
+                            torch.zeros(60, 2, nkv, 64, 8, dtype=torch.bfloat16, device=DEV))
+
+
 # ---- 17..64 rows: shared activations, K cut into partial sums -----------------------------
 
 @pytest.mark.parametrize("M", [17, 32, 33, 48, 50, 64, 5])

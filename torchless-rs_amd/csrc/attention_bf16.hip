@@ -454,30 +454,50 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
 // Merge the splits of one (sequence, head): common maximum, weighted sums, in the order of the
 // splits.  (A second kernel and not the last workgroup of the first: what other XCDs wrote is
 // only sure to be seen across a kernel boundary without flushing L2 from inside the kernel.)
+// One wave per (row, head).  Splits are taken 8 at a time with all their loads (maxima, sums and
+// this lane's elements) issued together, so that a usual split count costs one trip to memory;
+// chunks merge by the running-maximum rule.
 __global__ void __launch_bounds__(64)
 attn_decode_combine_kernel(const float* __restrict__ part, int n_splits, int d, bf16* __restrict__ out) {
-  extern __shared__ float fac[];                       // [n_splits] weight of each split
+  constexpr int CH = 8, MAXV = 4;                      // d <= 256: at most 4 elements a lane
   const size_t bh = blockIdx.x;
   const float* src = part + bh * n_splits * (d + 2);
   const int lane = threadIdx.x;
-  float mm = -INFINITY;
-  for (int s = lane; s < n_splits; s += 64) mm = fmaxf(mm, src[(size_t)s * (d + 2)]);
-  mm = wave_max(mm);
-  float ll = 0.f;
-  for (int s = lane; s < n_splits; s += 64) {
-    const float ms = src[(size_t)s * (d + 2)];
-    const float f = (ms == -INFINITY) ? 0.f : __expf(ms - mm);
-    fac[s] = f;
-    ll += src[(size_t)s * (d + 2) + 1] * f;
+  const size_t stride = d + 2;
+  float mm = -INFINITY, ll = 0.f, acc[MAXV];
+#pragma unroll
+  for (int v = 0; v < MAXV; ++v) acc[v] = 0.f;
+  for (int s0 = 0; s0 < n_splits; s0 += CH) {
+    float ms[CH], ls[CH], vs[CH][MAXV];
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const bool ok = s0 + c < n_splits;
+      const float* p = src + (size_t)(ok ? s0 + c : s0) * stride;
+      ms[c] = ok ? p[0] : -INFINITY;
+      ls[c] = p[1];
+#pragma unroll
+      for (int v = 0; v < MAXV; ++v) vs[c][v] = (lane + 64 * v < d) ? p[2 + lane + 64 * v] : 0.f;
+    }
+    float mc = mm;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) mc = fmaxf(mc, ms[c]);
+    if (mc == -INFINITY) continue;                     // nothing visible so far
+    const float keep = (mm == -INFINITY) ? 0.f : __expf(mm - mc);
+    ll *= keep;
+#pragma unroll
+    for (int v = 0; v < MAXV; ++v) acc[v] *= keep;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const float f = (ms[c] == -INFINITY) ? 0.f : __expf(ms[c] - mc);
+      ll += ls[c] * f;
+#pragma unroll
+      for (int v = 0; v < MAXV; ++v) acc[v] += vs[c][v] * f;
+    }
+    mm = mc;
   }
-  ll = wave_sum(ll);
-  __syncthreads();
-  for (int dv = lane; dv < d; dv += 64) {
-    float acc = 0.f;
-#pragma unroll 4
-    for (int s = 0; s < n_splits; ++s) acc += src[(size_t)s * (d + 2) + 2 + dv] * fac[s];
-    out[bh * d + dv] = (bf16)(acc / ll);
-  }
+#pragma unroll
+  for (int v = 0; v < MAXV; ++v)
+    if (lane + 64 * v < d) out[bh * d + lane + 64 * v] = (bf16)(acc[v] / ll);
 }
 
 template <int DPAD>
@@ -517,7 +537,7 @@ static int launch_decode(const bf16* q, const bf16* pages, const int* table, int
                                                             head_groups, part, out);
   TL_LAUNCH_CHECK("attn_decode");
   if (n_splits > 1) {
-    attn_decode_combine_kernel<<<B * nq, 64, n_splits * sizeof(float), st>>>(part, n_splits, d, out);
+    attn_decode_combine_kernel<<<B * nq, 64, 0, st>>>(part, n_splits, d, out);
     TL_LAUNCH_CHECK("attn_decode_combine");
   }
   return 0;

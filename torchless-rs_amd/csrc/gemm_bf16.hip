@@ -147,6 +147,104 @@ static int launch_skinny(const bf16* A, const bf16* W, float* C, int M, int N, i
   return 0;
 }
 
+// ------------------------------------------------- q|k|v of single tokens ----
+// The skinny product (16 channels a workgroup, 8 waves over K, up to 16 rows) for the
+// fused projection of a step with one token a sequence, with what follows it done on
+// the sums while they are in LDS: rotation of q and k by the position, q to its buffer,
+// k and v into the sequence's page (v transposed).  To have both halves of a rotated
+// pair, a tile of a q or k head takes channels 8t..8t+7 and d/2+8t..d/2+8t+7; a tile of
+// a v head takes 16 in a row.  The sums and the rotation are those of the unfused
+// kernels, bit for bit (a' = a c - b s; b' = a s + b c; src/kernels/mod.rs:603-605 of
+// the reference).
+constexpr int QKV_WAVES = 8;
+
+__global__ void __launch_bounds__(QKV_WAVES * 64)
+gemm_qkv_rope_commit_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, int M, int K,
+                            const int* __restrict__ row_pos, const float* __restrict__ inv_freq,
+                            const int* __restrict__ table, int table_stride, int ring_pages, int nq,
+                            int nkv, int d, bf16* __restrict__ q, bf16* __restrict__ pages) {
+  __shared__ float red[QKV_WAVES][256];
+  __shared__ float cs[16][8], sn[16][8];
+  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+  const int li = lane % 16, kg = lane / 16;
+  const int tiles = d / 16, head = blockIdx.x / tiles, tt = blockIdx.x % tiles;
+  const int half = d / 2;
+  const bool rotated = head < nq + nkv;
+  const int ch = rotated ? (li < 8 ? 8 * tt + li : half + 8 * tt + li - 8) : 16 * tt + li;
+  const bf16* wrow = W + ((size_t)head * d + ch) * K;
+  const bf16* arow = A + (size_t)min(li, M - 1) * K;
+  const int steps = (K + 63) / 64;
+  const int per = (steps + QKV_WAVES - 1) / QKV_WAVES;
+  const int s0 = wave * per, s1 = min(steps, s0 + per);
+
+  f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+  auto load_step = [&](int s, bf16x8 (&wv)[2], bf16x8 (&av)[2]) {
+    const int k = s * 64 + kg * 16;
+    const bool ok0 = k + 8 <= K, ok1 = k + 16 <= K;
+    wv[0] = ok0 ? load8(wrow + k) : zero8();
+    wv[1] = ok1 ? load8(wrow + k + 8) : zero8();
+    av[0] = ok0 ? load8(arow + k) : zero8();
+    av[1] = ok1 ? load8(arow + k + 8) : zero8();
+  };
+  auto mma_step = [&](bf16x8 (&wv)[2], bf16x8 (&av)[2]) {
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[0], av[0], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[1], av[1], acc, 0, 0, 0);
+  };
+  bf16x8 w0[2], a0[2], w1[2], a1[2];
+  int s = s0;
+  if (s < s1) load_step(s, w0, a0);
+  if (rotated && tid < 128) {                  // while the first loads are under way
+    const int m = tid / 8, j = tid % 8;
+    if (m < M) sincosf(inv_freq[8 * tt + j] * (float)row_pos[m], &sn[m][j], &cs[m][j]);
+  }
+  for (; s + 1 < s1; s += 2) {
+    load_step(s + 1, w1, a1);
+    mma_step(w0, a0);
+    if (s + 2 < s1) load_step(s + 2, w0, a0);
+    mma_step(w1, a1);
+  }
+  if (s < s1) mma_step(w0, a0);
+#pragma unroll
+  for (int r = 0; r < 4; ++r) red[wave][r * 64 + lane] = acc[r];     // D[n = 4 kg + r][m = li]
+  __syncthreads();
+  auto total = [&](int nl, int m) {
+    const int idx = (nl % 4) * 64 + (nl / 4) * 16 + m;
+    float v = 0.f;
+#pragma unroll
+    for (int w = 0; w < QKV_WAVES; ++w) v += red[w][idx];
+    return v;
+  };
+  const size_t page_elems = 2 * (size_t)nkv * PAGE * d;
+  if (rotated) {
+    if (tid < 128) {
+      const int m = tid / 8, j = tid % 8;
+      if (m < M) {
+        float ra, rb;
+        rotate_pair(total(j, m), total(j + 8, m), cs[m][j], sn[m][j], ra, rb);
+        const int i = 8 * tt + j;
+        bf16* dst;
+        if (head < nq) {
+          dst = q + ((size_t)m * nq + head) * d;
+        } else {
+          const int p = row_pos[m];
+          const int page = table[(size_t)m * table_stride + (p / PAGE) % ring_pages];
+          dst = pages + (size_t)page * page_elems + ((size_t)(head - nq) * PAGE + p % PAGE) * d;
+        }
+        dst[i] = (bf16)ra;
+        dst[i + half] = (bf16)rb;
+      }
+    }
+  } else if (tid < 256) {
+    const int m = tid / 16, nl = tid % 16;
+    if (m < M) {
+      const int p = row_pos[m];
+      const int page = table[(size_t)m * table_stride + (p / PAGE) % ring_pages];
+      bf16* vd = pages + (size_t)page * page_elems + (size_t)nkv * PAGE * d;
+      vd[((size_t)(head - nq - nkv) * d + 16 * tt + nl) * PAGE + p % PAGE] = (bf16)total(nl, m);
+    }
+  }
+}
+
 // ------------------------------------------------------------------- mid ----
 // 17..64 rows (decode at larger batches).  Per byte of W there are now enough
 // MFMAs that the activations must be shared: a workgroup owns 64 output
@@ -633,4 +731,26 @@ extern "C" int tl_gemm_mid_bf16(const void* A, const void* W, void* C, int M, in
   if (M <= 32) return launch_mid<2>(a, w, c, M, N, K, n_split, epilogue, st);
   if (M <= 48) return launch_mid<3>(a, w, c, M, N, K, n_split, epilogue, st);
   return launch_mid<4>(a, w, c, M, N, K, n_split, epilogue, st);
+}
+
+// q|k|v of a step with one token a sequence (row m is sequence m, at position row_pos[m]):
+// W is [(nq + 2 nkv) d, K]; q receives [M, nq, d], the pages k and v of the new position.
+extern "C" int tl_gemm_qkv_rope_commit(const void* A, const void* W, int M, int K, const int* row_pos,
+                                       const float* inv_freq, const int* table, int table_stride,
+                                       int ring_pages, int nq, int nkv, int d, void* q, void* pages,
+                                       hipStream_t st) {
+  TL_REQUIRE(M >= 0 && M <= 16 && K > 0 && K % 8 == 0, "qkv_rope_commit: bad sizes M=%d K=%d (at most 16 rows, "
+             "K a multiple of 8)", M, K);
+  TL_REQUIRE(nq > 0 && nkv > 0 && d >= 16 && d % 16 == 0, "qkv_rope_commit: bad heads nq=%d nkv=%d d=%d (head "
+             "sizes in steps of 16)", nq, nkv, d);
+  TL_REQUIRE(ring_pages > 0 && table_stride > 0, "qkv_rope_commit: bad cache geometry ring_pages=%d "
+             "table_stride=%d", ring_pages, table_stride);
+  TL_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "qkv_rope_commit: operands must be 16-byte aligned");
+  if (M == 0) return 0;
+  const int grid = (nq + 2 * nkv) * (d / 16);
+  gemm_qkv_rope_commit_kernel<<<grid, QKV_WAVES * 64, 0, st>>>((const bf16*)A, (const bf16*)W, M, K, row_pos,
+                                                              inv_freq, table, table_stride, ring_pages, nq,
+                                                              nkv, d, (bf16*)q, (bf16*)pages);
+  TL_LAUNCH_CHECK("gemm_qkv_rope_commit");
+  return 0;
 }

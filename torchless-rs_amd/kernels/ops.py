@@ -358,6 +358,33 @@ def rope_commit(qkv: torch.Tensor, row_pos, inv_freq, table, ring_pages: int, nq
                                 n, nq, nkv, d, _p(q), _p(pages), _code(q.dtype), _stream()))
 
 
+def qkv_rope_commit_ok(a: torch.Tensor, w: torch.Tensor, d: int, pages: torch.Tensor) -> bool:
+    """Whether `qkv_rope_commit` serves this step: bfloat16 all through, at most 16 rows."""
+    return bf16_gemm_ok(a, w) and a.shape[0] <= 16 and d % 16 == 0 and pages.dtype == torch.bfloat16
+
+
+def qkv_rope_commit(a: torch.Tensor, w: torch.Tensor, row_pos, inv_freq, table, ring_pages: int, nq: int,
+                    nkv: int, d: int, q: torch.Tensor, pages: torch.Tensor) -> None:
+    """For a step with one token a sequence (at most 16): the product a @ w^T with w = q|k|v,
+    the rotation of q and k, q into its buffer and k, v into the pages, in one kernel; the
+    same bits as `gemm` and then `rope_commit`."""
+    n, K = a.shape
+    _req(a, "qkv_rope_commit.a", torch.bfloat16)
+    _req(w, "qkv_rope_commit.w", torch.bfloat16, ((nq + 2 * nkv) * d, K))
+    _req(row_pos, "qkv_rope_commit.row_pos", torch.int32, (n,))
+    _req(inv_freq, "qkv_rope_commit.inv_freq", torch.float32, (d // 2,))
+    _req(q, "qkv_rope_commit.q", torch.bfloat16, (n, nq, d))
+    _req(table, "qkv_rope_commit.table", torch.int32)
+    _req(pages, "qkv_rope_commit.pages", torch.bfloat16)
+    if pages.dim() != 5 or tuple(pages.shape[1:]) != (2, nkv, 64, d):
+        raise KernelError(f"qkv_rope_commit.pages: shape {tuple(pages.shape)}, kernel needs [*, 2, {nkv}, 64, {d}]")
+    if table.dim() != 2 or table.shape[0] != n:
+        raise KernelError("qkv_rope_commit.table: needs one row per sequence")
+    _check(lib().tl_gemm_qkv_rope_commit(_p(a), _p(w), n, K, _p(row_pos), _p(inv_freq), _p(table),
+                                         table.shape[1], int(ring_pages), nq, nkv, d, _p(q), _p(pages),
+                                         _stream()))
+
+
 def aligned_columns(n_cached, n_new):
     """Column offsets (and their total) at which sequences lie when each is
     given room from the last multiple of 64 below its cached length up to its

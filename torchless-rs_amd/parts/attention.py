@@ -78,11 +78,15 @@ class AttentionMixer(Mixer):
         out = ws.get("attn_out", (n, nq, d), ctx.dtype)
         if self.own_kv and ctx.all_single and not run.kv_read_later:
             # one token a sequence: k and v go straight into the pages, then everything is read there
-            qkv = self.qkv.partial(y, ctx, "attn_qkv_parts")         # partial sums, added up by the rotation
-            if qkv is None:
-                qkv = ws.get("attn_qkv", (n, (nq + 2 * nkv) * d), torch.float32)
-                self.qkv(y, qkv)
-            ops.rope_commit(qkv, ctx.row_pos, inv_freq, table, group.ring_pages, nq, nkv, d, q, pages)
+            if ops.qkv_rope_commit_ok(y, self.qkv.weight, d, pages):
+                ops.qkv_rope_commit(y, self.qkv.weight, ctx.row_pos, inv_freq, table, group.ring_pages,
+                                    nq, nkv, d, q, pages)     # product, rotation and commit in one
+            else:
+                qkv = self.qkv.partial(y, ctx, "attn_qkv_parts")     # partial sums, added up by the rotation
+                if qkv is None:
+                    qkv = ws.get("attn_qkv", (n, (nq + 2 * nkv) * d), torch.float32)
+                    self.qkv(y, qkv)
+                ops.rope_commit(qkv, ctx.row_pos, inv_freq, table, group.ring_pages, nq, nkv, d, q, pages)
             ops.attention(q, None, None, pages, table, group.ring_pages, ctx, ctx.len_after,
                           self.window, self.scale, out)
             self.o.add_into(out.view(n, nq * d), x, ctx, "attn_o_parts")
