@@ -459,6 +459,7 @@ def decode_groups(B: int, nq: int, nkv: int) -> int:
 
 
 SPLIT_TARGET = 512          # workgroups a decode step's attention aims at
+SPLIT_PAGES = 4             # fewest pages a part of the keys has
 
 
 def decode_splits(B: int, nq: int, nkv: int, max_pages: int) -> int:
@@ -466,7 +467,7 @@ def decode_splits(B: int, nq: int, nkv: int, max_pages: int) -> int:
     has some two workgroups a compute unit to run, each with at least
     four pages (measured: more parts cost more in the merge than they gain)."""
     groups = decode_groups(B, nq, nkv)
-    return max(1, min(-(-max_pages // 4), -(-SPLIT_TARGET // groups), 4096))
+    return max(1, min(-(-max_pages // SPLIT_PAGES), -(-SPLIT_TARGET // groups), 4096))
 
 
 def uses_transposed_values(dtype: torch.dtype, d: int, all_single: bool) -> bool:
