@@ -11,6 +11,7 @@ the rows asked for.  A sequence's result does not depend on its batch-mates.
 """
 from __future__ import annotations
 
+import gc
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Sequence, Tuple
 
@@ -194,6 +195,7 @@ class _Graph:
     workspace: Workspace
     graph: object = None
     logits: Optional[torch.Tensor] = None
+    uploaded: Optional[torch.cuda.Event] = None      # the last copy out of `staging`
 
 
 class Engine:
@@ -211,6 +213,10 @@ class Engine:
         self.use_graphs = use_graphs
         self.max_graphs = 32
         self._graphs: Dict[tuple, _Graph] = {}
+        # The model's objects live as long as the process: take them out of the collector's
+        # sight, or its passes over them (a millisecond each, every few steps) stall the steps.
+        gc.collect()
+        gc.freeze()
 
     # ---- slots -----------------------------------------------------------
     def alloc(self) -> int:
@@ -263,8 +269,13 @@ class Engine:
                        staging=torch.empty(packed.flat.size, dtype=torch.int32).pin_memory(),
                        workspace=Workspace(self.device))
             self._graphs[key] = g
+        if g.uploaded is not None:
+            g.uploaded.synchronize()                 # the staging area is free to be written again
         g.staging.numpy()[:] = packed.flat
-        g.meta.copy_(g.staging)
+        g.meta.copy_(g.staging, non_blocking=True)
+        if g.uploaded is None:
+            g.uploaded = torch.cuda.Event()
+        g.uploaded.record()
         if g.graph is None and g.logits is not None:
             ctx, want_rows, n_want = context_from(packed, g.meta, self.cache, self.model.dtype,
                                                   self.device, g.workspace)

@@ -18,16 +18,33 @@ class Sampler:
         self.config = config
         self.device = device
         self._probs = None
+        self._stage = None               # pinned (sequence, step) pairs, and their copy on the device
+        self._counters = None
+        self._out = None
+        self._uploaded = None
 
     def sample(self, logits: torch.Tensor, seq_ids: Sequence[int], steps: Sequence[int]) -> List[int]:
         """logits: float32 [B, V] on the GPU -> B token ids."""
         B, V = logits.shape
         c = self.config
-        counters = torch.tensor([[int(s), int(t)] for s, t in zip(seq_ids, steps)], dtype=torch.int32,
-                                device=logits.device).view(B, 2)
+        if self._stage is None or self._stage.shape[0] < B:
+            self._stage = torch.empty((max(B, 64), 2), dtype=torch.int32).pin_memory()
+            self._counters = torch.empty((max(B, 64), 2), dtype=torch.int32, device=logits.device)
+            self._out = torch.empty((max(B, 64),), dtype=torch.int32, device=logits.device)
+            self._uploaded = None
+        if self._uploaded is not None:
+            self._uploaded.synchronize()             # the pinned pairs are free to be written again
+        stage = self._stage.numpy()
+        stage[:B, 0] = seq_ids
+        stage[:B, 1] = steps
+        counters = self._counters[:B]
+        counters.copy_(self._stage[:B], non_blocking=True)
+        if self._uploaded is None:
+            self._uploaded = torch.cuda.Event()
+        self._uploaded.record()
         if self._probs is None or self._probs.shape[0] < B or self._probs.shape[1] != V:
             self._probs = torch.empty((B, V), dtype=torch.float32, device=logits.device)
-        out = torch.empty((B,), dtype=torch.int32, device=logits.device)
+        out = self._out[:B]
         ops.sample(logits.contiguous(), float(c.temperature), int(c.top_k or 0), float(c.top_p or 0.0),
                    int(c.seed), counters, self._probs[:B], out)
         return out.tolist()
