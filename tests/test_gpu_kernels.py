@@ -581,6 +581,85 @@ def test_qkv_rope_commit_equals_product_then_rope_commit(ops, nq, nkv, d, K, len
                             torch.zeros(60, 2, nkv, 64, 8, dtype=torch.bfloat16, device=DEV))
 
 
+# ---- an RMSNorm cut in two around products of at most 16 rows ----------------------------
+
+@pytest.mark.parametrize("M", [1, 5, 16])
+@pytest.mark.parametrize("N,K,N2", [(200, 72, 50), (64, 264, 16384), (1000, 96, 130)])
+def test_gemm_norm_halves(ops, M, N, K, N2):
+    """The product that completes the stream writes x * w and its workgroups' sums of x^2;
+    the product that reads them applies rsqrt(mean + eps): together the plain norm between."""
+    eps = 1e-5
+    x0 = rnd(M, N, seed=51, scale=2.0)
+    a = rnd(M, K, seed=52, dtype=torch.bfloat16)
+    w = rnd(N, K, seed=53, dtype=torch.bfloat16)
+    g = (1 + 0.2 * rnd(N, seed=54))
+    x = x0.clone().to(DEV)
+    xt = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ssq = torch.full((16, -(-N // 16)), float("nan"), device=DEV)                # [row][workgroup]
+    groups = ops.gemm_bf16_norm(a.to(DEV), w.to(DEV), x, accumulate=True, norm_weight=g.to(DEV), xt=xt, ssq_out=ssq)
+    want_x = x0.double() + a.double() @ w.double().t()
+    assert rel_err(x, want_x) < 3e-6
+    plain_x = x0.clone().to(DEV)
+    ops.gemm_bf16(a.to(DEV), w.to(DEV), plain_x, accumulate=True)
+    assert torch.equal(plain_x, x)                                    # the stream itself is unchanged by the extra
+    assert groups == -(-N // 16)
+    assert rel_err(ssq[:M].sum(1), (x.double().cpu() ** 2).sum(1)) < 1e-5
+    assert rel_err(xt, x.double().cpu() * g.double()) < KTOL["bfloat16"]
+    factor = ops.RowFactor(ssq, groups, N, eps)
+    normed = plain.rmsnorm(x.double().cpu(), g.double(), eps)
+    w2 = rnd(N2, N, seed=55, dtype=torch.bfloat16, scale=0.3)
+    out = torch.full((M, N2), float("nan"), device=DEV)
+    ops.gemm_bf16_norm(xt, w2.to(DEV), out, factor=factor)
+    assert rel_err(out, normed @ w2.double().t()) < KTOL["bfloat16"]
+    # exactly: the unscaled product times the factor of the row
+    raw = torch.empty(M, N2, device=DEV)
+    ops.gemm_bf16(xt, w2.to(DEV), raw)
+    r = torch.rsqrt(ssq[:M].double().sum(1) / N + eps).float()
+    assert rel_err(out, raw.double().cpu() * r.double().cpu()[:, None]) < 1e-6
+    if N2 % 64 == 0:
+        from torchless_rs_amd.parts.linear import interleave_pairs
+        h = torch.full((M, N2 // 2), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ops.gemm_bf16_norm(xt, w2.to(DEV), h, silu_pair=True, factor=factor)
+        full = (normed @ w2.double().t()).view(M, N2 // 64, 2, 32)
+        assert rel_err(h, (plain.silu(full[:, :, 0]) * full[:, :, 1]).reshape(M, N2 // 2)) < KTOL["bfloat16"]
+    with pytest.raises(ops.KernelError, match="at most 16 rows"):
+        ops.gemm_bf16_norm(torch.zeros(17, K, dtype=torch.bfloat16, device=DEV), w.to(DEV),
+                           torch.zeros(17, N, device=DEV))
+    with pytest.raises(ops.KernelError, match="accumulate"):
+        ops.gemm_bf16_norm(a.to(DEV), w.to(DEV), x, norm_weight=g.to(DEV), xt=xt, ssq_out=ssq)
+
+
+def test_qkv_rope_commit_with_row_factor(ops):
+    from torchless_rs_amd.parts.position import Rotary
+    nq, nkv, d, K, lens, eps = 6, 2, 48, 136, [0, 63, 64, 300, 7], 1e-6
+    n = len(lens)
+    c = paged_case(ops, "bfloat16", nq, nkv, d, None, lens_cached=lens, lens_new=[1] * n, seed=12, n_pages=60)
+    x = rnd(n, K, seed=13, scale=3.0)
+    g = (1 + 0.2 * rnd(K, seed=14))
+    xt = (x * g).to(torch.bfloat16).to(DEV)
+    parts = 5                                                   # the sums of squares, cut into 5 unequal shares
+    cuts = [0, 10, 50, 51, 100, K]
+    ssq = torch.zeros(16, parts)
+    for j in range(parts):
+        ssq[:n, j] = (x[:, cuts[j]:cuts[j + 1]] ** 2).sum(1)
+    factor = ops.RowFactor(ssq.to(DEV), parts, K, eps)
+    w = rnd((nq + 2 * nkv) * d, K, seed=15, dtype=torch.bfloat16, scale=0.2).to(DEV)
+    inv = Rotary(d, 10000.0).inv_freq(DEV)
+    q = torch.full((n, nq, d), float("nan"), dtype=torch.bfloat16, device=DEV)
+    pages = c["pages"].clone()
+    ops.qkv_rope_commit(xt, w, c["row_pos"], inv, c["table"], c["ring"], nq, nkv, d, q, pages, factor=factor)
+    y = plain.rmsnorm(x.double(), g.double(), eps)
+    full = (y @ w.double().cpu().t()).view(n, nq + 2 * nkv, d)
+    pos = c["row_pos"].cpu().long()
+    assert rel_err(q, plain.rope(full[:, :nq], pos, 10000.0)) < KTOL["bfloat16"]
+    want_k = plain.rope(full[:, nq:nq + nkv], pos, 10000.0)
+    table = c["table"].cpu()
+    for b in range(n):
+        p = int(pos[b]); pg = int(table[b, p // 64])
+        assert rel_err(pages[pg, 0, :, p % 64], want_k[b]) < KTOL["bfloat16"]
+        assert rel_err(pages[pg, 1].reshape(nkv, d, 64)[:, :, p % 64], full[b, nq + nkv:]) < KTOL["bfloat16"]
+
+
 # ---- 17..64 rows: shared activations, K cut into partial sums -----------------------------
 
 @pytest.mark.parametrize("M", [17, 32, 33, 48, 50, 64, 5])

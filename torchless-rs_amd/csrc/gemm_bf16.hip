@@ -30,12 +30,66 @@ constexpr int EPI_ACCUMULATE = 1;   // C += product (float; the residual stream)
 constexpr int EPI_SILU_PAIR = 2;    // W's rows come in groups of 64 (32 gate rows, their 32 up rows):
                                     // C is bfloat16 [M, N/2] = silu(gate) * up
 
+// An RMSNorm cut in two around a product of at most 16 rows, so that the norm needs no
+// kernel of its own.  The product that completes the residual stream (accumulate epilogue)
+// also writes xt = bfloat16(x * norm_w) and, per workgroup and row, the sum of x^2 over its
+// channels (`ssq_out`, [16][workgroups]).  The product that reads xt adds those sums up in
+// a fixed order and multiplies its results by rsqrt(sum * inv_h + eps) (`ssq_in`, `n_part`):
+// y = x / sqrt(mean(x^2) + eps) * w  (src/kernels/mod.rs:558-568 of the reference), with the
+// division moved behind the product, where it is a factor per row.
+struct NormSplit {
+  const float* ssq_in;      // reader: partial sums [16][n_part]; null: no factor
+  int n_part;
+  float inv_h, eps;
+  const float* norm_w;      // writer: the next norm's weight [N]; null: plain epilogue
+  bf16* xt;                 // [M][N]
+  float* ssq_out;           // [16][gridDim.x]
+};
+
+// rsqrt(mean + eps) of rows 0..15 into rs[16], by the first 256 threads (16 per row), in two
+// steps so that the loads are under way while the product runs: `fetch` early, `finish` before
+// the barrier that precedes the epilogue.  ssq_in is [16][n_part].
+struct RowFactors {
+  f32x4 part[4];
+  __device__ __forceinline__ void fetch(const NormSplit& ns) {
+    const int tid = threadIdx.x, m = tid / 16, jl = tid % 16;
+    if (tid >= 256) return;
+    const float* row = ns.ssq_in + (size_t)m * ns.n_part;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int j = jl * 4 + 64 * i;
+      f32x4 v = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (j + 3 < ns.n_part && ns.n_part % 4 == 0) {
+        v = *reinterpret_cast<const f32x4*>(row + j);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (j + e < ns.n_part) v[e] = row[j + e];
+      }
+      part[i] = v;
+    }
+  }
+  __device__ __forceinline__ void finish(const NormSplit& ns, float* rs) {
+    const int tid = threadIdx.x, m = tid / 16, jl = tid % 16;
+    if (tid >= 256) return;
+    float v = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v += (part[i][0] + part[i][1]) + (part[i][2] + part[i][3]);
+    const float* row = ns.ssq_in + (size_t)m * ns.n_part;
+    for (int j = 256 + jl; j < ns.n_part; j += 16) v += row[j];      // more than 256 workgroups wrote
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+    if (jl == 0) rs[m] = rsqrtf(v * ns.inv_h + ns.eps);
+  }
+};
+
 // ---------------------------------------------------------------- skinny ----
 template <int NT, int MT, int SK_WAVES>
 __global__ void __launch_bounds__(SK_WAVES * 64)
 gemm_skinny_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float* __restrict__ C, int M,
-                   int N, int K, int epilogue) {
+                   int N, int K, int epilogue, NormSplit ns) {
   __shared__ float red[SK_WAVES][NT * MT * 256];
+  __shared__ float rs[16];
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const int li = lane % 16, kg = lane / 16;
   const int n0 = blockIdx.x * (16 * NT);
@@ -85,6 +139,9 @@ gemm_skinny_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float
   bf16x8 w0[NT][2], a0[MT][2], w1[NT][2], a1[MT][2];
   int s = s0;
   if (s < s1) load_step(s, w0, a0);
+  const bool scaled = MT == 1 && ns.ssq_in != nullptr;
+  RowFactors rf;
+  if (scaled) rf.fetch(ns);
   for (; s + 1 < s1; s += 2) {
     load_step(s + 1, w1, a1);
     mma_step(w0, a0);
@@ -93,6 +150,7 @@ gemm_skinny_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float
   }
   if (s < s1) mma_step(w0, a0);
 
+  if (scaled) rf.finish(ns, rs);
   // acc[t][u][r] is D[n = 4*kg + r][m = li] of tile (t, u)
 #pragma unroll
   for (int t = 0; t < NT; ++t)
@@ -108,7 +166,7 @@ gemm_skinny_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float
     float v = 0.f;
 #pragma unroll
     for (int w = 0; w < SK_WAVES; ++w) v += red[w][idx];
-    return v;
+    return scaled ? v * rs[m % 16] : v;
   };
   if (epilogue == EPI_SILU_PAIR) {
     // rows come in groups of 64: 32 gate rows, then the 32 up rows that belong to them
@@ -127,22 +185,32 @@ gemm_skinny_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float
     }
     return;
   }
+  const bool writer = MT == 1 && ns.norm_w != nullptr;          // with EPI_ACCUMULATE only (checked on the host)
   for (int e = threadIdx.x; e < NB * 16 * MT; e += SK_WAVES * 64) {
     const int nl = e % NB, m = e / NB;
     const float v = total(nl, m);
     const int n = n0 + nl;
+    float xn = 0.f;
     if (n < N && m < M) {
       float* c = C + (size_t)m * N + n;
-      *c = (epilogue == EPI_ACCUMULATE) ? *c + v : v;
+      xn = (epilogue == EPI_ACCUMULATE) ? *c + v : v;
+      *c = xn;
+      if (writer) ns.xt[(size_t)m * N + n] = (bf16)(xn * ns.norm_w[n]);
+    }
+    if (writer) {                  // whole waves get here: NB lanes in a row share m
+      float q = xn * xn;
+#pragma unroll
+      for (int o = NB / 2; o > 0; o >>= 1) q += __shfl_xor(q, o, WAVE);
+      if (nl == 0) ns.ssq_out[(size_t)m * gridDim.x + blockIdx.x] = q;
     }
   }
 }
 
 template <int NT, int MT, int SK_WAVES = 8>
 static int launch_skinny(const bf16* A, const bf16* W, float* C, int M, int N, int K, int epilogue,
-                         hipStream_t st) {
+                         hipStream_t st, NormSplit ns = NormSplit{}) {
   const int grid = (N + 16 * NT - 1) / (16 * NT);
-  gemm_skinny_kernel<NT, MT, SK_WAVES><<<grid, SK_WAVES * 64, 0, st>>>(A, W, C, M, N, K, epilogue);
+  gemm_skinny_kernel<NT, MT, SK_WAVES><<<grid, SK_WAVES * 64, 0, st>>>(A, W, C, M, N, K, epilogue, ns);
   TL_LAUNCH_CHECK("gemm_skinny");
   return 0;
 }
@@ -162,9 +230,10 @@ __global__ void __launch_bounds__(QKV_WAVES * 64)
 gemm_qkv_rope_commit_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, int M, int K,
                             const int* __restrict__ row_pos, const float* __restrict__ inv_freq,
                             const int* __restrict__ table, int table_stride, int ring_pages, int nq,
-                            int nkv, int d, bf16* __restrict__ q, bf16* __restrict__ pages) {
+                            int nkv, int d, bf16* __restrict__ q, bf16* __restrict__ pages, NormSplit ns) {
   __shared__ float red[QKV_WAVES][256];
   __shared__ float cs[16][8], sn[16][8];
+  __shared__ float rs[16];
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
   const int li = lane % 16, kg = lane / 16;
   const int tiles = d / 16, head = blockIdx.x / tiles, tt = blockIdx.x % tiles;
@@ -197,6 +266,9 @@ gemm_qkv_rope_commit_kernel(const bf16* __restrict__ A, const bf16* __restrict__
     const int m = tid / 8, j = tid % 8;
     if (m < M) sincosf(inv_freq[8 * tt + j] * (float)row_pos[m], &sn[m][j], &cs[m][j]);
   }
+  const bool scaled = ns.ssq_in != nullptr;
+  RowFactors rf;
+  if (scaled) rf.fetch(ns);
   for (; s + 1 < s1; s += 2) {
     load_step(s + 1, w1, a1);
     mma_step(w0, a0);
@@ -204,6 +276,7 @@ gemm_qkv_rope_commit_kernel(const bf16* __restrict__ A, const bf16* __restrict__
     mma_step(w1, a1);
   }
   if (s < s1) mma_step(w0, a0);
+  if (scaled) rf.finish(ns, rs);
 #pragma unroll
   for (int r = 0; r < 4; ++r) red[wave][r * 64 + lane] = acc[r];     // D[n = 4 kg + r][m = li]
   __syncthreads();
@@ -212,7 +285,7 @@ gemm_qkv_rope_commit_kernel(const bf16* __restrict__ A, const bf16* __restrict__
     float v = 0.f;
 #pragma unroll
     for (int w = 0; w < QKV_WAVES; ++w) v += red[w][idx];
-    return v;
+    return scaled ? v * rs[m] : v;
   };
   const size_t page_elems = 2 * (size_t)nkv * PAGE * d;
   if (rotated) {
@@ -735,9 +808,11 @@ extern "C" int tl_gemm_mid_bf16(const void* A, const void* W, void* C, int M, in
 
 // q|k|v of a step with one token a sequence (row m is sequence m, at position row_pos[m]):
 // W is [(nq + 2 nkv) d, K]; q receives [M, nq, d], the pages k and v of the new position.
+// With ssq_in, row m's sums are multiplied by rsqrt(sum_j ssq_in[m][j] * inv_h + eps) first.
 extern "C" int tl_gemm_qkv_rope_commit(const void* A, const void* W, int M, int K, const int* row_pos,
                                        const float* inv_freq, const int* table, int table_stride,
                                        int ring_pages, int nq, int nkv, int d, void* q, void* pages,
+                                       const float* ssq_in, int n_part, float inv_h, float eps,
                                        hipStream_t st) {
   TL_REQUIRE(M >= 0 && M <= 16 && K > 0 && K % 8 == 0, "qkv_rope_commit: bad sizes M=%d K=%d (at most 16 rows, "
              "K a multiple of 8)", M, K);
@@ -746,11 +821,47 @@ extern "C" int tl_gemm_qkv_rope_commit(const void* A, const void* W, int M, int 
   TL_REQUIRE(ring_pages > 0 && table_stride > 0, "qkv_rope_commit: bad cache geometry ring_pages=%d "
              "table_stride=%d", ring_pages, table_stride);
   TL_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "qkv_rope_commit: operands must be 16-byte aligned");
+  TL_REQUIRE(ssq_in == nullptr || n_part > 0, "qkv_rope_commit: %d partial sums of squares", n_part);
   if (M == 0) return 0;
   const int grid = (nq + 2 * nkv) * (d / 16);
+  NormSplit ns{};
+  ns.ssq_in = ssq_in; ns.n_part = n_part; ns.inv_h = inv_h; ns.eps = eps;
   gemm_qkv_rope_commit_kernel<<<grid, QKV_WAVES * 64, 0, st>>>((const bf16*)A, (const bf16*)W, M, K, row_pos,
                                                               inv_freq, table, table_stride, ring_pages, nq,
-                                                              nkv, d, (bf16*)q, (bf16*)pages);
+                                                              nkv, d, (bf16*)q, (bf16*)pages, ns);
   TL_LAUNCH_CHECK("gemm_qkv_rope_commit");
   return 0;
+}
+
+// The product for at most 16 rows with an RMSNorm cut in two around it (see NormSplit).
+// ssq_in [16][n_part] (or null): a factor per row on the results.  norm_w [N], xt [M][N],
+// ssq_out [16][workgroups] (or all null): with the accumulate epilogue, also write
+// xt = bfloat16(C * norm_w) and the workgroups' sums of C^2; *n_groups receives the number
+// of workgroups, which is the n_part of the product that reads xt.
+extern "C" int tl_gemm_bf16_norm(const void* A, const void* W, void* C, int M, int N, int K, int epilogue,
+                                 const float* ssq_in, int n_part, float inv_h, float eps,
+                                 const float* norm_w, void* xt, float* ssq_out, int ssq_capacity,
+                                 int* n_groups, hipStream_t st) {
+  TL_REQUIRE(M >= 0 && M <= 16 && N > 0 && K > 0 && K % 8 == 0, "gemm_bf16_norm: bad sizes M=%d N=%d K=%d (at most "
+             "16 rows, K a multiple of 8)", M, N, K);
+  TL_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "gemm_bf16_norm: operands must be 16-byte aligned");
+  TL_REQUIRE(epilogue >= 0 && epilogue <= 2, "gemm_bf16_norm: unknown epilogue %d", epilogue);
+  TL_REQUIRE(epilogue != EPI_SILU_PAIR || N % 64 == 0, "gemm_bf16_norm: the paired epilogue needs N=%d to be "
+             "a multiple of 64", N);
+  TL_REQUIRE(ssq_in == nullptr || n_part > 0, "gemm_bf16_norm: %d partial sums of squares", n_part);
+  const bool writer = norm_w != nullptr;
+  TL_REQUIRE(!writer || (epilogue == EPI_ACCUMULATE && xt != nullptr && ssq_out != nullptr),
+             "gemm_bf16_norm: the next norm's half goes with the accumulate epilogue, xt and ssq_out");
+  const bool wide = N >= 16384 || epilogue == EPI_SILU_PAIR;
+  const bool four = wide && (M > 4 || epilogue == EPI_SILU_PAIR);
+  const int groups = four ? (N + 63) / 64 : (N + 15) / 16;
+  if (n_groups) *n_groups = groups;
+  TL_REQUIRE(!writer || ssq_capacity >= groups * 16, "gemm_bf16_norm: ssq_out holds %d floats, %d are needed",
+             ssq_capacity, groups * 16);
+  if (M == 0) return 0;
+  NormSplit ns{};
+  ns.ssq_in = ssq_in; ns.n_part = n_part; ns.inv_h = inv_h; ns.eps = eps;
+  ns.norm_w = norm_w; ns.xt = (bf16*)xt; ns.ssq_out = ssq_out;
+  if (four) return launch_skinny<4, 1, 4>((const bf16*)A, (const bf16*)W, (float*)C, M, N, K, epilogue, st, ns);
+  return launch_skinny<1, 1, 8>((const bf16*)A, (const bf16*)W, (float*)C, M, N, K, epilogue, st, ns);
 }

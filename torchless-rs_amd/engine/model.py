@@ -106,8 +106,14 @@ class Model:
         ws = ctx.workspace
         x = ws.get("residual", (ctx.n_rows, H), torch.float32)
         self.embedding.forward(ctx, ctx.tokens, x)
-        for run, binding in zip(self.spec.schedule, runs):
-            self.blocks[run.layer].forward(ctx, binding, x)
+        order = [self.blocks[run.layer] for run in self.spec.schedule]
+        for i, (block, binding) in enumerate(zip(order, runs)):
+            after = order[i + 1].entry_norm() if i + 1 < len(order) and hasattr(order[i + 1], "entry_norm") else None
+            if after is not None:
+                block.forward(ctx, binding, x, norm_after=after)
+            else:
+                block.forward(ctx, binding, x)
+        ctx.prenormed = None                 # nothing reads a norm's first half past the last block
         for commit in ctx.host.pop("deferred", []):
             commit()
         flush_pending(ctx, x)

@@ -239,6 +239,60 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: b
         _check(lib().tl_gemm_bf16_variant(_p(a), _p(w), _p(out), M, N, K, epi, int(variant), _stream()))
 
 
+class RowFactor:
+    """The second half of an RMSNorm cut in two around a product: sums of x^2 per
+    workgroup of the product that wrote the stream (`ssq` [16, n_part], float32), from
+    which the reading product makes rsqrt(sum / size + eps) per row."""
+
+    def __init__(self, ssq: torch.Tensor, n_part: int, size: int, eps: float):
+        self.ssq, self.n_part, self.size, self.eps = ssq, int(n_part), int(size), float(eps)
+
+
+def norm_split_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
+    """Can `gemm_bf16_norm` take this product (bfloat16, at most 16 rows)?"""
+    return bf16_gemm_ok(a, w) and a.shape[0] <= 16
+
+
+def gemm_bf16_norm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False,
+                   silu_pair: bool = False, factor: Optional[RowFactor] = None,
+                   norm_weight: Optional[torch.Tensor] = None, xt: Optional[torch.Tensor] = None,
+                   ssq_out: Optional[torch.Tensor] = None) -> int:
+    """`gemm_bf16` for at most 16 rows with the halves of an RMSNorm around it.
+    `factor`: every row of the result is multiplied by its rsqrt(mean(x^2) + eps).
+    `norm_weight`, `xt`, `ssq_out` (with `accumulate`): out += product, xt =
+    bfloat16(out * norm_weight), ssq_out[m, g] = the sum of out[m, :]^2 over workgroup g's
+    channels.  Returns the number of workgroups (the reader's n_part)."""
+    M, K = a.shape
+    N = w.shape[0]
+    _req(a, "gemm.a", torch.bfloat16)
+    _req(w, "gemm.w", torch.bfloat16, (N, K))
+    if silu_pair:
+        if accumulate or N % 64:
+            raise KernelError("gemm: the paired epilogue stores, and needs N to be a multiple of 64")
+        _req(out, "gemm.out", torch.bfloat16, (M, N // 2))
+        epi = EPI_SILU_PAIR
+    else:
+        _req(out, "gemm.out", torch.float32, (M, N))
+        epi = EPI_ACCUMULATE if accumulate else EPI_STORE
+    ssq_in, n_part, inv_h, eps = None, 0, 0.0, 0.0
+    if factor is not None:
+        _req(factor.ssq, "gemm.factor", torch.float32)
+        if factor.ssq.numel() < factor.n_part * 16 or factor.n_part < 1:
+            raise KernelError(f"gemm.factor: {factor.ssq.numel()} floats for {factor.n_part} workgroups")
+        ssq_in, n_part, inv_h, eps = factor.ssq, factor.n_part, 1.0 / factor.size, factor.eps
+    cap = 0
+    if norm_weight is not None:
+        _req(norm_weight, "gemm.norm_weight", torch.float32, (N,))
+        _req(xt, "gemm.xt", torch.bfloat16, (M, N))
+        _req(ssq_out, "gemm.ssq_out", torch.float32)
+        cap = ssq_out.numel()
+    groups = ctypes.c_int(0)
+    _check(lib().tl_gemm_bf16_norm(_p(a), _p(w), _p(out), M, N, K, epi, _p(ssq_in), n_part,
+                                   ctypes.c_float(inv_h), ctypes.c_float(eps), _p(norm_weight), _p(xt),
+                                   _p(ssq_out), cap, ctypes.byref(groups), _stream()))
+    return groups.value
+
+
 def mid_splits(M: int, N: int, K: int) -> int:
     """For 17..64 rows: into how many slices K is cut so that some 400
     workgroups (64 output channels each) are at work; 1 where N alone gives
@@ -364,10 +418,11 @@ def qkv_rope_commit_ok(a: torch.Tensor, w: torch.Tensor, d: int, pages: torch.Te
 
 
 def qkv_rope_commit(a: torch.Tensor, w: torch.Tensor, row_pos, inv_freq, table, ring_pages: int, nq: int,
-                    nkv: int, d: int, q: torch.Tensor, pages: torch.Tensor) -> None:
+                    nkv: int, d: int, q: torch.Tensor, pages: torch.Tensor,
+                    factor: Optional[RowFactor] = None) -> None:
     """For a step with one token a sequence (at most 16): the product a @ w^T with w = q|k|v,
     the rotation of q and k, q into its buffer and k, v into the pages, in one kernel; the
-    same bits as `gemm` and then `rope_commit`."""
+    same bits as `gemm` and then `rope_commit`.  `factor`: see `gemm_bf16_norm`."""
     n, K = a.shape
     _req(a, "qkv_rope_commit.a", torch.bfloat16)
     _req(w, "qkv_rope_commit.w", torch.bfloat16, ((nq + 2 * nkv) * d, K))
@@ -380,8 +435,15 @@ def qkv_rope_commit(a: torch.Tensor, w: torch.Tensor, row_pos, inv_freq, table, 
         raise KernelError(f"qkv_rope_commit.pages: shape {tuple(pages.shape)}, kernel needs [*, 2, {nkv}, 64, {d}]")
     if table.dim() != 2 or table.shape[0] != n:
         raise KernelError("qkv_rope_commit.table: needs one row per sequence")
+    ssq_in, n_part, inv_h, eps = None, 0, 0.0, 0.0
+    if factor is not None:
+        _req(factor.ssq, "qkv_rope_commit.factor", torch.float32)
+        if factor.ssq.numel() < factor.n_part * 16 or factor.n_part < 1:
+            raise KernelError(f"qkv_rope_commit.factor: {factor.ssq.numel()} floats for {factor.n_part} workgroups")
+        ssq_in, n_part, inv_h, eps = factor.ssq, factor.n_part, 1.0 / factor.size, factor.eps
     _check(lib().tl_gemm_qkv_rope_commit(_p(a), _p(w), n, K, _p(row_pos), _p(inv_freq), _p(table),
                                          table.shape[1], int(ring_pages), nq, nkv, d, _p(q), _p(pages),
+                                         _p(ssq_in), n_part, ctypes.c_float(inv_h), ctypes.c_float(eps),
                                          _stream()))
 
 

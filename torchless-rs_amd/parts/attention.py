@@ -24,12 +24,14 @@ import torch
 from ..cache.cache import KVRequest
 from ..kernels import ops
 from ..weights.binding import WeightSpec
-from .base import Mixer, PartSpec, make_part, register_part
+from .base import Mixer, PartSpec, make_part, register_part, take_row_factor
 from .linear import Linear
 
 
 class AttentionMixer(Mixer):
     graph_safe = True
+    closes_stream = True          # its last write to the stream is `Linear.add_into`
+    takes_row_factor = True       # its q|k|v product can do the division of the norm before it
 
     def __init__(self, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int,
                  position: PartSpec, window: Optional[int] = None, own_kv: bool = True,
@@ -76,11 +78,14 @@ class AttentionMixer(Mixer):
         inv_freq = self.position.inv_freq(y.device)
         q = ws.get("attn_q", (n, nq, d), ctx.dtype)
         out = ws.get("attn_out", (n, nq, d), ctx.dtype)
+        fused = (self.own_kv and ctx.all_single and not run.kv_read_later
+                 and ops.qkv_rope_commit_ok(y, self.qkv.weight, d, pages))
+        factor = take_row_factor(ctx, usable=fused)
         if self.own_kv and ctx.all_single and not run.kv_read_later:
             # one token a sequence: k and v go straight into the pages, then everything is read there
-            if ops.qkv_rope_commit_ok(y, self.qkv.weight, d, pages):
+            if fused:
                 ops.qkv_rope_commit(y, self.qkv.weight, ctx.row_pos, inv_freq, table, group.ring_pages,
-                                    nq, nkv, d, q, pages)     # product, rotation and commit in one
+                                    nq, nkv, d, q, pages, factor=factor)     # product, rotation and commit in one
             else:
                 qkv = self.qkv.partial(y, ctx, "attn_qkv_parts")     # partial sums, added up by the rotation
                 if qkv is None:

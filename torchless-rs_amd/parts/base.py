@@ -166,6 +166,19 @@ class RunBinding:
     state: Optional[torch.Tensor] = None      # [max_slots, *shape]
 
 
+def take_row_factor(ctx: "StepContext", usable: bool):
+    """For a part whose input came from a norm: the factor per row that its first product
+    has to apply (None: the input is normed already).  A part that cannot apply it
+    (`usable` false) gets the plain norm written into its input instead."""
+    f = ctx.row_factor
+    ctx.row_factor = None
+    if f is not None and not usable:
+        ctx.settle()
+        f = None
+    ctx.settle = None
+    return f
+
+
 def flush_pending(ctx: "StepContext", x: torch.Tensor) -> None:
     """Add partial products that a part left in `ctx.pending` to the stream."""
     if ctx.pending is not None:
@@ -228,4 +241,15 @@ class StepContext:
     # a product may leave them here instead of adding them itself; whoever reads the stream
     # next (a norm that can, else `flush`) adds them up
     pending: Optional[torch.Tensor] = None
+    # An RMSNorm may be cut in two around the products next to it (steps of at most 16 rows):
+    # `norm_ahead` is the norm that reads the stream next, set by whoever knows it while a
+    # part runs whose last write to the stream is `Linear.add_into` (`closes_stream`), which
+    # may then do the norm's first half; `prenormed` is what such a
+    # product left: (norm, x * weight in the compute dtype, `ops.RowFactor`); `row_factor`
+    # is handed by the norm to the part that reads its output, which must take it
+    # (`take_row_factor`) and pass it to its first product, or ask `settle` for the plain norm
+    norm_ahead: Any = None
+    prenormed: Any = None
+    row_factor: Any = None
+    settle: Any = None
     host: Dict[str, Any] = field(default_factory=dict)     # the same data on the host

@@ -10,12 +10,14 @@ import torch
 
 from ..kernels import ops
 from ..weights.binding import WeightSpec
-from .base import FeedForward, register_part
+from .base import FeedForward, register_part, take_row_factor
 from .linear import Linear, interleave_pairs
 
 
 class SwiGLU(FeedForward):
     graph_safe = True
+    closes_stream = True          # its last write to the stream is `Linear.add_into`
+    takes_row_factor = True       # its gate|up product can do the division of the norm before it
 
     def __init__(self, hidden_size: int, intermediate_size: int, prefix: str = "mlp."):
         self.H = int(hidden_size)
@@ -45,7 +47,10 @@ class SwiGLU(FeedForward):
     def forward(self, ctx, y: torch.Tensor, x: torch.Tensor) -> None:
         n = y.shape[0]
         h = ctx.workspace.get("ffn_h", (n, self.I), ctx.dtype)
-        if self.paired and self.gate_up.mid(y):
+        factor = take_row_factor(ctx, usable=self.paired and ops.norm_split_ok(y, self.gate_up.weight))
+        if factor is not None:
+            ops.gemm_bf16_norm(y, self.gate_up.weight, h, silu_pair=True, factor=factor)
+        elif self.paired and self.gate_up.mid(y):
             ops.gemm_mid_bf16(y, self.gate_up.weight, h, 1, silu_pair=True)
         elif self.paired and ops.bf16_gemm_ok(y, self.gate_up.weight):
             if n > ops.LIBRARY_ROWS:

@@ -17,9 +17,12 @@ class Linear:
         self.weight = weight.contiguous()
         self.out_features, self.in_features = self.weight.shape
 
-    def __call__(self, a: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
-        """out[M, N] (+)= a[M, K] @ W^T; out is float32."""
-        if self.mid(a):
+    def __call__(self, a: torch.Tensor, out: torch.Tensor, accumulate: bool = False, factor=None) -> None:
+        """out[M, N] (+)= a[M, K] @ W^T; out is float32.  `factor` (`ops.RowFactor`): the
+        second half of the norm that made `a`, a factor per row (at most 16 rows)."""
+        if factor is not None:
+            ops.gemm_bf16_norm(a, self.weight, out, accumulate, factor=factor)
+        elif self.mid(a):
             ops.gemm_mid_bf16(a, self.weight, out, 1, accumulate)
         else:
             ops.gemm(a, self.weight, out, accumulate)
@@ -44,6 +47,16 @@ class Linear:
         """x += a @ W^T, now or as partial sums left in `ctx.pending`."""
         from .base import flush_pending
         flush_pending(ctx, x)
+        norm = ctx.norm_ahead
+        if (norm is not None and ops.norm_split_ok(a, self.weight) and norm.size == self.out_features
+                and norm.weight is not None and norm.weight.dtype == torch.float32):
+            # the next norm's first half rides on this product
+            xt = ctx.workspace.get("prenormed_y", (a.shape[0], self.out_features), torch.bfloat16)
+            ssq = ctx.workspace.get(name + "_ssq", (16, -(-self.out_features // 16)), torch.float32)
+            groups = ops.gemm_bf16_norm(a, self.weight, x, accumulate=True, norm_weight=norm.weight, xt=xt,
+                                        ssq_out=ssq)
+            ctx.prenormed = (norm, xt, ops.RowFactor(ssq, groups, norm.size, norm.eps))
+            return
         parts = self.partial(a, ctx, name)
         if parts is None:
             self(a, x, accumulate=True)

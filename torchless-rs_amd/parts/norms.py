@@ -14,6 +14,7 @@ from .base import Norm, register_part
 class RMSNorm(Norm):
     graph_safe = True
     takes_pending = True        # adds partial products left in ctx.pending while it reads the stream
+    splits = True               # a product before it may do its sums, a product after it its division
 
     def __init__(self, size: int, eps: float):
         self.size = int(size)
