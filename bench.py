@@ -75,7 +75,7 @@ def main() -> int:
         steps (model step + greedy sampling)."""
         held = min(context, W) if W else context
         eng = engine or Engine(model, max_tokens=batch * (-(-held // 64) * 64 + 64), max_slots=batch)
-        plen = max(1, context - steps - warmup)
+        plen = max(1, context - steps - warmup - 1)
         slots = [eng.alloc() for _ in range(batch)]
         chunk = 2048
         for s in slots:                                  # prompt by prompt, in chunks
@@ -84,12 +84,19 @@ def main() -> int:
                 part = ids[c0:c0 + chunk]
                 last = c0 + chunk >= plen
                 lg = eng.step([SeqInput(s, part, [len(part) - 1] if last else [])])
-        toks = sampler.sample(lg, [0], [0]) * batch
+        first = sampler.sample(lg, [0], [0]) * batch
+        lg = eng.step([SeqInput(s, [t], [0]) for s, t in zip(slots, first)])
+        drawn = sampler.draw(lg, list(range(batch)), [0] * batch)
+        entries = [SeqInput(s, [0], [0]) for s in slots]
 
         def one():
-            nonlocal toks
-            lg = eng.step([SeqInput(s, [t], [0]) for s, t in zip(slots, toks)])
-            toks = sampler.sample(lg, list(range(batch)), [0] * batch)
+            # as the generation loop runs: the next step is launched with the drawn tokens still on
+            # the device, then the host reads the tokens of the step before
+            nonlocal drawn
+            lg = eng.step(entries, device_tokens=drawn.device)
+            ahead = sampler.draw(lg, list(range(batch)), [0] * batch)
+            drawn.tokens()
+            drawn = ahead
 
         for _ in range(warmup):
             one()

@@ -104,3 +104,68 @@ def test_plan_by_pages():
     assert plan_batches([1] * 5, fits, 2) == [[0, 1], [2, 3], [4]]
     with pytest.raises(ValueError, match="more than the cache holds"):
         plan_batches([10, 300], fits, None)
+
+
+# ---- running ahead: the next step is launched before the host has read the tokens -----------
+
+class AheadEngine(StrawEngine):
+    """Takes a step's tokens from a tensor 'on the device' when asked to."""
+
+    def step(self, batch, device_tokens=None, token_rows=None):
+        if device_tokens is not None:
+            assert all(list(b.tokens) == [0] for b in batch) and len(token_rows) == len(batch)
+            batch = [type(b)(b.slot, [int(device_tokens[r])], b.want) for b, r in zip(batch, token_rows)]
+        return super().step(batch)
+
+
+class DrawingSampler(ArgmaxSampler):
+    def __init__(self):
+        super().__init__()
+        self.unread = 0                # draws whose tokens the host has not looked at yet
+
+    def draw(self, logits, seq_ids, steps):
+        self.calls.append((list(seq_ids), list(steps)))
+        ids = logits.argmax(-1).to(torch.int32)
+        self.unread += 1
+        outer = self
+
+        class Drawn:
+            device = ids
+
+            def tokens(self):
+                outer.unread -= 1
+                return ids.tolist()
+        return Drawn()
+
+
+@pytest.mark.parametrize("prompts,max_tokens,stops", [
+    ([[1, 2, 3], [10], [20, 21]], 4, []),
+    ([[1], [40], [7]], 6, [43, 9]),
+    ([[4]], 3, [5]),
+    ([[4], [6]], 1, []),
+    ([[i] for i in range(5)], 3, [3, 6]),
+])
+def test_running_ahead_gives_the_same_tokens(prompts, max_tokens, stops):
+    seen_a, seen_b = [], []
+    a = generate(StrawEngine(slots=2), ArgmaxSampler(), prompts, max_tokens, stops, max_batch=2,
+                 on_token=lambda i, t: seen_a.append((i, t)))
+    eng, smp = AheadEngine(slots=2), DrawingSampler()
+    b = generate(eng, smp, prompts, max_tokens, stops, max_batch=2, on_token=lambda i, t: seen_b.append((i, t)))
+    assert [(r.tokens, r.finish_reason) for r in a] == [(r.tokens, r.finish_reason) for r in b]
+    assert sorted(seen_a) == sorted(seen_b)
+    assert not eng.held and smp.unread == 0                  # every slot given back, every draw read
+
+
+def test_running_ahead_steps():
+    eng, smp = AheadEngine(), DrawingSampler()
+    out = generate(eng, smp, [[1], [40], [7]], max_tokens=6, stop_ids=[43, 9])
+    assert out[1].tokens == [41, 42] and out[2].tokens == [8]
+    # a sequence that draws a stop id has run one row more than without running ahead
+    # ([[1, 1, 1], [1, 1, 1], [1, 1], [1], [1], [1]]); budgets are known beforehand: no row past them
+    assert eng.steps == [[1, 1, 1], [1, 1, 1], [1, 1, 1], [1, 1], [1], [1]]
+    assert smp.calls[2] == ([0, 1, 2], [2, 2, 2])            # (request, its step) as without running ahead
+    eng, smp = AheadEngine(), DrawingSampler()
+    generate(eng, smp, [[1, 2], [5]], max_tokens=3)
+    assert eng.steps == [[2, 1], [1, 1], [1, 1]]             # 3 tokens each: the last is never fed
+    out = generate(AheadEngine(), DrawingSampler(), [[1]], max_tokens=5, run_ahead=False)
+    assert out[0].tokens == [2, 3, 4, 5, 6]

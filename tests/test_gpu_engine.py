@@ -281,6 +281,60 @@ def test_temperature_generation_follows_the_seeded_draws(zoo):
     assert len(again) == len(out)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_running_ahead_gives_the_tokens_of_the_step_by_step_loop(zoo, dtype):
+    """The next step takes the drawn tokens on the device before the host has read them;
+    stop ids, budgets and batches one after another come out as in the loop that waits."""
+    from torchless_rs_amd import SamplingConfig
+    from torchless_rs_amd.engine.generate import generate
+    from torchless_rs_amd.sampling.sampler import Sampler
+    DEV = "cuda:0"
+    eng, z = engine_for(zoo, "A", dtype), zoo["A"]
+    ps = (z["prompts"] * 3)[:7]
+    for cfg in (SamplingConfig.greedy(), SamplingConfig(temperature=0.9, top_k=20, seed=3)):
+        wait = generate(eng, Sampler(cfg, DEV), ps, 12, run_ahead=False)
+        stop = [wait[1].tokens[3], wait[4].tokens[0]]
+        for stops in ([], stop):
+            a = generate(eng, Sampler(cfg, DEV), ps, 12, stops, run_ahead=False)
+            b = generate(eng, Sampler(cfg, DEV), ps, 12, stops, run_ahead=True)
+            assert [(r.tokens, r.finish_reason) for r in a] == [(r.tokens, r.finish_reason) for r in b]
+            eng.cache.check()
+            assert not eng.cache.length
+
+
+def test_a_step_with_tokens_on_the_device(zoo):
+    from torchless_rs_amd.engine import SeqInput, StepError
+    DEV = "cuda:0"
+    eng, z = engine_for(zoo, "B", "float32"), zoo["B"]
+    V = z["cfg"]["vocab_size"]
+    ps = z["prompts"][:3]
+    slots = [eng.alloc() for _ in ps]
+    eng.step([SeqInput(s, p, []) for s, p in zip(slots, ps)])
+    toks = [5, 7, 11]
+    dev = torch.tensor([11, 99, 5, 7, V + 3], dtype=torch.int32, device=DEV)
+    a = eng.step([SeqInput(s, [0], [0]) for s in slots], device_tokens=dev, token_rows=[2, 3, 0]).clone()
+    for s in slots:
+        eng.free(s)
+    slots = [eng.alloc() for _ in ps]
+    eng.step([SeqInput(s, p, []) for s, p in zip(slots, ps)])
+    b = eng.step([SeqInput(s, [t], [0]) for s, t in zip(slots, toks)]).clone()
+    assert torch.equal(a, b)
+    c = eng.step([SeqInput(slots[0], [0], [0])], device_tokens=dev, token_rows=[4]).clone()    # outside the vocabulary: read as 0
+    for s in slots:
+        eng.free(s)
+    s0 = eng.alloc()
+    eng.step([SeqInput(s0, ps[0] + [toks[0]], [])])
+    assert torch.equal(c, eng.step([SeqInput(s0, [0], [0])]))
+    with pytest.raises(StepError, match="token_rows outside"):
+        eng.step([SeqInput(s0, [0], [0])], device_tokens=dev, token_rows=[5])
+    with pytest.raises(StepError, match="one token per entry"):
+        eng.step([SeqInput(s0, [0, 1], [0])], device_tokens=dev, token_rows=[0])
+    with pytest.raises(StepError, match="int32"):
+        eng.step([SeqInput(s0, [0], [0])], device_tokens=dev.long(), token_rows=[0])
+    eng.free(s0)
+    eng.cache.check()
+
+
 # ---- trace replay ----------------------------------------------------------------
 
 def replay(model_dir, dtype, lines, tmp, max_tokens=1024):

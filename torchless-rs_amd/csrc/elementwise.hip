@@ -291,6 +291,18 @@ __global__ void silu_mul_pairs_kernel(const bf16* __restrict__ gu, long long chu
   *reinterpret_cast<bf16x8*>(out + n * I + group * 32 + part * 8) = o;
 }
 
+// tokens[j] = src[idx[j]]: the ids that the sampler left on the device become the next step's
+// input without a trip to the host.  An id outside the vocabulary becomes 0 (no row of the
+// embedding lies there).
+__global__ void take_tokens_kernel(const int* __restrict__ src, const int* __restrict__ idx, int n,
+                                   int n_src, int vocab, int* __restrict__ tokens) {
+  const int j = blockIdx.x * blockDim.x + threadIdx.x;
+  if (j >= n) return;
+  const int r = idx[j];
+  const int t = (r >= 0 && r < n_src) ? src[r] : 0;
+  tokens[j] = (t >= 0 && t < vocab) ? t : 0;
+}
+
 __global__ void gather_rows_kernel(const float* __restrict__ x, const int* __restrict__ idx, int H,
                                    float* __restrict__ out) {
   const int m = blockIdx.x;
@@ -470,6 +482,14 @@ int tl_silu_mul_pairs(const void* gu, int n, int I, void* out, hipStream_t st) {
   TL_REQUIRE((chunks + 255) / 256 < 2147483647LL, "silu_mul_pairs: too many elements");
   silu_mul_pairs_kernel<<<(unsigned)((chunks + 255) / 256), 256, 0, st>>>((const bf16*)gu, chunks, I, (bf16*)out);
   TL_LAUNCH_CHECK("silu_mul_pairs");
+  return 0;
+}
+
+int tl_take_tokens(const int* src, const int* idx, int n, int n_src, int vocab, int* tokens, hipStream_t st) {
+  TL_REQUIRE(n >= 0 && n_src > 0 && vocab > 0, "take_tokens: bad sizes n=%d n_src=%d vocab=%d", n, n_src, vocab);
+  if (n == 0) return 0;
+  take_tokens_kernel<<<(n + 255) / 256, 256, 0, st>>>(src, idx, n, n_src, vocab, tokens);
+  TL_LAUNCH_CHECK("take_tokens");
   return 0;
 }
 

@@ -109,10 +109,13 @@ def _table_width(n_pages: int, ring_pages: int) -> int:
     return max(1, min(w, ring_pages))
 
 
-def pack_step(cache: Cache, batch: Sequence[SeqInput], vocab_size: int) -> PackedStep:
+def pack_step(cache: Cache, batch: Sequence[SeqInput], vocab_size: int,
+              token_rows: Optional[Sequence[int]] = None) -> PackedStep:
     """Check a step's entries, get their pages, and lay the batch out: tokens,
     row positions, row-to-sequence map, prefix sums, slots, lengths, wanted
-    rows and page tables in one array."""
+    rows and page tables in one array.  `token_rows` (one per entry, each entry
+    bringing one token): the tokens lie on the device, entry b's in row
+    token_rows[b] of a tensor given to the step; the indices go last in the array."""
     if not batch:
         raise StepError("a step needs at least one sequence")
     B = len(batch)
@@ -128,6 +131,10 @@ def pack_step(cache: Cache, batch: Sequence[SeqInput], vocab_size: int) -> Packe
                 raise StepError(f"entry {b}: wanted index {w} outside its {n_new[b]} tokens")
     N = int(n_new.sum())
     tokens = np.concatenate([np.asarray(s.tokens, dtype=np.int64) for s in batch])
+    if token_rows is not None:
+        if len(token_rows) != B or N != B:
+            raise StepError("tokens on the device: one row index per entry, and one token per entry")
+        tokens = np.zeros(B, dtype=np.int64)
     if tokens.min() < 0 or tokens.max() >= vocab_size:
         bad = int(tokens[(tokens < 0) | (tokens >= vocab_size)][0])
         raise StepError(f"token id {bad} is outside the vocabulary of {vocab_size}")
@@ -152,6 +159,8 @@ def pack_step(cache: Cache, batch: Sequence[SeqInput], vocab_size: int) -> Packe
     tile_off, aligned_cols = aligned_columns(len_before, n_new)
     parts = [tokens, row_pos, row_seq, cu, np.array([s.slot for s in batch]), len_before,
              len_after, want_rows, np.array(tile_off)] + [t.reshape(-1) for t in tables]
+    if token_rows is not None:
+        parts.append(np.asarray(token_rows, dtype=np.int64))
     return PackedStep(
         flat=np.concatenate(parts).astype(np.int32), sizes=[p.size for p in parts], n_rows=N, n_seqs=B,
         n_want=int(want_rows.size), strides=tuple(t.shape[1] for t in tables),
@@ -237,28 +246,53 @@ class Engine:
         return build_context(self.cache, batch, self.vocab_size, self.model.dtype, self.device,
                              self.workspace)
 
-    def step(self, batch: Sequence[SeqInput]) -> torch.Tensor:
+    def step(self, batch: Sequence[SeqInput], device_tokens: Optional[torch.Tensor] = None,
+             token_rows: Optional[Sequence[int]] = None) -> torch.Tensor:
         """Run one step; returns float32 logits [number of wanted rows, V] in
         the order of the entries and of their `want` lists.  The tensor is a
         view of the engine's workspace: it is overwritten by a later step.
 
+        `device_tokens` (int32 on the GPU, e.g. what the sampler just drew) with
+        `token_rows`: every entry brings one token, entry b's is
+        device_tokens[token_rows[b]] (the entries' own `tokens` are ignored), so
+        that a step can be launched before the host has seen the last one's
+        tokens.  Ids outside the vocabulary are read as 0.
+
         Steps in which every sequence brings one token are launch-bound; the
         second time a shape of such a step (batch size, page-table widths) is
         seen it is captured as a HIP graph, and from then on replayed."""
-        packed = pack_step(self.cache, batch, self.vocab_size)
+        if device_tokens is not None:
+            if token_rows is None:
+                token_rows = list(range(len(batch)))
+            if device_tokens.dtype != torch.int32 or not device_tokens.is_cuda or not device_tokens.is_contiguous():
+                raise StepError("device_tokens must be a contiguous int32 tensor on the GPU")
+            if any(not (0 <= r < device_tokens.numel()) for r in token_rows):
+                raise StepError(f"token_rows outside the {device_tokens.numel()} tokens on the device")
+        elif token_rows is not None:
+            raise StepError("token_rows without device_tokens")
+        packed = pack_step(self.cache, batch, self.vocab_size, token_rows)
         growth = [(s.slot, len(s.tokens)) for s in batch]
         if self.use_graphs and packed.all_single and self.model.graph_safe:
-            logits = self._graph_step(packed)
+            logits = self._graph_step(packed, device_tokens)
         else:
             dev = torch.from_numpy(packed.flat).to(self.device, non_blocking=False)
+            self._take_tokens(packed, dev, device_tokens)
             ctx, want_rows, n_want = context_from(packed, dev, self.cache, self.model.dtype,
                                                   self.device, self.workspace)
             logits = self.model.forward(ctx, self.runs, want_rows, n_want)
         self.cache.commit(growth)
         return logits
 
-    def _graph_step(self, packed: PackedStep) -> torch.Tensor:
-        key = packed.key
+    def _take_tokens(self, packed: PackedStep, dev: torch.Tensor, device_tokens: Optional[torch.Tensor]) -> None:
+        """Fill the token section of the uploaded array from tokens on the device."""
+        if device_tokens is None:
+            return
+        from ..kernels import ops
+        B = packed.n_seqs
+        ops.take_tokens(device_tokens, dev[dev.numel() - B:], self.vocab_size, dev[:B])
+
+    def _graph_step(self, packed: PackedStep, device_tokens: Optional[torch.Tensor] = None) -> torch.Tensor:
+        key = packed.key + (device_tokens is not None,)
         g = self._graphs.get(key)
         if g is None:
             # first sight: run it as it is, in the workspace the graph will own, so that
@@ -276,6 +310,7 @@ class Engine:
         if g.uploaded is None:
             g.uploaded = torch.cuda.Event()
         g.uploaded.record()
+        self._take_tokens(packed, g.meta, device_tokens)
         if g.graph is None and g.logits is not None:
             ctx, want_rows, n_want = context_from(packed, g.meta, self.cache, self.model.dtype,
                                                   self.device, g.workspace)

@@ -11,8 +11,8 @@ and gives its slot back while the others go on; when a batch is done the next
 requests take the freed slots, until every request is served.
 
 The loop touches the engine only through `alloc`, `free`, `step` and
-`fits`, and the sampler through `sample`, so its decisions can be tested
-without a GPU.
+`fits`, and the sampler through `sample` (or `draw`), so its decisions can be
+tested without a GPU.
 """
 from __future__ import annotations
 
@@ -57,10 +57,18 @@ def plan_batches(n_tokens_needed: Sequence[int], fits: Callable[[List[int]], boo
 
 def generate(engine, sampler, prompts: Sequence[Sequence[int]], max_tokens: int,
              stop_ids: Sequence[int] = (), max_batch: Optional[int] = None,
-             on_token: Optional[Callable[[int, int], None]] = None) -> List[GenerationResult]:
+             on_token: Optional[Callable[[int, int], None]] = None,
+             run_ahead: Optional[bool] = None) -> List[GenerationResult]:
     """Generate for every prompt; results come back in the order of the
     prompts.  `on_token(request, token)` is called for each token as it is
-    produced."""
+    produced.
+
+    `run_ahead` (default: if the sampler can `draw`): the next step is launched
+    with the drawn tokens still on the device, before the host has read them, so
+    that the GPU does not wait while the host looks at tokens and prepares a
+    step.  A sequence whose token turns out to be a stop id has then run one
+    row too many; the row is dropped with the sequence.  The tokens are the
+    same either way."""
     for i, p in enumerate(prompts):
         if len(p) < 1:
             raise ValueError(f"prompt {i} is empty; a prompt needs at least one token")
@@ -70,29 +78,58 @@ def generate(engine, sampler, prompts: Sequence[Sequence[int]], max_tokens: int,
         for r in results:
             r.finish_reason = "length"
         return results
+    if run_ahead is None:
+        run_ahead = hasattr(sampler, "draw")
     need = [len(p) + max_tokens - 1 for p in prompts]        # the last token is never fed
+
+    def accept(i: int, t: int) -> bool:
+        """Book request i's token; is the request finished?"""
+        r = results[i]
+        if t in stop:
+            r.finish_reason = "stop"
+        else:
+            r.tokens.append(t)
+            if on_token is not None:
+                on_token(i, t)
+            if len(r.tokens) >= max_tokens:
+                r.finish_reason = "length"
+        return bool(r.finish_reason)
+
     for batch in plan_batches(need, engine.fits, max_batch):
         slots = {i: engine.alloc() for i in batch}
         live = list(batch)
-        feed = {i: list(prompts[i]) for i in batch}
-        while live:
-            logits = engine.step([SeqInput(slots[i], feed[i], [len(feed[i]) - 1]) for i in live])
-            ids = sampler.sample(logits, live, [len(results[i].tokens) for i in live])
-            nxt = []
-            for i, t in zip(live, ids):
-                r = results[i]
-                if t in stop:
-                    r.finish_reason = "stop"
-                else:
-                    r.tokens.append(t)
-                    if on_token is not None:
-                        on_token(i, t)
-                    if len(r.tokens) >= max_tokens:
-                        r.finish_reason = "length"
-                if r.finish_reason:
+        logits = engine.step([SeqInput(slots[i], list(prompts[i]), [len(prompts[i]) - 1]) for i in live])
+        if not run_ahead:
+            while True:
+                ids = sampler.sample(logits, live, [len(results[i].tokens) for i in live])
+                nxt, feed = [], {}
+                for i, t in zip(live, ids):
+                    if accept(i, t):
+                        engine.free(slots.pop(i))
+                    else:
+                        feed[i] = [t]
+                        nxt.append(i)
+                live = nxt
+                if not live:
+                    break
+                logits = engine.step([SeqInput(slots[i], feed[i], [0]) for i in live])
+            continue
+        # run ahead: `order` are the requests whose tokens `drawn` holds (row by row); those of
+        # them that are not known to be finished go into the next step at once
+        order = live
+        drawn = sampler.draw(logits, order, [len(results[i].tokens) for i in order])
+        while order:
+            # a request that is alive and whose budget this token does not use up goes on, unless
+            # the token is a stop id, which the host does not know yet
+            ahead = [i for i in order if i in slots and len(results[i].tokens) + 1 < max_tokens]
+            nxt_drawn = None
+            if ahead:
+                rows = [order.index(i) for i in ahead]
+                logits = engine.step([SeqInput(slots[i], [0], [0]) for i in ahead],
+                                     device_tokens=drawn.device, token_rows=rows)
+                nxt_drawn = sampler.draw(logits, ahead, [len(results[i].tokens) + 1 for i in ahead])
+            for i, t in zip(order, drawn.tokens()):
+                if i in slots and accept(i, t):           # (a request dropped earlier: its row ran for nothing)
                     engine.free(slots.pop(i))
-                else:
-                    feed[i] = [t]
-                    nxt.append(i)
-            live = nxt
+            order, drawn = ahead, nxt_drawn
     return results

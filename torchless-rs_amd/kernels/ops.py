@@ -178,6 +178,15 @@ def silu_mul_pairs(gu: torch.Tensor, out: torch.Tensor) -> None:
     _check(lib().tl_silu_mul_pairs(_p(gu), n, I2 // 2, _p(out), _stream()))
 
 
+def take_tokens(src: torch.Tensor, idx: torch.Tensor, vocab: int, tokens: torch.Tensor) -> None:
+    """tokens[j] = src[idx[j]] (int32, on the device); ids outside [0, vocab) become 0."""
+    n = tokens.shape[0]
+    _req(src, "take_tokens.src", torch.int32)
+    _req(idx, "take_tokens.idx", torch.int32, (n,))
+    _req(tokens, "take_tokens.tokens", torch.int32, (n,))
+    _check(lib().tl_take_tokens(_p(src), _p(idx), n, src.numel(), int(vocab), _p(tokens), _stream()))
+
+
 def gather_rows(x: torch.Tensor, idx: torch.Tensor, out: torch.Tensor) -> None:
     m, H = idx.shape[0], x.shape[1]
     _req(x, "gather.x", torch.float32)

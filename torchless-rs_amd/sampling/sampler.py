@@ -13,6 +13,18 @@ from ..kernels import ops
 from .config import SamplingConfig
 
 
+class Drawn:
+    """The tokens of one draw: on the device at once (`device`, int32 [B], valid until the
+    sampler's next draw has been launched), on the host when `tokens()` is asked for."""
+
+    def __init__(self, device: torch.Tensor, host: torch.Tensor, done: "torch.cuda.Event"):
+        self.device, self._host, self._done = device, host, done
+
+    def tokens(self) -> List[int]:
+        self._done.synchronize()
+        return self._host.tolist()
+
+
 class Sampler:
     def __init__(self, config: SamplingConfig, device):
         self.config = config
@@ -22,15 +34,20 @@ class Sampler:
         self._counters = None
         self._out = None
         self._uploaded = None
+        self._host = None                # two pinned buffers for the tokens, used in turn
+        self._turn = 0
 
-    def sample(self, logits: torch.Tensor, seq_ids: Sequence[int], steps: Sequence[int]) -> List[int]:
-        """logits: float32 [B, V] on the GPU -> B token ids."""
+    def draw(self, logits: torch.Tensor, seq_ids: Sequence[int], steps: Sequence[int]) -> Drawn:
+        """logits: float32 [B, V] on the GPU -> B token ids, without waiting for them: the
+        kernel and the copy to the host are launched, `Drawn.tokens()` waits."""
         B, V = logits.shape
         c = self.config
         if self._stage is None or self._stage.shape[0] < B:
-            self._stage = torch.empty((max(B, 64), 2), dtype=torch.int32).pin_memory()
-            self._counters = torch.empty((max(B, 64), 2), dtype=torch.int32, device=logits.device)
-            self._out = torch.empty((max(B, 64),), dtype=torch.int32, device=logits.device)
+            cap = max(B, 64)
+            self._stage = torch.empty((cap, 2), dtype=torch.int32).pin_memory()
+            self._counters = torch.empty((cap, 2), dtype=torch.int32, device=logits.device)
+            self._out = torch.empty((cap,), dtype=torch.int32, device=logits.device)
+            self._host = [torch.empty((cap,), dtype=torch.int32).pin_memory() for _ in range(2)]
             self._uploaded = None
         if self._uploaded is not None:
             self._uploaded.synchronize()             # the pinned pairs are free to be written again
@@ -47,7 +64,16 @@ class Sampler:
         out = self._out[:B]
         ops.sample(logits.contiguous(), float(c.temperature), int(c.top_k or 0), float(c.top_p or 0.0),
                    int(c.seed), counters, self._probs[:B], out)
-        return out.tolist()
+        host = self._host[self._turn][:B]
+        self._turn ^= 1
+        host.copy_(out, non_blocking=True)
+        done = torch.cuda.Event()
+        done.record()
+        return Drawn(out, host, done)
+
+    def sample(self, logits: torch.Tensor, seq_ids: Sequence[int], steps: Sequence[int]) -> List[int]:
+        """logits: float32 [B, V] on the GPU -> B token ids."""
+        return self.draw(logits, seq_ids, steps).tokens()
 
     def last_distribution(self, B: int) -> torch.Tensor:
         """The probabilities the last draw was made from (temperature > 0)."""
