@@ -1,6 +1,7 @@
 """Decode and prefill throughput of the Mistral-7B-v0.1 shape on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 8192] [--layers L]
+                    [--shape 7b-v0.1|7b-v0.3|nemo-12b]
 
 One JSON line: decoded tokens a second of the default run (batch 8 at the
 context length of the configuration), the prefill of one 2,048-token prompt,
@@ -21,10 +22,17 @@ sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 HBM_PEAK_GBS = 8000.0                 # MI355X, published
 PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}
 
-# Mistral-7B-v0.1 shape: the third configuration of the baseline
+# Mistral-7B-v0.1 shape: the third configuration of the baseline, and the default
 SHAPE = dict(num_hidden_layers=32, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8,
              head_dim=128, intermediate_size=14336, vocab_size=32000, rope_theta=10000.0,
              sliding_window=4096, rms_norm_eps=1e-5)
+# the baseline's other shapes of the same architecture, for --shape
+SHAPES = {
+    "7b-v0.1": ("Mistral-7B-v0.1 shape", SHAPE),
+    "7b-v0.3": ("Mistral-7B-v0.3 shape", dict(SHAPE, vocab_size=32768, rope_theta=1e6, sliding_window=None)),
+    "nemo-12b": ("Mistral-NeMo-12B shape", dict(SHAPE, num_hidden_layers=40, hidden_size=5120, vocab_size=131072,
+                                                 rope_theta=1e6, sliding_window=None)),
+}
 
 
 def main() -> int:
@@ -34,7 +42,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=4)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=8192)
-    ap.add_argument("--layers", type=int, default=SHAPE["num_hidden_layers"])
+    ap.add_argument("--shape", choices=sorted(SHAPES), default="7b-v0.1")
+    ap.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64")
     ap.add_argument("--only", choices=["prefill", "decode"], default=None,
@@ -51,7 +60,10 @@ def main() -> int:
     from torchless_rs_amd.sampling.sampler import Sampler
     from torchless_rs_amd.weights import random_tensors
 
-    cfgd = dict(SHAPE, architectures=["MistralForCausalLM"], num_hidden_layers=args.layers)
+    shape_name, shape = SHAPES[args.shape]
+    if args.layers is None:
+        args.layers = shape["num_hidden_layers"]
+    cfgd = dict(shape, architectures=["MistralForCausalLM"], num_hidden_layers=args.layers)
     cfg = config_from_dict(cfgd)
     dev = "cuda:0"
     t0 = time.time()
@@ -155,12 +167,13 @@ def main() -> int:
             print(f"[bench] decode b{b}: {b / s_b:.1f} tok/s", file=sys.stderr, flush=True)
 
     out = {
-        "metric": "decode tok/s at batch 8 (Mistral-7B-v0.1 shape), with prefill tok/s at 2,048 tokens",
+        "metric": f"decode tok/s at batch {args.batch} ({shape_name}), with prefill tok/s at "
+                  f"{args.prefill_tokens:,} tokens",
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(sec * 1e3, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic: random weights N(0,0.02) seed 5, uniform random token ids",
-        "config": {"model": "Mistral-7B-v0.1 shape", "layers": L, "layers_of_config": 32,
+        "config": {"model": shape_name, "layers": L, "layers_of_config": shape["num_hidden_layers"],
                    "hidden_size": H, "heads": nq, "kv_heads": nkv, "head_dim": d,
                    "intermediate_size": I, "vocab_size": V, "sliding_window": W,
                    "rope_theta": cfg.rope_theta, "rms_norm_eps": cfg.rms_norm_eps,
