@@ -48,8 +48,11 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
   bf16* Ks = reinterpret_cast<bf16*>(smem);          // [PF_BN][KLD]
   bf16* Vt = Ks + PF_BN * KLD;                       // [DPAD][PF_VLD]
 
-  // which sequence and which block of its rows; late blocks (most keys) first
-  int t = gridDim.x - 1 - blockIdx.x, b = 0;
+  // Which sequence and which block of its rows.  All workgroups of a step are usually resident
+  // at once, two a compute unit, and a late block has many times the keys of an early one: the
+  // first half of the heads takes the blocks from the last to the first, the second half from
+  // the first to the last, so that the two that meet on a compute unit have about the same sum.
+  int t = (blockIdx.y < (gridDim.y + 1) / 2) ? gridDim.x - 1 - blockIdx.x : blockIdx.x, b = 0;
   for (; b < B; ++b) {
     const int tiles = (cu_seqlens[b + 1] - cu_seqlens[b] + PF_BM - 1) / PF_BM;
     if (t < tiles) break;
