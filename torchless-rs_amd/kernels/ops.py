@@ -460,11 +460,13 @@ def aligned_columns(n_cached, n_new):
     """Column offsets (and their total) at which sequences lie when each is
     given room from the last multiple of 64 below its cached length up to its
     end, rounded up to 64: positions that are multiples of 64 then lie on
-    columns that are."""
+    columns that are.  The total is the row length of buffers laid out so."""
     off, total = [], 0
     for c, n in zip(n_cached, n_new):
         off.append(total)
         total += -(-((int(c) % 64) + int(n)) // 64) * 64
+    if total % 512 == 0:
+        total += 64          # rows a power of two apart would all fall on the same memory channels
     return off, total
 
 
