@@ -18,6 +18,9 @@ writes row `pos` of every layer as it goes (src/model/mod.rs:201-209).  Here
 Stale rows are never cleared: what a query may see is decided by the
 sequence's length and the window, as in the reference, where a reset only
 sets `pos = 0`.
+
+The books are kept in C++ by the host library; the classes here are its
+face and own the device storage.
 """
 from __future__ import annotations
 
@@ -26,7 +29,12 @@ from typing import Dict, List, Optional, Tuple
 
 import torch
 
-from .pool import CacheFull, CacheMisuse, FreeList
+import ctypes
+
+import numpy as np
+
+from . import native
+from .native import CacheFull, CacheMisuse      # noqa: F401
 
 PAGE = 64
 NO_RING = 1 << 24          # "ring" of a group that keeps every position: never wraps
@@ -51,19 +59,105 @@ def pages_for(n_tokens: int) -> int:
     return (n_tokens + PAGE - 1) // PAGE
 
 
+def _ints(values) -> np.ndarray:
+    return np.ascontiguousarray(np.asarray(values, dtype=np.int32))
+
+
+class _Pool:
+    """What is free and held of a group's pages (the books are the host library's)."""
+
+    def __init__(self, cache: "Cache", group: int, n: int):
+        self._c, self._g, self.n = cache, group, n
+
+    @property
+    def n_free(self) -> int:
+        return native.lib().tl_books_free_pages(self._c._h, self._g)
+
+    @property
+    def n_held(self) -> int:
+        return self.n - self.n_free
+
+    def holds(self, page: int) -> bool:
+        return bool(native.lib().tl_books_page_held(self._c._h, self._g, int(page)))
+
+
+class _Slots:
+    def __init__(self, cache: "Cache", n: int):
+        self._c, self.n = cache, n
+
+    @property
+    def n_free(self) -> int:
+        return native.lib().tl_books_free_slots(self._c._h)
+
+    @property
+    def n_held(self) -> int:
+        return self.n - self.n_free
+
+    def holds(self, slot: int) -> bool:
+        return bool(native.lib().tl_books_holds(self._c._h, int(slot)))
+
+
+class _PagesOfSlot:
+    """group.pages_of_slot[slot] -> the slot's pages, in the order of the ring (a copy)."""
+
+    def __init__(self, cache: "Cache", group: int):
+        self._c, self._g = cache, group
+
+    def __getitem__(self, slot: int) -> List[int]:
+        buf = np.empty(self._c.n_pages, dtype=np.int32)
+        n = native.lib().tl_books_pages(self._c._h, self._g, int(slot), buf.ctypes.data, buf.size)
+        if n < 0:
+            raise KeyError(slot)
+        return buf[:n].tolist()
+
+    def __contains__(self, slot: int) -> bool:
+        return self._c.slots.holds(slot)
+
+    def __iter__(self):
+        return iter(self._c.held_slots())
+
+    def __len__(self) -> int:
+        return len(self._c.held_slots())
+
+
+class _Lengths:
+    """cache.length[slot] -> positions the slot holds; behaves as a read-only dict."""
+
+    def __init__(self, cache: "Cache"):
+        self._c = cache
+
+    def __getitem__(self, slot: int) -> int:
+        n = native.lib().tl_books_length(self._c._h, int(slot))
+        if n < 0:
+            raise KeyError(slot)
+        return n
+
+    def __contains__(self, slot: int) -> bool:
+        return self._c.slots.holds(slot)
+
+    def __iter__(self):
+        return iter(self._c.held_slots())
+
+    def __len__(self) -> int:
+        return self._c.max_slots - self._c.slots.n_free
+
+    def values(self):
+        return [self[s] for s in self._c.held_slots()]
+
+
 class KVGroup:
     """Storage of the runs that share one `KVRequest`."""
 
-    def __init__(self, request: KVRequest, runs: List[int], n_pages: int, dtype, device,
-                 allocate: bool):
+    def __init__(self, cache: "Cache", index: int, request: KVRequest, runs: List[int], n_pages: int, dtype,
+                 device, allocate: bool):
         self.request = request
         self.runs = list(runs)
         self.layer_of_run = {r: i for i, r in enumerate(self.runs)}
         self.n_pages = n_pages
         # pages one sequence can hold: a ring for a window, else without bound (the pool is the limit)
         self.ring_pages = pages_for(request.window) if request.window else NO_RING
-        self.pool = FreeList(n_pages, "page")
-        self.pages_of_slot: Dict[int, List[int]] = {}
+        self.pool = _Pool(cache, index, n_pages)
+        self.pages_of_slot = _PagesOfSlot(cache, index)
         self.storage = None
         if allocate:
             # [layer, page, K|V, kv_head, row, head_dim]
@@ -76,8 +170,9 @@ class KVGroup:
 
 
 class Cache:
-    """Slots, pages and state.  All bookkeeping is on the host and can be used
-    without a device (`allocate=False`)."""
+    """Slots, pages and state.  The books (who holds what) are kept by the host
+    library (csrc/host/books.cpp) and can be used without a device
+    (`allocate=False`)."""
 
     def __init__(self, kv_requests: Dict[int, KVRequest], state_requests: Dict[int, StateRequest],
                  max_tokens: int, dtype=torch.bfloat16, device="cpu", max_slots: Optional[int] = None,
@@ -88,13 +183,18 @@ class Cache:
         self.max_slots = int(max_slots) if max_slots else self.n_pages
         self.dtype = dtype
         self.device = device
-        self.slots = FreeList(self.max_slots, "slot")
-        self.length: Dict[int, int] = {}
         by_req: Dict[KVRequest, List[int]] = {}
         for run in sorted(kv_requests):
             by_req.setdefault(kv_requests[run], []).append(run)
+        self._h = None
         self.groups: List[KVGroup] = [
-            KVGroup(req, runs, self.n_pages, dtype, device, allocate) for req, runs in by_req.items()]
+            KVGroup(self, gi, req, runs, self.n_pages, dtype, device, allocate)
+            for gi, (req, runs) in enumerate(by_req.items())]
+        rings, pages = _ints([g.ring_pages for g in self.groups]), _ints([g.n_pages for g in self.groups])
+        self._h = ctypes.c_void_p(native.lib().tl_books_new(self.max_slots, len(self.groups),
+                                                            rings.ctypes.data, pages.ctypes.data))
+        self.slots = _Slots(self, self.max_slots)
+        self.length = _Lengths(self)
         self.group_of_run: Dict[int, int] = {
             r: gi for gi, g in enumerate(self.groups) for r in g.runs}
         self.state: Dict[int, Optional[torch.Tensor]] = {}
@@ -103,63 +203,44 @@ class Cache:
             self.state[run] = torch.zeros((self.max_slots,) + tuple(req.shape), dtype=req.dtype,
                                           device=device) if allocate else None
 
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h:
+            native.lib().tl_books_delete(h)
+
     # ---- slots -----------------------------------------------------------
     def alloc_slot(self) -> int:
-        s = self.slots.take()
-        self.length[s] = 0
-        for g in self.groups:
-            g.pages_of_slot[s] = []
+        out = ctypes.c_int(-1)
+        native.check(native.lib().tl_books_alloc_slot(self._h, ctypes.byref(out)))
+        s = out.value
         for run, t in self.state.items():
             if t is not None:
                 t[s].zero_()
         return s
 
     def free_slot(self, slot: int) -> None:
-        self.slots.give_back(slot)
-        for g in self.groups:
-            for p in g.pages_of_slot.pop(slot):
-                g.pool.give_back(p)
-        del self.length[slot]
+        native.check(native.lib().tl_books_free_slot(self._h, int(slot)))
 
-    def _held(self, slot: int) -> None:
-        if not self.slots.holds(slot):
-            raise CacheMisuse(f"slot {slot} is not held")
+    def held_slots(self) -> List[int]:
+        buf = np.empty(self.max_slots, dtype=np.int32)
+        n = native.lib().tl_books_held_slots(self._h, buf.ctypes.data, buf.size)
+        return buf[:n].tolist()
 
     # ---- growth ----------------------------------------------------------
     def prepare(self, growth: List[Tuple[int, int]]) -> None:
         """Make room for `n_new` more positions in each `(slot, n_new)`.
         Either every sequence gets its pages or none is changed."""
-        need = [0] * len(self.groups)
-        seen = set()
-        for slot, n_new in growth:
-            self._held(slot)
-            if slot in seen:
-                raise CacheMisuse(f"slot {slot} appears twice in one step")
-            seen.add(slot)
-            if n_new < 1:
-                raise ValueError(f"slot {slot}: a step must bring at least one token")
-            for gi, g in enumerate(self.groups):
-                need[gi] += g.pages_needed(self.length[slot] + n_new) - len(g.pages_of_slot[slot])
-        for gi, g in enumerate(self.groups):
-            if need[gi] > g.pool.n_free:
-                raise CacheFull(
-                    f"the step needs {need[gi]} more pages of {PAGE} positions, {g.pool.n_free} of "
-                    f"{g.n_pages} are free; raise max_tokens")
-        for slot, n_new in growth:
-            for g in self.groups:
-                pages = g.pages_of_slot[slot]
-                while len(pages) < g.pages_needed(self.length[slot] + n_new):
-                    pages.append(g.pool.take())
+        slots, n_new = _ints([g[0] for g in growth]), _ints([g[1] for g in growth])
+        native.check(native.lib().tl_books_prepare(self._h, len(growth), slots.ctypes.data, n_new.ctypes.data))
 
     def fits(self, lengths: List[int]) -> bool:
         """Would new sequences of these final lengths find slots and pages now?"""
-        if len(lengths) > self.slots.n_free:
-            return False
-        return all(sum(g.pages_needed(n) for n in lengths) <= g.pool.n_free for g in self.groups)
+        ls = np.ascontiguousarray(np.asarray(lengths, dtype=np.int64))
+        return bool(native.lib().tl_books_fits(self._h, len(lengths), ls.ctypes.data))
 
     def commit(self, growth: List[Tuple[int, int]]) -> None:
-        for slot, n_new in growth:
-            self.length[slot] += n_new
+        slots, n_new = _ints([g[0] for g in growth]), _ints([g[1] for g in growth])
+        native.check(native.lib().tl_books_commit(self._h, len(growth), slots.ctypes.data, n_new.ctypes.data))
 
     # ---- views for kernels -------------------------------------------------
     def kv_layer(self, run: int) -> Tuple[KVGroup, int]:
@@ -173,15 +254,4 @@ class Cache:
 
     def check(self) -> None:
         """Invariants: no page or slot lost, held twice, or both free and held."""
-        self.slots.check()
-        for g in self.groups:
-            g.pool.check()
-            held = [p for pages in g.pages_of_slot.values() for p in pages]
-            assert len(held) == len(set(held)), "a page is held by two sequences"
-            assert len(held) == g.pool.n_held, "a page is held by no sequence"
-            for p in held:
-                assert g.pool.holds(p)
-            assert set(g.pages_of_slot) == set(self.length), "slots and page lists differ"
-            for s, pages in g.pages_of_slot.items():
-                assert len(pages) == g.pages_needed(self.length[s]) or \
-                    len(pages) >= g.pages_needed(self.length[s])
+        native.check(native.lib().tl_books_check(self._h))

@@ -11,6 +11,7 @@ the rows asked for.  A sequence's result does not depend on its batch-mates.
 """
 from __future__ import annotations
 
+import ctypes
 import gc
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Sequence, Tuple
@@ -25,9 +26,7 @@ from ..weights.safetensors_io import ModelFiles, TensorDict
 from .model import Model
 
 
-class StepError(ValueError):
-    """A step that cannot be run as asked (unknown slot, token id outside the
-    vocabulary, empty batch, ...)."""
+from ..cache.native import StepError        # noqa: E402  (raised by the host library's packer too)
 
 
 @dataclass
@@ -100,74 +99,59 @@ class PackedStep:
         return (self.n_seqs, self.n_rows, self.n_want, self.strides)
 
 
-def _table_width(n_pages: int, ring_pages: int) -> int:
-    """Width of a step's page table: the next power of two, so that it (and
-    what is derived from it) changes rarely while sequences grow."""
-    w = 1
-    while w < n_pages:
-        w *= 2
-    return max(1, min(w, ring_pages))
-
-
 def pack_step(cache: Cache, batch: Sequence[SeqInput], vocab_size: int,
               token_rows: Optional[Sequence[int]] = None) -> PackedStep:
     """Check a step's entries, get their pages, and lay the batch out: tokens,
     row positions, row-to-sequence map, prefix sums, slots, lengths, wanted
-    rows and page tables in one array.  `token_rows` (one per entry, each entry
-    bringing one token): the tokens lie on the device, entry b's in row
-    token_rows[b] of a tensor given to the step; the indices go last in the array."""
-    if not batch:
-        raise StepError("a step needs at least one sequence")
+    rows, aligned column offsets and page tables in one array (the work is the
+    host library's `tl_pack_step`).  A page table's width is the next power of
+    two, so that it changes rarely while sequences grow.  `token_rows` (one per
+    entry, each entry bringing one token): the tokens lie on the device, entry
+    b's in row token_rows[b] of a tensor given to the step; the indices go last
+    in the array."""
+    from ..cache import native
     B = len(batch)
-    n_new = np.zeros(B, dtype=np.int64)
-    for b, s in enumerate(batch):
-        if not cache.slots.holds(s.slot):
-            raise StepError(f"entry {b}: slot {s.slot} is not held")
-        n_new[b] = len(s.tokens)
-        if n_new[b] < 1:
-            raise StepError(f"entry {b}: a sequence must bring at least one token")
-        for w in s.want:
-            if not (0 <= w < n_new[b]):
-                raise StepError(f"entry {b}: wanted index {w} outside its {n_new[b]} tokens")
-    N = int(n_new.sum())
-    tokens = np.concatenate([np.asarray(s.tokens, dtype=np.int64) for s in batch])
+    if not B:
+        raise StepError("a step needs at least one sequence")
+    slots = np.fromiter((s.slot for s in batch), dtype=np.int32, count=B)
+    n_new = np.fromiter((len(s.tokens) for s in batch), dtype=np.int32, count=B)
+    n_want = np.fromiter((len(s.want) for s in batch), dtype=np.int32, count=B)
+    N, NW = int(n_new.sum()), int(n_want.sum())
+    try:
+        tokens = np.fromiter((t for s in batch for t in s.tokens), dtype=np.int64, count=N)
+        want = np.fromiter((w for s in batch for w in s.want), dtype=np.int64, count=NW)
+    except (TypeError, ValueError) as e:
+        raise StepError(f"tokens and wanted indices must be integers ({e})") from None
+    if N and token_rows is None and (tokens.min() < -2 ** 31 or tokens.max() >= 2 ** 31):
+        raise StepError(f"token id {int(tokens.max())} is outside the vocabulary of {vocab_size}")
+    tokens, want = tokens.astype(np.int32), np.clip(want, -1, 2 ** 31 - 1).astype(np.int32)
+    rows = None
     if token_rows is not None:
-        if len(token_rows) != B or N != B:
+        if len(token_rows) != B:
             raise StepError("tokens on the device: one row index per entry, and one token per entry")
-        tokens = np.zeros(B, dtype=np.int64)
-    if tokens.min() < 0 or tokens.max() >= vocab_size:
-        bad = int(tokens[(tokens < 0) | (tokens >= vocab_size)][0])
-        raise StepError(f"token id {bad} is outside the vocabulary of {vocab_size}")
-    growth = [(s.slot, int(n)) for s, n in zip(batch, n_new)]
-    len_before = np.array([cache.length[s.slot] for s in batch], dtype=np.int64)
-    cache.prepare(growth)                       # raises CacheFull / CacheMisuse untouched
-    len_after = len_before + n_new
-    cu = np.zeros(B + 1, dtype=np.int64)
-    np.cumsum(n_new, out=cu[1:])
-    row_seq = np.repeat(np.arange(B), n_new)
-    row_pos = np.arange(N) - cu[row_seq] + len_before[row_seq]
-    want_rows = np.array([cu[b] + w for b, s in enumerate(batch) for w in s.want], dtype=np.int64)
-    tables = []
-    for g in cache.groups:
-        stride = _table_width(max(len(g.pages_of_slot[s.slot]) for s in batch), g.ring_pages)
-        t = np.zeros((B, stride), dtype=np.int64)
-        for b, s in enumerate(batch):
-            pg = g.pages_of_slot[s.slot]
-            t[b, :len(pg)] = pg
-        tables.append(t)
-    from ..kernels.ops import aligned_columns
-    tile_off, aligned_cols = aligned_columns(len_before, n_new)
-    parts = [tokens, row_pos, row_seq, cu, np.array([s.slot for s in batch]), len_before,
-             len_after, want_rows, np.array(tile_off)] + [t.reshape(-1) for t in tables]
-    if token_rows is not None:
-        parts.append(np.asarray(token_rows, dtype=np.int64))
+        rows = np.ascontiguousarray(np.asarray(token_rows, dtype=np.int32))
+    G = len(cache.groups)
+    cap = 3 * N + (B + 1) + 5 * B + NW + B * sum(min(g.ring_pages, max(1, 2 * cache.n_pages)) for g in cache.groups)
+    flat = np.empty(cap, dtype=np.int32)
+    sizes = np.zeros(12 + G, dtype=np.int32)
+    info = np.zeros(8 + G, dtype=np.int64)
+    n_out = ctypes.c_long(0)
+    native.check(native.lib().tl_pack_step(
+        cache._h, B, slots.ctypes.data, n_new.ctypes.data, tokens.ctypes.data, n_want.ctypes.data,
+        want.ctypes.data, int(vocab_size), rows.ctypes.data if rows is not None else None, flat.ctypes.data,
+        cap, sizes.ctypes.data, info.ctypes.data, ctypes.byref(n_out)))
+    pieces = int(info[6])
+    szs = sizes[:pieces].tolist()
+    off = np.concatenate([[0], np.cumsum(szs)])
+    flat = flat[:n_out.value]
+    len_before, len_after, cu = flat[off[5]:off[6]], flat[off[6]:off[7]], flat[off[3]:off[4]]
     return PackedStep(
-        flat=np.concatenate(parts).astype(np.int32), sizes=[p.size for p in parts], n_rows=N, n_seqs=B,
-        n_want=int(want_rows.size), strides=tuple(t.shape[1] for t in tables),
-        all_single=bool((n_new == 1).all()), max_new=int(n_new.max()),
-        max_len_after=int(len_after.max()),
-        host={"n_new": n_new, "len_before": len_before, "len_after": len_after, "cu": cu,
-              "slots": [s.slot for s in batch], "aligned_cols": aligned_cols})
+        flat=flat, sizes=szs, n_rows=int(info[0]), n_seqs=B, n_want=int(info[1]),
+        strides=tuple(int(w) for w in info[7:7 + G]), all_single=bool(info[2]), max_new=int(info[3]),
+        max_len_after=int(info[4]),
+        host={"n_new": n_new.astype(np.int64), "len_before": len_before.astype(np.int64),
+              "len_after": len_after.astype(np.int64), "cu": cu.astype(np.int64), "slots": slots.tolist(),
+              "aligned_cols": int(info[5])})
 
 
 def context_from(packed: PackedStep, dev: torch.Tensor, cache: Cache, dtype: torch.dtype, device,

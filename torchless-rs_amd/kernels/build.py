@@ -1,9 +1,11 @@
-"""Compiling the HIP sources for gfx950 into one shared library, and loading it.
+"""Compiling the sources into two shared libraries, and loading them: the HIP
+kernels for gfx950 (`libtorchless_hip.so`, hipcc) and the host side of cache
+and step (`libtorchless_host.so`, plain C++, no GPU needed).
 
-`build()` always compiles.  `load()` loads the library that is there and
-builds only if none is.  The library goes to `csrc/_build/` inside the
-package; if that cannot be written (a read-only checkout), to a folder of
-the user's own under the system's temporary directory.
+`build()` always compiles both.  `load()` and `load_host()` load the library
+that is there and build only if none is.  The libraries go to `csrc/_build/`
+inside the package; if that cannot be written (a read-only checkout), to a
+folder of the user's own under the system's temporary directory.
 """
 from __future__ import annotations
 
@@ -20,12 +22,14 @@ from typing import List, Optional
 
 ARCH = "gfx950"
 LIB_NAME = "libtorchless_hip.so"
+HOST_LIB_NAME = "libtorchless_host.so"
 _CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
 HIPCC_FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
                "-Wno-unused-result"]
 
 _lib: Optional[ctypes.CDLL] = None
+_host_lib: Optional[ctypes.CDLL] = None
 _lock = threading.Lock()
 
 
@@ -39,6 +43,36 @@ def _say(msg: str) -> None:
 
 def sources() -> List[str]:
     return sorted(os.path.join(_CSRC, f) for f in os.listdir(_CSRC) if f.endswith(".hip"))
+
+
+def host_sources() -> List[str]:
+    d = os.path.join(_CSRC, "host")
+    return sorted(os.path.join(d, f) for f in os.listdir(d) if f.endswith(".cpp"))
+
+
+def find_cxx() -> str:
+    for c in (os.environ.get("CXX"), shutil.which("g++"), shutil.which("c++"), shutil.which("clang++"),
+              "/opt/rocm/llvm/bin/clang++"):
+        if c and (os.path.isfile(c) or shutil.which(c)):
+            return c
+    raise ExtensionMissing("no C++ compiler found (looked at $CXX, g++, c++, clang++)")
+
+
+def build_host(verbose: bool = True) -> str:
+    """Compile the host library; returns its path."""
+    cxx = find_cxx()
+    out_dir = next((d for d in build_dirs() if _writable_dir(d)), None)
+    if out_dir is None:
+        raise ExtensionMissing(f"no writable build folder among {build_dirs()}")
+    lib = os.path.join(out_dir, HOST_LIB_NAME)
+    tmp = lib + f".tmp{os.getpid()}"
+    t0 = time.time()
+    _run_with_progress([cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", *host_sources(), "-o", tmp],
+                       "the host library")
+    os.replace(tmp, lib)
+    if verbose:
+        _say(f"built {lib} in {time.time() - t0:.0f} s")
+    return lib
 
 
 def _writable_dir(path: str) -> bool:
@@ -89,7 +123,8 @@ def _run_with_progress(cmd: List[str], what: str) -> None:
 
 
 def build(verbose: bool = True) -> str:
-    """Compile every source and link the library; returns its path."""
+    """Compile every source and link both libraries; returns the path of the kernels'."""
+    build_host(verbose)
     hipcc = find_hipcc()
     out_dir = next((d for d in build_dirs() if _writable_dir(d)), None)
     if out_dir is None:
@@ -117,18 +152,18 @@ def build(verbose: bool = True) -> str:
     return lib
 
 
-def built_library() -> Optional[str]:
+def built_library(name: str = LIB_NAME) -> Optional[str]:
     for d in build_dirs():
-        p = os.path.join(d, LIB_NAME)
+        p = os.path.join(d, name)
         if os.path.isfile(p):
             return p
     return None
 
 
-def _warn_if_stale(lib: str) -> None:
+def _warn_if_stale(lib: str, srcs: Optional[List[str]] = None) -> None:
     try:
-        newest = max(os.path.getmtime(os.path.join(_CSRC, f)) for f in os.listdir(_CSRC)
-                     if f.endswith((".hip", ".hpp")))
+        srcs = srcs or [os.path.join(_CSRC, f) for f in os.listdir(_CSRC) if f.endswith((".hip", ".hpp"))]
+        newest = max(os.path.getmtime(f) for f in srcs)
         if newest > os.path.getmtime(lib) + 1.0:
             _say(f"warning: a source is newer than {lib}; build again to pick it up")
     except OSError:
@@ -151,3 +186,21 @@ def load() -> ctypes.CDLL:
         except OSError as e:
             raise ExtensionMissing(f"cannot load {path}: {e}") from None
         return _lib
+
+
+def load_host() -> ctypes.CDLL:
+    """The host library, built first if there is none."""
+    global _host_lib
+    with _lock:
+        if _host_lib is not None:
+            return _host_lib
+        path = built_library(HOST_LIB_NAME)
+        if path is None:
+            path = build_host()
+        else:
+            _warn_if_stale(path, host_sources())
+        try:
+            _host_lib = ctypes.CDLL(path)
+        except OSError as e:
+            raise ExtensionMissing(f"cannot load {path}: {e}") from None
+        return _host_lib

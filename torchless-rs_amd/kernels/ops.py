@@ -460,14 +460,16 @@ def aligned_columns(n_cached, n_new):
     """Column offsets (and their total) at which sequences lie when each is
     given room from the last multiple of 64 below its cached length up to its
     end, rounded up to 64: positions that are multiples of 64 then lie on
-    columns that are.  The total is the row length of buffers laid out so."""
-    off, total = [], 0
-    for c, n in zip(n_cached, n_new):
-        off.append(total)
-        total += -(-((int(c) % 64) + int(n)) // 64) * 64
-    if total % 512 == 0:
-        total += 64          # rows a power of two apart would all fall on the same memory channels
-    return off, total
+    columns that are.  The total is the row length of buffers laid out so (kept
+    off multiples of 512: rows a power of two apart would all fall on the same
+    memory channels).  The rule is the host library's, which lays out steps."""
+    import numpy as np
+    from ..cache import native
+    c = np.ascontiguousarray(np.asarray(list(n_cached), dtype=np.int64))
+    n = np.ascontiguousarray(np.asarray(list(n_new), dtype=np.int64))
+    off = np.zeros(len(c), dtype=np.int32)
+    total = native.lib().tl_aligned_columns(len(c), c.ctypes.data, n.ctypes.data, off.ctypes.data)
+    return off.tolist(), int(total)
 
 
 def attn_prefill_bf16(q, k_new, vt_new, tile_off, pages, table, ring_pages: int, row_pos, cu_seqlens,
