@@ -161,6 +161,38 @@ def test_a_prompt_in_chunks_longer_than_the_ring(zoo, dtype):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", NAMES)
+def test_small_steps_of_several_tokens(zoo, name, dtype):
+    """Two sequences together in steps of 1 to 9 tokens each: at most 16 rows a step, where a
+    norm is cut in two around the products next to it, but not one token a sequence, so that
+    the part behind the norm sometimes has to ask for the plain norm."""
+    from torchless_rs_amd.engine import SeqInput
+    eng, z = engine_for(zoo, name, dtype), zoo[name]
+    a, b = z["prompts"][2][:17], z["prompts"][3][:30]
+    want = [plain.forward(z["w"], z["cfg"], p) for p in (a, b)]
+    sa, sb = eng.alloc(), eng.alloc()
+    got, fed = {sa: [], sb: []}, {sa: 0, sb: 0}
+    cuts = [(3, 7), (1, 1), (5, 9), (1, 2), (7, 1), (0, 8), (0, 2)]
+    for na, nb in cuts:
+        batch = []
+        for s, ids, n in ((sa, a, na), (sb, b, nb)):
+            part = ids[fed[s]:fed[s] + n]
+            if part:
+                batch.append(SeqInput(s, part, list(range(len(part)))))
+                fed[s] += len(part)
+        lg = eng.step(batch).clone()
+        r = 0
+        for e in batch:
+            got[e.slot].append(lg[r:r + len(e.tokens)])
+            r += len(e.tokens)
+    assert fed[sa] == len(a) and fed[sb] == len(b)
+    eng.free(sa)
+    eng.free(sb)
+    assert rel_err(torch.cat(got[sa]), want[0]) < TOL[dtype]
+    assert rel_err(torch.cat(got[sb]), want[1]) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
 def test_first_tokens(zoo, name, dtype):
     from torchless_rs_amd.engine import SeqInput
     eng, z = engine_for(zoo, name, dtype), zoo[name]
