@@ -1,16 +1,21 @@
 // bfloat16 products on the matrix cores, C[M,N] (+)= A[M,K] * W[N,K]^T, float
 // accumulation, weights row-major [out, in] as the checkpoint stores them.
 //
-//  * gemm_skinny: M <= 64 rows (decode).  The step is bound by reading W once
-//    from HBM, so W streams from global memory straight into MFMA operands:
-//    a workgroup owns 16*NT output channels, its 8 waves split K between them
-//    and every lane keeps several 16-byte loads in flight; the partial sums
-//    meet in LDS.  The activations are the other operand, read through the
-//    caches.  A row's result does not depend on M.
-//  * gemm_tiled: any M (prefill).  128x128x64 tiles staged through LDS,
-//    4 waves of 64x64, 32x32x16 MFMA, next tile prefetched into registers.
+//  * gemm_skinny: at most 16 rows a tile (decode).  The step is bound by reading
+//    W once from HBM, so W streams from global memory straight into MFMA
+//    operands: a workgroup owns 16*NT output channels, its waves split K
+//    between them and every lane keeps several 16-byte loads in flight; the
+//    partial sums meet in LDS.  The activations are the other operand, read
+//    through the caches.  A row's result does not depend on M.  The epilogue
+//    may carry the halves of an RMSNorm (NormSplit).
+//  * gemm_qkv_rope_commit: the skinny product for the fused q|k|v projection of
+//    single-token steps, with rotation and the write into the cache's pages.
+//  * gemm_mid: 17..64 rows.  The activations of a k-step are shared by the four
+//    waves through LDS; K may be cut over workgroups into partial sums.
+//  * gemm_tiled, gemm_big: more rows (prefill).  128x128x64 and 256x128x64 tiles
+//    staged through LDS, 32x32x16 MFMA, next tile prefetched into registers.
 //
-// Both need K % 8 == 0 and 16-byte aligned rows; callers fall back to the
+// All need K % 8 == 0 and 16-byte aligned rows; callers fall back to the
 // plain kernel otherwise.
 #include "common.hpp"
 
