@@ -5,7 +5,8 @@
 
 One JSON line: decoded tokens a second of the default run (batch 8 at the
 context length of the configuration), the prefill of one 2,048-token prompt,
-the decode step's share of the HBM roofline, and decoding at batch 1 and 64.
+the decode step's share of the HBM roofline, decoding at batch 1 and 64, and
+what a plain read and a chain of MFMAs reach on the machine ("ceilings").
 Weights are random (seeded), token ids synthetic.  The context is built by a
 real prefill of synthetic prompts.
 """
@@ -166,6 +167,14 @@ def main() -> int:
             points[f"decode_b{b}"] = round(b / s_b, 1)
             print(f"[bench] decode b{b}: {b / s_b:.1f} tok/s", file=sys.stderr, flush=True)
 
+    # what the simplest kernels get here: a plain read of 8 GiB, independent MFMAs on registers
+    from torchless_rs_amd.kernels import ops as _ops
+    del model
+    torch.cuda.empty_cache()
+    ceilings = _ops.measure_ceilings(dev)
+    print(f"[bench] measured ceilings {ceilings}", file=sys.stderr, flush=True)
+    ceilings["decode_frac_of_read"] = round(achieved / ceilings["hbm_read_GBs"], 4)
+    ceilings["prefill_frac_of_mfma"] = round(pre_flops / (pre / 1e3) / (ceilings["mfma_bf16_TFLOPs"] * 1e12), 4)
     out = {
         "metric": f"decode tok/s at batch {args.batch} ({shape_name}), with prefill tok/s at "
                   f"{args.prefill_tokens:,} tokens",
@@ -183,6 +192,7 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4)},
         "points": points,
+        "ceilings": ceilings,
     }
     print(json.dumps(out), flush=True)
     return 0

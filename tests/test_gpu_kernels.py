@@ -725,3 +725,9 @@ def test_rope_commit_adds_partial_products(ops):
     ops.rope_commit(qkv, a["row_pos"], inv, a["table"], a["ring"], nq, nkv, d, q2, p2)
     assert torch.equal(q1, q2)
     assert torch.equal(torch.nan_to_num(p1.float(), nan=-7.0), torch.nan_to_num(p2.float(), nan=-7.0))
+
+
+def test_ceilings_are_measured(ops):
+    """The plain read and the MFMA chain that bench.py quotes run and give sane figures."""
+    c = ops.measure_ceilings(DEV, gib=0.25)
+    assert 100.0 < c["hbm_read_GBs"] < 20000.0 and 50.0 < c["mfma_bf16_TFLOPs"] < 5000.0

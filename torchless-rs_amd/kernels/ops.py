@@ -572,3 +572,33 @@ def attention(q, k_new, v_new, pages, table, ring_pages: int, ctx, n_cached, win
     else:
         attn_plain(q, k_new, v_new, pages, table, ring_pages, ctx.row_seq, ctx.row_pos, ctx.cu_seqlens,
                    n_cached, window, scale, out)
+
+
+def measure_ceilings(device="cuda:0", gib: float = 8.0) -> dict:
+    """What the simplest kernels get on this machine: GB/s of one read of a buffer far larger
+    than the caches, and TFLOP/s of independent bfloat16 MFMAs on registers (the best of a
+    few runs and launch shapes each)."""
+    import time
+    n_bytes = int(gib * 2 ** 30) // 16 * 16
+    buf = torch.empty(n_bytes // 4, dtype=torch.float32, device=device).normal_()
+    sink = torch.zeros(256 * 32, dtype=torch.float32, device=device)
+    best_read = 0.0
+    for blocks in (256 * 4, 256 * 8, 256 * 16, 256 * 32):
+        for _ in range(3):
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            _check(lib().tl_stream_read(_p(buf), ctypes.c_size_t(n_bytes), _p(sink), blocks, _stream()))
+            torch.cuda.synchronize()
+            best_read = max(best_read, n_bytes / (time.perf_counter() - t) / 1e9)
+    del buf
+    best_mfma = 0.0
+    for blocks in (256, 256 * 2, 256 * 4):
+        iters = 8192
+        for _ in range(3):
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            _check(lib().tl_mfma_chain(iters, blocks, _p(sink), _stream()))
+            torch.cuda.synchronize()
+            flop = blocks * 4 * iters * 8 * 2 * 32 * 32 * 16
+            best_mfma = max(best_mfma, flop / (time.perf_counter() - t) / 1e12)
+    return {"hbm_read_GBs": round(best_read, 1), "mfma_bf16_TFLOPs": round(best_mfma, 1)}
