@@ -563,12 +563,13 @@ def test_qkv_rope_commit_equals_product_then_rope_commit(ops, nq, nkv, d, K, len
     q1 = torch.empty(n, nq, d, dtype=torch.bfloat16, device=DEV)
     pages1 = c["pages"].clone()
     ops.rope_commit(qkv, c["row_pos"], inv, c["table"], c["ring"], nq, nkv, d, q1, pages1)
-    q2 = torch.full_like(q1, float("nan"))
-    pages2 = c["pages"].clone()
-    assert ops.qkv_rope_commit_ok(y, w, d, pages2)
-    ops.qkv_rope_commit(y, w, c["row_pos"], inv, c["table"], c["ring"], nq, nkv, d, q2, pages2)
-    assert torch.equal(q1, q2)
-    assert torch.equal(torch.nan_to_num(pages1.float(), nan=-7.0), torch.nan_to_num(pages2.float(), nan=-7.0))
+    assert ops.qkv_rope_commit_ok(y, w, d, c["pages"])
+    for kv_half in (None, False, True):                      # the launcher's choice, whole tiles, half tiles for k and v
+        q2 = torch.full_like(q1, float("nan"))
+        pages2 = c["pages"].clone()
+        ops.qkv_rope_commit(y, w, c["row_pos"], inv, c["table"], c["ring"], nq, nkv, d, q2, pages2, kv_half=kv_half)
+        assert torch.equal(q1, q2)
+        assert torch.equal(torch.nan_to_num(pages1.float(), nan=-7.0), torch.nan_to_num(pages2.float(), nan=-7.0))
     # and against the plain rotation of the plain product
     full = (y.double().cpu() @ w.double().cpu().t()).view(n, nq + 2 * nkv, d)
     pos = c["row_pos"].cpu().long()

@@ -226,26 +226,44 @@ static int launch_skinny(const bf16* A, const bf16* W, float* C, int M, int N, i
 // the sums while they are in LDS: rotation of q and k by the position, q to its buffer,
 // k and v into the sequence's page (v transposed).  To have both halves of a rotated
 // pair, a tile of a q or k head takes channels 8t..8t+7 and d/2+8t..d/2+8t+7; a tile of
-// a v head takes 16 in a row.  The sums and the rotation are those of the unfused
-// kernels, bit for bit (a' = a c - b s; b' = a s + b c; src/kernels/mod.rs:603-605 of
-// the reference).
+// a v head takes 16 in a row.  With kv_half the tiles of k and v heads are half as large
+// (4 pairs, or 8 channels, in the first 8 rows of the MFMA tile; the other rows load
+// nothing): the launcher asks for that when it spreads the workgroups more evenly over
+// the compute units (7B: 384 tiles are one and a half a unit, 256 + 256 are two for all).
+// The sums and the rotation are those of the unfused kernels, bit for bit
+// (a' = a c - b s; b' = a s + b c; src/kernels/mod.rs:603-605 of the reference).
 constexpr int QKV_WAVES = 8;
 
 __global__ void __launch_bounds__(QKV_WAVES * 64)
 gemm_qkv_rope_commit_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, int M, int K,
                             const int* __restrict__ row_pos, const float* __restrict__ inv_freq,
                             const int* __restrict__ table, int table_stride, int ring_pages, int nq,
-                            int nkv, int d, bf16* __restrict__ q, bf16* __restrict__ pages, NormSplit ns) {
+                            int nkv, int d, bf16* __restrict__ q, bf16* __restrict__ pages, NormSplit ns,
+                            int kv_half) {
   __shared__ float red[QKV_WAVES][256];
   __shared__ float cs[16][8], sn[16][8];
   __shared__ float rs[16];
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
   const int li = lane % 16, kg = lane / 16;
-  const int tiles = d / 16, head = blockIdx.x / tiles, tt = blockIdx.x % tiles;
   const int half = d / 2;
+  // which head, which tile of it, and how many pairs (or, for v, channels / 2) the tile holds
+  int head, tt, np = 8;
+  {
+    const int full = d / 16, q_tiles = nq * full;
+    if (!kv_half || (int)blockIdx.x < q_tiles) {
+      head = blockIdx.x / full;
+      tt = blockIdx.x % full;
+    } else {
+      const int r = blockIdx.x - q_tiles;
+      head = nq + r / (2 * full);
+      tt = r % (2 * full);
+      np = 4;
+    }
+  }
   const bool rotated = head < nq + nkv;
-  const int ch = rotated ? (li < 8 ? 8 * tt + li : half + 8 * tt + li - 8) : 16 * tt + li;
-  const bf16* wrow = W + ((size_t)head * d + ch) * K;
+  const bool loads = li < 2 * np;               // rows of the MFMA tile that hold a channel
+  const int ch = rotated ? (li < np ? np * tt + li : half + np * tt + li - np) : 2 * np * tt + li;
+  const bf16* wrow = W + ((size_t)head * d + (loads ? ch : 0)) * K;
   const bf16* arow = A + (size_t)min(li, M - 1) * K;
   const int steps = (K + 63) / 64;
   const int per = (steps + QKV_WAVES - 1) / QKV_WAVES;
@@ -255,8 +273,8 @@ gemm_qkv_rope_commit_kernel(const bf16* __restrict__ A, const bf16* __restrict__
   auto load_step = [&](int s, bf16x8 (&wv)[2], bf16x8 (&av)[2]) {
     const int k = s * 64 + kg * 16;
     const bool ok0 = k + 8 <= K, ok1 = k + 16 <= K;
-    wv[0] = ok0 ? load8(wrow + k) : zero8();
-    wv[1] = ok1 ? load8(wrow + k + 8) : zero8();
+    wv[0] = (ok0 && loads) ? load8(wrow + k) : zero8();
+    wv[1] = (ok1 && loads) ? load8(wrow + k + 8) : zero8();
     av[0] = ok0 ? load8(arow + k) : zero8();
     av[1] = ok1 ? load8(arow + k + 8) : zero8();
   };
@@ -269,7 +287,7 @@ gemm_qkv_rope_commit_kernel(const bf16* __restrict__ A, const bf16* __restrict__
   if (s < s1) load_step(s, w0, a0);
   if (rotated && tid < 128) {                  // while the first loads are under way
     const int m = tid / 8, j = tid % 8;
-    if (m < M) sincosf(inv_freq[8 * tt + j] * (float)row_pos[m], &sn[m][j], &cs[m][j]);
+    if (m < M && j < np) sincosf(inv_freq[np * tt + j] * (float)row_pos[m], &sn[m][j], &cs[m][j]);
   }
   const bool scaled = ns.ssq_in != nullptr;
   RowFactors rf;
@@ -296,10 +314,10 @@ gemm_qkv_rope_commit_kernel(const bf16* __restrict__ A, const bf16* __restrict__
   if (rotated) {
     if (tid < 128) {
       const int m = tid / 8, j = tid % 8;
-      if (m < M) {
+      if (m < M && j < np) {
         float ra, rb;
-        rotate_pair(total(j, m), total(j + 8, m), cs[m][j], sn[m][j], ra, rb);
-        const int i = 8 * tt + j;
+        rotate_pair(total(j, m), total(j + np, m), cs[m][j], sn[m][j], ra, rb);
+        const int i = np * tt + j;
         bf16* dst;
         if (head < nq) {
           dst = q + ((size_t)m * nq + head) * d;
@@ -314,11 +332,11 @@ gemm_qkv_rope_commit_kernel(const bf16* __restrict__ A, const bf16* __restrict__
     }
   } else if (tid < 256) {
     const int m = tid / 16, nl = tid % 16;
-    if (m < M) {
+    if (m < M && nl < 2 * np) {
       const int p = row_pos[m];
       const int page = table[(size_t)m * table_stride + (p / PAGE) % ring_pages];
       bf16* vd = pages + (size_t)page * page_elems + (size_t)nkv * PAGE * d;
-      vd[((size_t)(head - nq - nkv) * d + 16 * tt + nl) * PAGE + p % PAGE] = (bf16)total(nl, m);
+      vd[((size_t)(head - nq - nkv) * d + 2 * np * tt + nl) * PAGE + p % PAGE] = (bf16)total(nl, m);
     }
   }
 }
@@ -814,11 +832,12 @@ extern "C" int tl_gemm_mid_bf16(const void* A, const void* W, void* C, int M, in
 // q|k|v of a step with one token a sequence (row m is sequence m, at position row_pos[m]):
 // W is [(nq + 2 nkv) d, K]; q receives [M, nq, d], the pages k and v of the new position.
 // With ssq_in, row m's sums are multiplied by rsqrt(sum_j ssq_in[m][j] * inv_h + eps) first.
+// kv_half: 1 halves the tiles of k and v heads, 0 does not, -1 lets the launcher choose.
 extern "C" int tl_gemm_qkv_rope_commit(const void* A, const void* W, int M, int K, const int* row_pos,
                                        const float* inv_freq, const int* table, int table_stride,
                                        int ring_pages, int nq, int nkv, int d, void* q, void* pages,
                                        const float* ssq_in, int n_part, float inv_h, float eps,
-                                       hipStream_t st) {
+                                       int kv_half, hipStream_t st) {
   TL_REQUIRE(M >= 0 && M <= 16 && K > 0 && K % 8 == 0, "qkv_rope_commit: bad sizes M=%d K=%d (at most 16 rows, "
              "K a multiple of 8)", M, K);
   TL_REQUIRE(nq > 0 && nkv > 0 && d >= 16 && d % 16 == 0, "qkv_rope_commit: bad heads nq=%d nkv=%d d=%d (head "
@@ -828,12 +847,25 @@ extern "C" int tl_gemm_qkv_rope_commit(const void* A, const void* W, int M, int 
   TL_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "qkv_rope_commit: operands must be 16-byte aligned");
   TL_REQUIRE(ssq_in == nullptr || n_part > 0, "qkv_rope_commit: %d partial sums of squares", n_part);
   if (M == 0) return 0;
-  const int grid = (nq + 2 * nkv) * (d / 16);
+  const int full = (nq + 2 * nkv) * (d / 16), mixed = nq * (d / 16) + 2 * nkv * (d / 8);
+  if (kv_half < 0) {
+    // in units of half a tile, on as many compute units as the device has: which way ends sooner?
+    static int cus = 0;
+    if (cus == 0) {
+      int dev = 0, n = 0;
+      if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+        n = 256;
+      cus = n;
+    }
+    const int t_full = 2 * ((full + cus - 1) / cus), t_mixed = (2 * nq * (d / 16) + 2 * nkv * (d / 8) + cus - 1) / cus;
+    kv_half = t_mixed < t_full;
+  }
+  const int grid = kv_half ? mixed : full;
   NormSplit ns{};
   ns.ssq_in = ssq_in; ns.n_part = n_part; ns.inv_h = inv_h; ns.eps = eps;
   gemm_qkv_rope_commit_kernel<<<grid, QKV_WAVES * 64, 0, st>>>((const bf16*)A, (const bf16*)W, M, K, row_pos,
                                                               inv_freq, table, table_stride, ring_pages, nq,
-                                                              nkv, d, (bf16*)q, (bf16*)pages, ns);
+                                                              nkv, d, (bf16*)q, (bf16*)pages, ns, kv_half);
   TL_LAUNCH_CHECK("gemm_qkv_rope_commit");
   return 0;
 }

@@ -428,10 +428,11 @@ def qkv_rope_commit_ok(a: torch.Tensor, w: torch.Tensor, d: int, pages: torch.Te
 
 def qkv_rope_commit(a: torch.Tensor, w: torch.Tensor, row_pos, inv_freq, table, ring_pages: int, nq: int,
                     nkv: int, d: int, q: torch.Tensor, pages: torch.Tensor,
-                    factor: Optional[RowFactor] = None) -> None:
+                    factor: Optional[RowFactor] = None, kv_half: Optional[bool] = None) -> None:
     """For a step with one token a sequence (at most 16): the product a @ w^T with w = q|k|v,
     the rotation of q and k, q into its buffer and k, v into the pages, in one kernel; the
-    same bits as `gemm` and then `rope_commit`.  `factor`: see `gemm_bf16_norm`."""
+    same bits as `gemm` and then `rope_commit`.  `factor`: see `gemm_bf16_norm`.  `kv_half`
+    (tests): force or forbid the smaller tiles for k and v that the launcher may choose."""
     n, K = a.shape
     _req(a, "qkv_rope_commit.a", torch.bfloat16)
     _req(w, "qkv_rope_commit.w", torch.bfloat16, ((nq + 2 * nkv) * d, K))
@@ -453,7 +454,7 @@ def qkv_rope_commit(a: torch.Tensor, w: torch.Tensor, row_pos, inv_freq, table, 
     _check(lib().tl_gemm_qkv_rope_commit(_p(a), _p(w), n, K, _p(row_pos), _p(inv_freq), _p(table),
                                          table.shape[1], int(ring_pages), nq, nkv, d, _p(q), _p(pages),
                                          _p(ssq_in), n_part, ctypes.c_float(inv_h), ctypes.c_float(eps),
-                                         _stream()))
+                                         -1 if kv_half is None else int(kv_half), _stream()))
 
 
 def aligned_columns(n_cached, n_new):
