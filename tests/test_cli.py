@@ -42,3 +42,14 @@ def test_ids_and_sampling_names():
     assert parse_ids("1, 5 17") == [1, 5, 17]
     assert SamplingConfig().temperature == 1.0                            # sampler/mod.rs:46-54
     assert SamplingConfig.greedy().is_greedy and not SamplingConfig.with_temperature(0.8).is_greedy
+
+
+def test_bench_serves_one_gpu_only():
+    import os
+    import subprocess
+    import sys
+    repo = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(repo, "bench.py"), "--gpus", "2"], capture_output=True,
+                       text=True, timeout=120)
+    assert r.returncode == 2
+    assert len(r.stdout.strip().splitlines()) == 1 and "one GPU" in r.stdout
