@@ -357,7 +357,7 @@ def add_partials(x: torch.Tensor, parts: torch.Tensor) -> None:
     _check(lib().tl_add_partials(_p(x), _p(parts), parts.shape[0], n, H, _stream()))
 
 
-LIBRARY_ROWS = 128          # above this many rows the library's product beats ours
+LIBRARY_ROWS = 64           # above this many rows the library's product beats ours (measured at the 7B sizes)
 
 
 def gemm_library(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
