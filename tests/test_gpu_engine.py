@@ -367,6 +367,48 @@ def test_a_step_with_tokens_on_the_device(zoo):
     eng.cache.check()
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name,seed", [("A", 0), ("B", 1), ("C", 2)])
+def test_random_schedules(zoo, name, dtype, seed):
+    """Sequences come and go at random: each step takes some of the live ones, each with a random
+    number of its next tokens (one token each in every third step, so that captured graphs are
+    replayed too); a finished one gives its slot to a new one.  Every row must match the plain
+    implementation of its own sequence."""
+    import random
+    from torchless_rs_amd.engine import SeqInput
+    eng, z = engine_for(zoo, name, dtype), zoo[name]
+    V = z["cfg"]["vocab_size"]
+    rng = random.Random(seed)
+    lengths = [rng.choice([3, 20, 66, 130]) + rng.randrange(5) for _ in range(7)]
+    seqs = prompts(V, lengths, seed=90 + seed)
+    want = [plain.forward(z["w"], z["cfg"], p) for p in seqs]
+    waiting, live, fed, got = list(range(len(seqs))), {}, {}, {i: [] for i in range(len(seqs))}
+    step = 0
+    while waiting or live:
+        while waiting and len(live) < 4:
+            i = waiting.pop(0)
+            live[i], fed[i] = eng.alloc(), 0
+        step += 1
+        chosen = [i for i in live if rng.random() < 0.7] or [next(iter(live))]
+        batch = []
+        for i in chosen:
+            left = len(seqs[i]) - fed[i]
+            n = 1 if step % 3 == 0 else min(left, rng.choice([1, 2, 5, 17, 40, 70]))
+            batch.append(SeqInput(live[i], seqs[i][fed[i]:fed[i] + n], list(range(n))))
+            fed[i] += n
+        lg = eng.step(batch).clone()
+        r = 0
+        for i, e in zip(chosen, batch):
+            got[i].append(lg[r:r + len(e.tokens)])
+            r += len(e.tokens)
+            if fed[i] == len(seqs[i]):
+                eng.free(live.pop(i))
+        eng.cache.check()
+    for i in range(len(seqs)):
+        assert rel_err(torch.cat(got[i]), want[i]) < TOL[dtype], i
+    assert not eng.cache.length
+
+
 # ---- trace replay ----------------------------------------------------------------
 
 def replay(model_dir, dtype, lines, tmp, max_tokens=1024):
