@@ -86,6 +86,56 @@ def test_rope_split(ops, dt, nq, nkv, d, theta):
 
 
 @pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("window", [None, 128])
+@pytest.mark.parametrize("nq,nkv,d", [(4, 2, 16), (6, 3, 80), (2, 1, 256)])
+def test_values_by_tiles_and_their_commit(ops, dt, window, nq, nkv, d):
+    """`v_tiles` writes what `rope_split` writes into vt, and `kv_commit_tiles` commits what
+    `kv_commit` commits, for sequences that start inside a page, span pages and wrap a ring."""
+    from torchless_rs_amd.cache import PAGE
+    from torchless_rs_amd.parts.position import Rotary
+    cached, new = [0, 70, 64, 130, 5], [2, 4, 64, 200, 59]
+    B, n = len(cached), sum(new)
+    i32 = lambda l: torch.tensor(l, dtype=torch.int32, device=DEV)
+    qkv = rnd(n, (nq + 2 * nkv) * d, seed=61).to(DEV)
+    row_seq = i32([b for b in range(B) for _ in range(new[b])])
+    row_pos = i32([cached[b] + i for b in range(B) for i in range(new[b])])
+    cu = i32([sum(new[:b]) for b in range(B + 1)])
+    after = [c + m for c, m in zip(cached, new)]
+    off, cols = ops.aligned_columns(cached, new)
+    inv = Rotary(d, 10000.0).inv_freq(DEV)
+    q, k, v = (torch.empty(n, h, d, dtype=DT[dt], device=DEV) for h in (nq, nkv, nkv))
+    vt_old = torch.full((nkv, d, cols), 7.0, dtype=DT[dt], device=DEV)
+    ops.rope_split(qkv, row_pos, inv, nq, nkv, d, q, k, v, vt_old, row_seq, i32(off), i32(cached))
+    k2 = torch.empty_like(k)
+    q2 = torch.empty_like(q)
+    ops.rope_split(qkv, row_pos, inv, nq, nkv, d, q2, k2, None)                 # without the values
+    assert torch.equal(q, q2) and torch.equal(k, k2)
+    vt_new = torch.full((nkv, d, cols), 7.0, dtype=DT[dt], device=DEV)
+    ops.v_tiles(qkv, nq, nkv, d, vt_new, cu, i32(off), i32(cached), i32(after))
+    assert torch.equal(vt_old, vt_new)
+    assert int((vt_new != 7.0).sum()) >= nkv * d * n - 8                       # (a value may be 7.0 by chance)
+    # commit: pages of every sequence, rings for the window
+    ring = -(-window // PAGE) if window else 1 << 24
+    need = [min(-(-a // PAGE), ring) for a in after]
+    n_pages = sum(need) + 3
+    perm = torch.randperm(n_pages, generator=torch.Generator().manual_seed(5)).tolist()
+    table = torch.zeros(B, max(need), dtype=torch.int32)
+    for b in range(B):
+        table[b, :need[b]] = torch.tensor([perm.pop() for _ in range(need[b])], dtype=torch.int32)
+    pages_old = torch.full((n_pages, 2, nkv, PAGE, d), 3.0, dtype=DT[dt], device=DEV)
+    pages_new = pages_old.clone()
+    ops.kv_commit(k, v, row_seq, row_pos, i32(after), table.to(DEV), ring, pages_old)
+    ops.kv_commit_tiles(k, vt_new, row_seq, row_pos, i32(off), i32(cached), i32(after), table.to(DEV), ring, pages_new)
+    assert torch.equal(pages_old, pages_new)
+    assert not torch.equal(pages_new, torch.full_like(pages_new, 3.0))
+    if window:                                    # 330 positions in a ring of 2 pages: the first 202 of the step are skipped
+        assert after[3] - ring * PAGE > 131
+    with pytest.raises(ops.KernelError, match="multiple of 64"):
+        ops.v_tiles(qkv, nq, nkv, d, torch.zeros(nkv, d, 100, dtype=DT[dt], device=DEV), cu, i32(off), i32(cached),
+                    i32(after))
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
 def test_silu_mul_and_gather(ops, dt):
     n, I = 5, 301
     gu = rnd(n, 2 * I, seed=4, scale=4.0)

@@ -168,8 +168,10 @@ __global__ void rope_split_kernel(const float* __restrict__ qkv, const int* __re
     dst[i + half] = from_f32<TO>(rb);
   }
   const float* vs = src + (size_t)(nq + nkv) * d;
-  TO* vd = v + (size_t)n * nkv * d;
-  for (int t = threadIdx.x; t < nkv * d; t += blockDim.x) vd[t] = from_f32<TO>(vs[t]);
+  if (v != nullptr) {
+    TO* vd = v + (size_t)n * nkv * d;
+    for (int t = threadIdx.x; t < nkv * d; t += blockDim.x) vd[t] = from_f32<TO>(vs[t]);
+  }
   if (vt != nullptr) {      // the same values transposed: [kv head][d][column of this row]
     const int b = row_seq[n];
     const int col = tile_off[b] + row_pos[n] - (n_cached[b] / PAGE) * PAGE;
@@ -203,6 +205,124 @@ __global__ void kv_commit_kernel(const T* __restrict__ k, const T* __restrict__ 
     const int h = t / d, i = t % d;
     kd[((size_t)h * PAGE + r) * d + i] = ks[t];
     vd[((size_t)h * d + i) * PAGE + r] = vs[t];
+  }
+}
+
+// ---- values by tiles of 64 positions ------------------------------------------
+// Buffers laid out by aligned columns hold sequence b from column tile_off[b] on, position
+// 64 * (n_cached[b] / 64) first, so that a tile of 64 columns is one cache page.  Which
+// sequence and which positions a tile of columns holds:
+struct ColumnTile {
+  int b, p0, lo, hi;        // sequence, position of column 0, positions [lo, hi) of this step in it
+};
+__device__ __forceinline__ ColumnTile column_tile(int col0, int B, const int* tile_off, const int* n_cached,
+                                                  const int* len_after) {
+  int b = 0;
+  while (b + 1 < B && tile_off[b + 1] <= col0) ++b;
+  const int cached = n_cached[b], after = len_after[b];
+  ColumnTile t;
+  t.b = b;
+  t.p0 = (cached / PAGE) * PAGE + (col0 - tile_off[b]);
+  t.lo = max(t.p0, cached);
+  t.hi = min(t.p0 + PAGE, after);            // lo >= hi: padding, nothing of this step
+  return t;
+}
+
+// vt[kv head][dv][column] = v of the row at that column, from the fused projection (float):
+// the transposed values of a step, written in whole lines (a row-by-row kernel writes them
+// two bytes at a time, a line apart).  grid: (columns / 64, kv heads, d / 64 rounded up).
+template <typename TO>
+__global__ void __launch_bounds__(256)
+v_tiles_kernel(const float* __restrict__ qkv, int width, int v_off, int d, TO* __restrict__ vt,
+               int vt_cols, int B, const int* __restrict__ cu_seqlens, const int* __restrict__ tile_off,
+               const int* __restrict__ n_cached, const int* __restrict__ len_after) {
+  __shared__ TO tile[64][PAGE + 2];
+  const int col0 = blockIdx.x * PAGE, kvh = blockIdx.y;
+  const ColumnTile t = column_tile(col0, B, tile_off, n_cached, len_after);
+  if (t.lo >= t.hi) return;
+  const int row0 = cu_seqlens[t.b] - n_cached[t.b];       // row of position p is row0 + p
+  const int c0 = blockIdx.z * 64, dc = min(64, d - c0);    // this block's 64 of the d values
+  // all loads first (16 a thread), then the stores: one trip to memory
+  float tmp[16];
+#pragma unroll
+  for (int u = 0; u < 16; ++u) {
+    const int idx = threadIdx.x + 256 * u;
+    const int r = idx / dc, i = idx % dc, p = t.p0 + r;
+    tmp[u] = (idx < PAGE * dc && p >= t.lo && p < t.hi)
+                 ? qkv[(size_t)(row0 + p) * width + v_off + kvh * d + c0 + i] : 0.f;
+  }
+#pragma unroll
+  for (int u = 0; u < 16; ++u) {
+    const int idx = threadIdx.x + 256 * u;
+    if (idx < PAGE * dc) tile[idx % dc][idx / dc] = from_f32<TO>(tmp[u]);
+  }
+  __syncthreads();
+#pragma unroll
+  for (int u = 0; u < 16; ++u) {
+    const int idx = threadIdx.x + 256 * u;
+    const int i = idx / PAGE, r = idx % PAGE, p = t.p0 + r;
+    if (i < dc && p >= t.lo && p < t.hi) vt[((size_t)kvh * d + c0 + i) * vt_cols + col0 + r] = tile[i][r];
+  }
+}
+
+// Commit of a step whose values lie transposed by tiles: the first blocks put the keys of 8 rows
+// each into their pages, the others copy a tile of values [d][64] of one KV head in whole lines.
+// Positions that the same step overwrites in a ring are skipped, as in kv_commit.
+template <typename T>
+__global__ void __launch_bounds__(256)
+kv_commit_tiles_kernel(const T* __restrict__ k, const T* __restrict__ vt, int vt_cols, int n,
+                       const int* __restrict__ row_seq, const int* __restrict__ row_pos, int B,
+                       const int* __restrict__ tile_off, const int* __restrict__ n_cached,
+                       const int* __restrict__ len_after, const int* __restrict__ table, int table_stride,
+                       int ring_pages, int nkv, int d, T* __restrict__ pages) {
+  const size_t page_elems = (size_t)2 * nkv * PAGE * d;
+  const int k_blocks = (n + 7) / 8;
+  if ((int)blockIdx.x < k_blocks) {
+    // 8 rows a block, 32 threads a row, 16 bytes at a time where the head size allows
+    constexpr int VEC = 16 / sizeof(T);
+    const int r_n = blockIdx.x * 8 + threadIdx.x / 32, lane = threadIdx.x % 32;
+    if (r_n >= n) return;
+    const int b = row_seq[r_n], p = row_pos[r_n];
+    if (p < len_after[b] - ring_pages * PAGE) return;
+    const int page = table[(size_t)b * table_stride + (p / PAGE) % ring_pages];
+    T* kd = pages + (size_t)page * page_elems;
+    const T* ks = k + (size_t)r_n * nkv * d;
+    if (d % VEC == 0 && ((uintptr_t)k % 16 == 0) && ((uintptr_t)pages % 16 == 0)) {
+      for (int c = lane; c < nkv * d / VEC; c += 32) {
+        const int e = c * VEC, h = e / d, i = e % d;
+        *reinterpret_cast<f32x4*>(&kd[((size_t)h * PAGE + p % PAGE) * d + i]) =
+            *reinterpret_cast<const f32x4*>(&ks[e]);
+      }
+    } else {
+      for (int t = lane; t < nkv * d; t += 32) {
+        const int h = t / d, i = t % d;
+        kd[((size_t)h * PAGE + p % PAGE) * d + i] = ks[t];
+      }
+    }
+    return;
+  }
+  const int v_block = blockIdx.x - k_blocks;
+  const int col0 = (v_block / nkv) * PAGE, kvh = v_block % nkv;
+  const ColumnTile t = column_tile(col0, B, tile_off, n_cached, len_after);
+  const int lo = max(t.lo, len_after[t.b] - ring_pages * PAGE);
+  if (lo >= t.hi) return;
+  const int page = table[(size_t)t.b * table_stride + (t.p0 / PAGE) % ring_pages];
+  T* vd = pages + (size_t)page * page_elems + (size_t)nkv * PAGE * d + (size_t)kvh * d * PAGE;
+  const T* vs = vt + (size_t)kvh * d * vt_cols + col0;
+  for (int base = 0; base < d * PAGE; base += 256 * 16) {      // 16 loads a thread, then their stores
+    T tmp[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      const int idx = base + threadIdx.x + 256 * u;
+      const int i = idx / PAGE, r = idx % PAGE, p = t.p0 + r;
+      if (i < d && p >= lo && p < t.hi) tmp[u] = vs[(size_t)i * vt_cols + r];
+    }
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      const int idx = base + threadIdx.x + 256 * u;
+      const int i = idx / PAGE, r = idx % PAGE, p = t.p0 + r;
+      if (i < d && p >= lo && p < t.hi) vd[(size_t)i * PAGE + r] = tmp[u];
+    }
   }
 }
 
@@ -433,6 +553,52 @@ int tl_kv_commit(const void* k, const void* v, int dt, const int* row_seq, const
   else
     TL_REQUIRE(false, "kv_commit: unknown dtype code %d", dt);
   TL_LAUNCH_CHECK("kv_commit");
+  return 0;
+}
+
+int tl_v_tiles(const float* qkv, int n, int nq, int nkv, int d, void* vt, int vt_cols, int dt, int B,
+               const int* cu_seqlens, const int* tile_off, const int* n_cached, const int* len_after,
+               hipStream_t st) {
+  TL_REQUIRE(n >= 0 && nq >= 0 && nkv > 0 && d > 0 && B > 0, "v_tiles: bad sizes n=%d nq=%d nkv=%d d=%d B=%d", n, nq,
+             nkv, d, B);
+  TL_REQUIRE(vt_cols > 0 && vt_cols % PAGE == 0 && nkv <= 65535, "v_tiles: %d columns (a multiple of 64), %d KV heads",
+             vt_cols, nkv);
+  if (n == 0) return 0;
+  const int width = (nq + 2 * nkv) * d, v_off = (nq + nkv) * d;
+  const dim3 grid(vt_cols / PAGE, nkv, (d + 63) / 64);
+  if (dt == DT_F32)
+    v_tiles_kernel<float><<<grid, 256, 0, st>>>(qkv, width, v_off, d, (float*)vt, vt_cols, B, cu_seqlens,
+                                                 tile_off, n_cached, len_after);
+  else if (dt == DT_BF16)
+    v_tiles_kernel<bf16><<<grid, 256, 0, st>>>(qkv, width, v_off, d, (bf16*)vt, vt_cols, B, cu_seqlens,
+                                                tile_off, n_cached, len_after);
+  else
+    TL_REQUIRE(false, "v_tiles: unknown dtype code %d", dt);
+  TL_LAUNCH_CHECK("v_tiles");
+  return 0;
+}
+
+int tl_kv_commit_tiles(const void* k, const void* vt, int vt_cols, int dt, const int* row_seq, const int* row_pos,
+                       int B, const int* tile_off, const int* n_cached, const int* len_after, const int* table,
+                       int table_stride, int ring_pages, int n, int nkv, int d, void* pages, hipStream_t st) {
+  TL_REQUIRE(n >= 0 && nkv > 0 && d > 0 && ring_pages > 0 && table_stride > 0 && B > 0,
+             "kv_commit_tiles: bad sizes n=%d nkv=%d d=%d ring_pages=%d table_stride=%d B=%d", n, nkv, d,
+             ring_pages, table_stride, B);
+  TL_REQUIRE(vt_cols > 0 && vt_cols % PAGE == 0, "kv_commit_tiles: %d columns (a multiple of 64)", vt_cols);
+  if (n == 0) return 0;
+  const long long blocks = (long long)((n + 7) / 8) + (long long)(vt_cols / PAGE) * nkv;
+  TL_REQUIRE(blocks < 2147483647LL, "kv_commit_tiles: too many blocks");
+  if (dt == DT_F32)
+    kv_commit_tiles_kernel<float><<<(unsigned)blocks, 256, 0, st>>>(
+        (const float*)k, (const float*)vt, vt_cols, n, row_seq, row_pos, B, tile_off, n_cached, len_after, table,
+        table_stride, ring_pages, nkv, d, (float*)pages);
+  else if (dt == DT_BF16)
+    kv_commit_tiles_kernel<bf16><<<(unsigned)blocks, 256, 0, st>>>(
+        (const bf16*)k, (const bf16*)vt, vt_cols, n, row_seq, row_pos, B, tile_off, n_cached, len_after, table,
+        table_stride, ring_pages, nkv, d, (bf16*)pages);
+  else
+    TL_REQUIRE(false, "kv_commit_tiles: unknown dtype code %d", dt);
+  TL_LAUNCH_CHECK("kv_commit_tiles");
   return 0;
 }
 

@@ -88,7 +88,8 @@ def rope_split(qkv: torch.Tensor, row_pos: torch.Tensor, inv_freq: torch.Tensor,
                d: int, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, vt: Optional[torch.Tensor] = None,
                row_seq=None, tile_off=None, n_cached=None) -> None:
     """Rotate q and k of the fused projection by their rows' positions and
-    write q [n,nq,d], k, v [n,nkv,d].  With `vt` [nkv, d, cols] the values are
+    write q [n,nq,d], k, v [n,nkv,d] (v may be None: the values are taken by
+    `v_tiles` then).  With `vt` [nkv, d, cols] the values are
     also written transposed, row n into column tile_off[b] + pos - 64 *
     (n_cached[b] // 64) of its sequence b = row_seq[n]."""
     n = qkv.shape[0]
@@ -98,7 +99,8 @@ def rope_split(qkv: torch.Tensor, row_pos: torch.Tensor, inv_freq: torch.Tensor,
     _req(q, "rope.q", None, (n, nq, d))
     if nkv:
         _req(k, "rope.k", q.dtype, (n, nkv, d))
-        _req(v, "rope.v", q.dtype, (n, nkv, d))
+        if v is not None:
+            _req(v, "rope.v", q.dtype, (n, nkv, d))
     cols = 0
     if vt is not None:
         _req(vt, "rope.vt", q.dtype)
@@ -131,6 +133,54 @@ def kv_commit(k: torch.Tensor, v: torch.Tensor, row_seq, row_pos, len_after, tab
         raise KernelError("kv_commit.table: needs one row per sequence")
     _check(lib().tl_kv_commit(_p(k), _p(v), _code(k.dtype), _p(row_seq), _p(row_pos), _p(len_after),
                               _p(table), table.shape[1], ring_pages, n, nkv, d, _p(pages), _stream()))
+
+
+def _tiles_args(B, cu_seqlens, tile_off, n_cached, len_after, what):
+    _req(tile_off, what + ".tile_off", torch.int32, (B,))
+    _req(n_cached, what + ".n_cached", torch.int32, (B,))
+    _req(len_after, what + ".len_after", torch.int32, (B,))
+    if cu_seqlens is not None:
+        _req(cu_seqlens, what + ".cu_seqlens", torch.int32, (B + 1,))
+
+
+def v_tiles(qkv: torch.Tensor, nq: int, nkv: int, d: int, vt: torch.Tensor, cu_seqlens, tile_off, n_cached,
+            len_after) -> None:
+    """The values of a step transposed, from the fused projection: vt[kv head, dv, column],
+    sequence b from column tile_off[b] on (`aligned_columns`), written by tiles of 64
+    positions in whole lines.  Columns that hold no position of this step are left alone."""
+    n = qkv.shape[0]
+    _req(qkv, "v_tiles.qkv", torch.float32, (n, (nq + 2 * nkv) * d))
+    _req(vt, "v_tiles.vt")
+    if vt.dim() != 3 or tuple(vt.shape[:2]) != (nkv, d) or vt.shape[2] % 64:
+        raise KernelError(f"v_tiles.vt: shape {tuple(vt.shape)}, kernel needs [{nkv}, {d}, a multiple of 64]")
+    B = tile_off.shape[0]
+    _tiles_args(B, cu_seqlens, tile_off, n_cached, len_after, "v_tiles")
+    _check(lib().tl_v_tiles(_p(qkv), n, nq, nkv, d, _p(vt), vt.shape[2], _code(vt.dtype), B, _p(cu_seqlens),
+                            _p(tile_off), _p(n_cached), _p(len_after), _stream()))
+
+
+def kv_commit_tiles(k: torch.Tensor, vt: torch.Tensor, row_seq, row_pos, tile_off, n_cached, len_after,
+                    table: torch.Tensor, ring_pages: int, pages: torch.Tensor) -> None:
+    """`kv_commit` for a step whose values lie transposed by tiles (`v_tiles`): keys row by
+    row, values a tile [d, 64] at a time in whole lines."""
+    n, nkv, d = k.shape
+    _req(k, "kv_commit.k", pages.dtype)
+    _req(vt, "kv_commit.vt", pages.dtype)
+    if vt.dim() != 3 or tuple(vt.shape[:2]) != (nkv, d) or vt.shape[2] % 64:
+        raise KernelError(f"kv_commit.vt: shape {tuple(vt.shape)}, kernel needs [{nkv}, {d}, a multiple of 64]")
+    _req(row_seq, "kv_commit.row_seq", torch.int32, (n,))
+    _req(row_pos, "kv_commit.row_pos", torch.int32, (n,))
+    B = tile_off.shape[0]
+    _tiles_args(B, None, tile_off, n_cached, len_after, "kv_commit")
+    _req(table, "kv_commit.table", torch.int32)
+    _req(pages, "kv_commit.pages")
+    if pages.dim() != 5 or tuple(pages.shape[1:]) != (2, nkv, 64, d):
+        raise KernelError(f"kv_commit.pages: shape {tuple(pages.shape)}, kernel needs [*, 2, {nkv}, 64, {d}]")
+    if table.dim() != 2 or table.shape[0] != B:
+        raise KernelError("kv_commit.table: needs one row per sequence")
+    _check(lib().tl_kv_commit_tiles(_p(k), _p(vt), vt.shape[2], _code(k.dtype), _p(row_seq), _p(row_pos), B,
+                                    _p(tile_off), _p(n_cached), _p(len_after), _p(table), table.shape[1],
+                                    ring_pages, n, nkv, d, _p(pages), _stream()))
 
 
 def attn_plain(q, k_new, v_new, pages, table, ring_pages: int, row_seq, row_pos, cu_seqlens, n_cached,

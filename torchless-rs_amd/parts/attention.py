@@ -101,12 +101,16 @@ class AttentionMixer(Mixer):
             qkv = ws.get("attn_qkv", (n, (nq + 2 * nkv) * d), torch.float32)
             self.qkv(y, qkv)
             k = ws.get("attn_k" + tag, (n, nkv, d), ctx.dtype)
-            v = ws.get("attn_v" + tag, (n, nkv, d), ctx.dtype)
-            vt = None
             if ops.uses_transposed_values(ctx.dtype, d, ctx.all_single):
+                # the matrix cores read values along the keys: only the transposed copy is made, by tiles
+                v = None
                 vt = ws.get("attn_vt" + tag, (nkv, d, ctx.host["aligned_cols"]), ctx.dtype)
-            ops.rope_split(qkv, ctx.row_pos, inv_freq, nq, nkv, d, q, k, v, vt, ctx.row_seq, ctx.tile_off,
-                           ctx.len_before)
+                ops.rope_split(qkv, ctx.row_pos, inv_freq, nq, nkv, d, q, k, None)
+                ops.v_tiles(qkv, nq, nkv, d, vt, ctx.cu_seqlens, ctx.tile_off, ctx.len_before, ctx.len_after)
+            else:
+                vt = None
+                v = ws.get("attn_v" + tag, (n, nkv, d), ctx.dtype)
+                ops.rope_split(qkv, ctx.row_pos, inv_freq, nq, nkv, d, q, k, v)
             if run.kv_read_later:
                 ctx.host[f"kv_new_{run.index}"] = (k, v, vt)
         else:
@@ -126,8 +130,12 @@ class AttentionMixer(Mixer):
                           self.window, self.scale, out, vt_new=vt)
             if self.own_kv:
                 def commit():
-                    ops.kv_commit(k, v, ctx.row_seq, ctx.row_pos, ctx.len_after, table,
-                                  group.ring_pages, pages)
+                    if vt is not None:
+                        ops.kv_commit_tiles(k, vt, ctx.row_seq, ctx.row_pos, ctx.tile_off, ctx.len_before,
+                                            ctx.len_after, table, group.ring_pages, pages)
+                    else:
+                        ops.kv_commit(k, v, ctx.row_seq, ctx.row_pos, ctx.len_after, table,
+                                      group.ring_pages, pages)
                 if run.kv_read_later:       # a later run still reads the old rows of the ring
                     ctx.host.setdefault("deferred", []).append(commit)
                 else:
