@@ -40,19 +40,28 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
                     const bf16* __restrict__ vt_new, int vt_cols, const int* __restrict__ tile_off,
                     const bf16* __restrict__ pages, const int* __restrict__ table, int table_stride,
                     int ring_pages, const int* __restrict__ row_pos, const int* __restrict__ cu_seqlens,
-                    const int* __restrict__ n_cached, int B, int nq, int nkv, int d, int window,
-                    float scale, bf16* __restrict__ out) {
+                    const int* __restrict__ n_cached, int B, int n_tiles, int cus_per_xcd, int nq, int nkv,
+                    int d, int window, float scale, bf16* __restrict__ out) {
   constexpr int KB = DPAD / 16, VB = DPAD / 32, KLD = DPAD + 8, CH = DPAD / 8;
   constexpr int PT = DPAD / 32;        // 16-byte chunks of keys, and of values, per thread and tile
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   bf16* Ks = reinterpret_cast<bf16*>(smem);          // [PF_BN][KLD]
   bf16* Vt = Ks + PF_BN * KLD;                       // [DPAD][PF_VLD]
 
-  // Which sequence and which block of its rows.  All workgroups of a step are usually resident
-  // at once, two a compute unit, and a late block has many times the keys of an early one: the
-  // first half of the heads takes the blocks from the last to the first, the second half from
-  // the first to the last, so that the two that meet on a compute unit have about the same sum.
-  int t = (blockIdx.y < (gridDim.y + 1) / 2) ? gridDim.x - 1 - blockIdx.x : blockIdx.x, b = 0;
+  // Which head and which block of rows.  The (head, block) pairs, heads in their order, are cut
+  // into 8 equal runs, and workgroup L takes pair L / 8 of run L % 8: workgroups are dealt round
+  // to the 8 XCDs, so an XCD works on a run of neighbouring heads, and the keys and values of
+  // their one or two KV heads stay in its L2 while the blocks of rows pass over them.  Inside a
+  // head the late blocks (most keys) come first, or last: the direction turns every `turn`
+  // heads, chosen so that the workgroups an XCD's compute units get in the first and in the
+  // second round (cus_per_xcd pairs apart) run in opposite directions and a long one meets a
+  // short one.
+  const int total = n_tiles * nq, per_xcd = (total + 7) / 8;
+  const int item = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
+  if ((int)(blockIdx.x / 8) >= per_xcd || item >= total) return;
+  const int h = item / n_tiles;
+  const int turn = max(1, cus_per_xcd / n_tiles);
+  int t = ((h / turn) % 2 == 0) ? n_tiles - 1 - item % n_tiles : item % n_tiles, b = 0;
   for (; b < B; ++b) {
     const int tiles = (cu_seqlens[b + 1] - cu_seqlens[b] + PF_BM - 1) / PF_BM;
     if (t < tiles) break;
@@ -60,7 +69,7 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
   }
   if (b == B) return;
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64, l32 = lane % 32, half = lane / 32;
-  const int h = blockIdx.y, kvh = h / (nq / nkv);
+  const int kvh = h / (nq / nkv);
   const int row0 = cu_seqlens[b], n_new = cu_seqlens[b + 1] - row0;
   const int cached = n_cached[b];
   const int p_first = row_pos[row0];
@@ -521,10 +530,24 @@ static int launch_prefill(const bf16* q, const bf16* k_new, const bf16* vt_new, 
       raised = true;
     }
   }
-  dim3 grid(n_tiles, nq);
+  const long long total = (long long)n_tiles * nq;
+  if (total > 2147483000LL) {
+    set_error("attn_prefill: %lld (head, block of rows) pairs are too many", total);
+    return 1;
+  }
+  const unsigned grid = (unsigned)((total + 7) / 8 * 8);
+  static int cus_per_xcd = 0;
+  if (cus_per_xcd == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 8)
+      n = 256;
+    cus_per_xcd = n / 8;
+  }
   attn_prefill_kernel<DPAD><<<grid, 256, smem, st>>>(q, k_new, vt_new, vt_cols, tile_off, pages, table,
                                                      table_stride, ring_pages, row_pos, cu_seqlens,
-                                                     n_cached, B, nq, nkv, d, window, scale, out);
+                                                     n_cached, B, n_tiles, cus_per_xcd, nq, nkv, d, window,
+                                                     scale, out);
   TL_LAUNCH_CHECK("attn_prefill");
   return 0;
 }
