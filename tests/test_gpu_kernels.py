@@ -635,7 +635,7 @@ def test_qkv_rope_commit_equals_product_then_rope_commit(ops, nq, nkv, d, K, len
 # ---- an RMSNorm cut in two around products of at most 16 rows ----------------------------
 
 @pytest.mark.parametrize("M", [1, 5, 16])
-@pytest.mark.parametrize("N,K,N2", [(200, 72, 50), (64, 264, 16384), (1000, 96, 130)])
+@pytest.mark.parametrize("N,K,N2", [(200, 72, 50), (64, 264, 16384), (1000, 96, 130), (4616, 72, 48)])   # the last: more than 256 workgroups wrote
 def test_gemm_norm_halves(ops, M, N, K, N2):
     """The product that completes the stream writes x * w and its workgroups' sums of x^2;
     the product that reads them applies rsqrt(mean + eps): together the plain norm between."""
