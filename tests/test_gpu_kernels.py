@@ -782,3 +782,64 @@ def test_ceilings_are_measured(ops):
     """The plain read and the MFMA chain that bench.py quotes run and give sane figures."""
     c = ops.measure_ceilings(DEV, gib=0.25)
     assert 100.0 < c["hbm_read_GBs"] < 20000.0 and 50.0 < c["mfma_bf16_TFLOPs"] < 5000.0
+
+
+@pytest.mark.parametrize("window", [None, 4096])
+def test_attention_over_a_long_context(ops, window):
+    """70,000 cached positions in scattered pages: the new token's query (decode kernel) and a
+    chunk of 130 new rows (prefill kernel) against the softmax written out for those rows only.
+    One far key is made to stand out, so that a page taken from the wrong place would show."""
+    nq, nkv, d, L, n_new = 2, 1, 16, 70000, 130
+    PAGE = 64
+    ring = -(-window // PAGE) if window else 1 << 24
+    T = L + n_new
+    g = torch.Generator().manual_seed(3)
+    q = torch.randn(T, nq, d, generator=g).to(torch.bfloat16)
+    k = torch.randn(T, nkv, d, generator=g).to(torch.bfloat16)
+    v = torch.randn(T, nkv, d, generator=g).to(torch.bfloat16)
+    far = L - 3000
+    q0 = q[L, 0].float()
+    k[far] = (q0 * (24.0 * math.sqrt(d) / float(q0 @ q0))).to(torch.bfloat16)   # score 24: row L's head 0 looks at `far`
+    held = min(-(-T // PAGE), ring)
+    perm = torch.randperm(held + 5, generator=g)
+    table = perm[:held].to(torch.int32).view(1, held)
+
+    def fill(upto):
+        pages = torch.full((held + 5, 2, nkv, PAGE, d), float("nan"), dtype=torch.bfloat16)
+        for p0 in range(max(0, (upto - ring * PAGE) // PAGE * PAGE) if window else 0, upto, PAGE):
+            pg = int(table[0, (p0 // PAGE) % ring])
+            n = min(PAGE, upto - p0)
+            pages[pg, 0, :, :n] = k[p0:p0 + n].transpose(0, 1)
+            pages[pg, 1].view(nkv, d, PAGE)[:, :, :n] = v[p0:p0 + n].permute(1, 2, 0)
+        return pages
+
+    def want(rows):
+        out = torch.empty(len(rows), nq, d, dtype=torch.float64)
+        for i, p in enumerate(rows):
+            lo = max(0, p - window + 1) if window else 0
+            for h in range(nq):
+                s = (k[lo:p + 1, 0].double() @ q[p, h].double()) / math.sqrt(d)
+                out[i, h] = torch.softmax(s, 0) @ v[lo:p + 1, 0].double()
+        return out
+
+    i32 = lambda l: torch.tensor(l, dtype=torch.int32, device=DEV)
+    # decode: position L, everything in the pages (the new key committed)
+    pages = fill(L + 1).to(DEV)
+    out = torch.empty(1, nq, d, dtype=torch.bfloat16, device=DEV)
+    for splits in (1, 7, 64):
+        part = torch.empty(nq * splits * (d + 2), device=DEV)
+        ops.attn_decode_bf16(q[L:L + 1].to(DEV), pages, table.to(DEV), ring, i32([L]), window, 1 / math.sqrt(d),
+                             splits, part, out)
+        assert rel_err(out, want([L])) < KTOL["bfloat16"], splits
+    assert rel_err(out[0, 0], v[far, 0].double()) < 0.05                # head 0 returns the far value
+    # prefill: rows L .. L + 129 over the cache of L positions
+    pages = fill(L).to(DEV)
+    off, cols = ops.aligned_columns([L], [n_new])
+    vt = torch.zeros(nkv, d, cols, dtype=torch.bfloat16)
+    vt[:, :, L % PAGE:L % PAGE + n_new] = v[L:].permute(1, 2, 0)
+    outp = torch.empty(n_new, nq, d, dtype=torch.bfloat16, device=DEV)
+    ops.attn_prefill_bf16(q[L:].contiguous().to(DEV), k[L:].contiguous().to(DEV), vt.to(DEV), i32(off), pages,
+                          table.to(DEV), ring, i32(list(range(L, T))), i32([0, n_new]), i32([L]), -(-n_new // 128),
+                          window, 1 / math.sqrt(d), outp)
+    rows = [L, L + 1, L + 63, L + 64, L + 129]
+    assert rel_err(outp[[r - L for r in rows]], want(rows)) < KTOL["bfloat16"]
