@@ -843,3 +843,13 @@ def test_attention_over_a_long_context(ops, window):
                           window, 1 / math.sqrt(d), outp)
     rows = [L, L + 1, L + 63, L + 64, L + 129]
     assert rel_err(outp[[r - L for r in rows]], want(rows)) < KTOL["bfloat16"]
+    # and all 70,130 rows in one step, nothing cached
+    off, cols = ops.aligned_columns([0], [T])
+    vt = torch.zeros(nkv, d, cols, dtype=torch.bfloat16)
+    vt[:, :, :T] = v.permute(1, 2, 0)
+    outp = torch.empty(T, nq, d, dtype=torch.bfloat16, device=DEV)
+    ops.attn_prefill_bf16(q.to(DEV), k.to(DEV), vt.to(DEV), i32(off), pages, table.to(DEV), ring,
+                          i32(list(range(T))), i32([0, T]), i32([0]), -(-T // 128), window, 1 / math.sqrt(d), outp)
+    rows = [0, 63, 64, 4095, 4096, 4097, 40000, L, T - 1]
+    assert rel_err(outp[rows], want(rows)) < KTOL["bfloat16"]
+    assert torch.isfinite(outp.float()).all()
