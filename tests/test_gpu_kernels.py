@@ -427,7 +427,8 @@ def test_gemm_dispatch_falls_back_when_k_is_odd(ops):
 # ---- bfloat16 attention on the matrix cores -----------------------------------------
 
 SHAPES = [(4, 2, 16, None), (6, 1, 32, 70), (5, 5, 48, 8), (8, 2, 128, 100), (2, 1, 256, None),
-          (3, 3, 80, 64), (32, 8, 128, 200), (20, 1, 64, None), (4, 4, 160, 130)]
+          (3, 3, 80, 64), (32, 8, 128, 200), (20, 1, 64, None), (4, 4, 160, 130), (6, 2, 96, None),
+          (2, 2, 192, 50), (2, 1, 224, None)]
 
 
 def transposed_values(ops, a, lens_cached, lens_new):

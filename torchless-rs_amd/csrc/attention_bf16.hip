@@ -17,6 +17,10 @@ namespace tl {
 
 __device__ __forceinline__ bf16x8 ld8(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
 __device__ __forceinline__ bf16x4 ld4(const bf16* p) { return *reinterpret_cast<const bf16x4*>(p); }
+// 16 bytes at a uniform base plus a lane's offset in bytes (32 bits: one address register)
+__device__ __forceinline__ bf16x8 ld8_at(const bf16* base, unsigned bytes) {
+  return *reinterpret_cast<const bf16x8*>(reinterpret_cast<const char*>(base) + bytes);
+}
 __device__ __forceinline__ bf16x8 z8() {
   bf16x8 z;
 #pragma unroll
@@ -34,7 +38,7 @@ __device__ __forceinline__ bf16x8 z8() {
 // fetched into registers while the current one is worked on.
 constexpr int PF_BM = 128, PF_BN = 64, PF_VLD = PF_BN + 4;
 
-template <int DPAD>
+template <int DPAD, bool LEAN>       // LEAN (d == DPAD, 256 % (DPAD / 8) == 0): whole tiles are fetched the short way
 __global__ void __launch_bounds__(256, DPAD <= 128 ? 2 : 1)
 attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
                     const bf16* __restrict__ vt_new, int vt_cols, const int* __restrict__ tile_off,
@@ -104,12 +108,40 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
   bf16x8 kfetch[PT], vfetch[PT];
   // tile j0 -> registers: keys as rows [key][d], values as rows [dv][key]
   const int seq_end = p_first + n_new;               // one past the sequence's last position
+  // Whole tiles of a head that fills its padded size take the short way: the workgroup's base
+  // address is uniform and a thread's chunks lie at fixed offsets from it, one stride apart.
+  static_assert(PF_BN == PAGE, "a tile of keys below n_cached is one page");
+  static_assert(!LEAN || 256 % CH == 0, "the short way needs every thread's chunks in one column of chunks");
+  const unsigned k_row = tid / CH, k_col = (tid % CH) * 16;                        // offsets in bytes
+  const unsigned v_row = tid / (PF_BN / 8), v_col = (tid % (PF_BN / 8)) * 16;
+  auto fetch_lean = [&](const bf16* kbase, unsigned k_stride, const bf16* vbase, unsigned v_stride) {
+    // the offsets are worked out anew for every tile (a multiply-add each): kept across the loop
+    // they would take sixteen registers that the loop does not have
+    unsigned kr = k_row, vr = v_row;
+    asm volatile("" : "+v"(kr), "+v"(vr));
+#pragma unroll
+    for (int i = 0; i < PT; ++i) {
+      kfetch[i] = ld8_at(kbase, (kr + i * (256 / CH)) * k_stride + k_col);
+      vfetch[i] = ld8_at(vbase, (vr + i * (256 / (PF_BN / 8))) * v_stride + v_col);
+    }
+  };
+  // tiles are fetched in their order: the place in the ring of pages is counted along, and the
+  // page of the tile after the next is looked up a tile early, so that no fetch waits for it
+  const int jt_first = j_lo / PF_BN;
+  int f_ring = jt_first % ring_pages;
+  int page_nxt = ((jt_first + 1) * PF_BN <= cached) ? table[(size_t)b * table_stride + f_ring] : 0;
   auto fetch = [&](int j0) {
+    const int page = page_nxt;
+    f_ring = (f_ring + 1 == ring_pages) ? 0 : f_ring + 1;
+    if (j0 + 2 * PF_BN <= cached) page_nxt = table[(size_t)b * table_stride + f_ring];
     if (j0 + PF_BN <= cached) {
       // a cached page: keys [64][d], values [d][64]
-      const int page = table[(size_t)b * table_stride + (j0 / PAGE) % ring_pages];
       const bf16* kpage = pages + (size_t)page * page_elems + (size_t)kvh * head_elems;
       const bf16* vpage = kpage + (size_t)nkv * head_elems;
+      if constexpr (LEAN) {
+        fetch_lean(kpage, 2u * d, vpage, 2u * PAGE);        // rows [64][d] and [d][64]
+        return;
+      }
 #pragma unroll
       for (int i = 0; i < PT; ++i) {
         const int c = tid + 256 * i;
@@ -124,6 +156,10 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
       // rows of this step, all of them written
       const bf16* krows = k_new + ((size_t)(row0 + j0 - cached) * nkv + kvh) * d;
       const bf16* vcols = vt_head + (j0 - j_base);
+      if constexpr (LEAN) {
+        fetch_lean(krows, 2u * nkv * d, vcols, 2u * vt_cols);
+        return;
+      }
 #pragma unroll
       for (int i = 0; i < PT; ++i) {
         const int c = tid + 256 * i;
@@ -188,7 +224,6 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
     }
   };
 
-  const int jt_first = j_lo / PF_BN;
   fetch(jt_first * PF_BN);
   for (int jt = jt_first; jt * PF_BN <= p_hi; ++jt) {
     const int j0 = jt * PF_BN;
@@ -246,35 +281,44 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
     const float c1 = scale * 1.44269504088896f, c0 = -m_use * 1.44269504088896f;
     float psum = 0.f;
     bf16x8 pb[2][2];
+    // probability e of the tile's 32 (e = 16 nb + r), in the order of the sum
+    auto soft = [&](int e) {
+      const int nb = e / 16, r = e % 16;
+      const float pv = __builtin_amdgcn_exp2f(fmaf(s[nb][r], c1, c0));
+      psum += pv;
+      pb[nb][r / 8][r % 8] = (bf16)pv;
+    };
+    // values of block vb against probabilities 8 qd .. 8 qd + 7 (qd = 2 nb + mm): these are keys
+    // kk + {0..3} and kk + 8 + {0..3}, kk = 32 nb + 16 mm + 4 half
+    auto vfrag = [&](int qd, int vb) {
+      const bf16* vrow = &Vt[(vb * 32 + l32) * PF_VLD + (qd / 2) * 32 + 16 * (qd % 2) + 4 * half];
+      const bf16x4 lo4 = ld4(vrow), hi4 = ld4(vrow + 8);
+      bf16x8 a;
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const float pv = __builtin_amdgcn_exp2f(fmaf(s[nb][r], c1, c0));
-        psum += pv;
-        pb[nb][r / 8][r % 8] = (bf16)pv;
+      for (int e = 0; e < 4; ++e) {
+        a[e] = lo4[e];
+        a[4 + e] = hi4[e];
       }
+      return a;
+    };
+    // The second product goes quarter by quarter of the tile's keys, and while the matrix cores
+    // work on one quarter the vector unit makes the probabilities of the next: the order below is
+    // pinned, one MFMA and its share of the next quarter's eight probabilities at a time.
+#pragma unroll
+    for (int e = 0; e < 8; ++e) soft(e);
+#pragma unroll
+    for (int qd = 0; qd < 4; ++qd) {
+#pragma unroll
+      for (int vb = 0; vb < VB; ++vb) {
+        o[vb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfrag(qd, vb), pb[qd / 2][qd % 2], o[vb], 0, 0, 0);
+        if (qd < 3) {
+#pragma unroll
+          for (int e = (8 * vb) / VB; e < (8 * (vb + 1)) / VB; ++e) soft(8 * (qd + 1) + e);
+        }
+      }
+    }
     psum += __shfl_xor(psum, 32, WAVE);
     l += psum;
-#pragma unroll
-    for (int vb = 0; vb < VB; ++vb) {
-#pragma unroll
-      for (int nb = 0; nb < 2; ++nb)
-#pragma unroll
-        for (int mm = 0; mm < 2; ++mm) {
-          // probabilities r = 8 mm .. 8 mm + 7 are keys kk + 4 half + {0..3} and kk + 8 + 4 half + {0..3}
-          const int kk = nb * 32 + 16 * mm + 4 * half;
-          const bf16* vrow = &Vt[(vb * 32 + l32) * PF_VLD + kk];
-          const bf16x4 lo4 = ld4(vrow), hi4 = ld4(vrow + 8);
-          bf16x8 a;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            a[e] = lo4[e];
-            a[4 + e] = hi4[e];
-          }
-          o[vb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[nb][mm], o[vb], 0, 0, 0);
-        }
-    }
   }
   if (q_ok) {
     bf16* op = out + ((size_t)(row0 + qr) * nq + h) * d;
@@ -518,11 +562,16 @@ static int launch_prefill(const bf16* q, const bf16* k_new, const bf16* vt_new, 
                           const int* cu_seqlens, const int* n_cached, int B, int n_tiles, int nq, int nkv,
                           int d, int window, float scale, bf16* out, hipStream_t st) {
   const size_t smem = ((size_t)PF_BN * (DPAD + 8) + (size_t)DPAD * PF_VLD) * sizeof(bf16);
+  constexpr bool can_lean = 256 % (DPAD / 8) == 0;
   if (smem > 48 * 1024) {
     static bool raised = false;
     if (!raised) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prefill_kernel<DPAD>),
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prefill_kernel<DPAD, false>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+      if constexpr (can_lean)
+        if (e == hipSuccess)
+          e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prefill_kernel<DPAD, true>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
       if (e != hipSuccess) {
         set_error("attn_prefill: cannot have %zu bytes of LDS: %s", smem, hipGetErrorString(e));
         return 2;
@@ -544,10 +593,16 @@ static int launch_prefill(const bf16* q, const bf16* k_new, const bf16* vt_new, 
       n = 256;
     cus_per_xcd = n / 8;
   }
-  attn_prefill_kernel<DPAD><<<grid, 256, smem, st>>>(q, k_new, vt_new, vt_cols, tile_off, pages, table,
-                                                     table_stride, ring_pages, row_pos, cu_seqlens,
-                                                     n_cached, B, n_tiles, cus_per_xcd, nq, nkv, d, window,
-                                                     scale, out);
+  if (can_lean && d == DPAD)
+    attn_prefill_kernel<DPAD, can_lean><<<grid, 256, smem, st>>>(q, k_new, vt_new, vt_cols, tile_off, pages, table,
+                                                             table_stride, ring_pages, row_pos, cu_seqlens,
+                                                             n_cached, B, n_tiles, cus_per_xcd, nq, nkv, d,
+                                                             window, scale, out);
+  else
+    attn_prefill_kernel<DPAD, false><<<grid, 256, smem, st>>>(q, k_new, vt_new, vt_cols, tile_off, pages, table,
+                                                              table_stride, ring_pages, row_pos, cu_seqlens,
+                                                              n_cached, B, n_tiles, cus_per_xcd, nq, nkv, d,
+                                                              window, scale, out);
   TL_LAUNCH_CHECK("attn_prefill");
   return 0;
 }
