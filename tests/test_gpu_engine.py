@@ -567,3 +567,33 @@ def test_layer_sizes_of_the_7b_shape(tmp_path, dtype):
     eng.free(a)
     assert rel_err(torch.cat(outs_a), wants[0][140:150]) < TOL[dtype]
     assert rel_err(torch.cat(outs_b), wants[1][65:70]) < TOL[dtype]
+
+
+def test_steps_of_65_to_128_rows_at_7b_layer_sizes(tmp_path):
+    """Between 65 and 128 rows the products of q|k|v, o and down are ours with K cut into partial
+    sums (gate|up is the library's): a prompt of 100 tokens in one step, then 70 sequences that
+    go on by one token each."""
+    from torchless_rs_amd import write_random_model
+    from torchless_rs_amd.engine import Engine, SeqInput, load_model
+    cfgd = {"architectures": ["MistralForCausalLM"], "num_hidden_layers": 2, "hidden_size": 4096,
+            "num_attention_heads": 32, "num_key_value_heads": 8, "intermediate_size": 14336,
+            "vocab_size": 32000, "rope_theta": 10000.0, "sliding_window": 96, "rms_norm_eps": 1e-5}
+    d = write_random_model(str(tmp_path / "wide"), cfgd, seed=7, std=0.02, dtype=torch.bfloat16)
+    cfg, w = read_model_dir(d)
+    eng = Engine(load_model(d, "bfloat16"), max_tokens=64 * 80)
+    long = prompts(32000, [101], seed=8)[0]
+    want = plain.forward(w, cfg, long, dtype=torch.float32)
+    a = eng.alloc()
+    lg = eng.step([SeqInput(a, long[:100], [0, 64, 99])]).clone()
+    assert rel_err(lg, want[[0, 64, 99]]) < TOL["bfloat16"]
+    lg = eng.step([SeqInput(a, long[100:], [0])]).clone()
+    assert rel_err(lg, want[[100]]) < TOL["bfloat16"]
+    eng.free(a)
+    many = prompts(32000, [4] * 70, seed=9)
+    slots = [eng.alloc() for _ in many]
+    eng.step([SeqInput(s, p[:3], []) for s, p in zip(slots, many)])
+    lg = eng.step([SeqInput(s, p[3:], [0]) for s, p in zip(slots, many)]).clone()
+    for i in (0, 1, 33, 64, 69):
+        assert rel_err(lg[i:i + 1], plain.forward(w, cfg, many[i], dtype=torch.float32)[[3]]) < TOL["bfloat16"]
+    for s in slots:
+        eng.free(s)

@@ -712,9 +712,9 @@ def test_qkv_rope_commit_with_row_factor(ops):
         assert rel_err(pages[pg, 1].reshape(nkv, d, 64)[:, :, p % 64], full[b, nq + nkv:]) < KTOL["bfloat16"]
 
 
-# ---- 17..64 rows: shared activations, K cut into partial sums -----------------------------
+# ---- 17..128 rows: shared activations, K cut into partial sums (above 64 rows the k-step is 128) --
 
-@pytest.mark.parametrize("M", [17, 32, 33, 48, 50, 64, 5])
+@pytest.mark.parametrize("M", [17, 32, 33, 48, 50, 64, 5, 65, 80, 97, 112, 128])
 @pytest.mark.parametrize("N,K,S", [(50, 72, 1), (64, 512, 2), (130, 776, 3), (200, 2000, 7), (384, 96, 1), (96, 4096, 16)])
 def test_gemm_mid_bf16(ops, M, N, K, S):
     a = rnd(M, K, seed=41, dtype=torch.bfloat16)
@@ -745,7 +745,7 @@ def test_gemm_mid_bf16(ops, M, N, K, S):
         assert rel_err(y, plain.rmsnorm(x.double().cpu(), g.double().cpu(), 1e-5)) < KTOL["bfloat16"]
 
 
-@pytest.mark.parametrize("M", [20, 64])
+@pytest.mark.parametrize("M", [20, 64, 72, 128])
 def test_gemm_mid_paired_silu_and_row_independence(ops, M):
     from torchless_rs_amd.parts.linear import interleave_pairs
     I, K = 160, 200

@@ -10,7 +10,7 @@
 //    may carry the halves of an RMSNorm (NormSplit).
 //  * gemm_qkv_rope_commit: the skinny product for the fused q|k|v projection of
 //    single-token steps, with rotation and the write into the cache's pages.
-//  * gemm_mid: 17..64 rows.  The activations of a k-step are shared by the four
+//  * gemm_mid: 17..128 rows.  The activations of a k-step are shared by the four
 //    waves through LDS; K may be cut over workgroups into partial sums.
 //  * gemm_tiled, gemm_big: more rows (prefill).  128x128x64 and 256x128x64 tiles
 //    staged through LDS, 32x32x16 MFMA, next tile prefetched into registers.
@@ -342,7 +342,7 @@ gemm_qkv_rope_commit_kernel(const bf16* __restrict__ A, const bf16* __restrict__
 }
 
 // ------------------------------------------------------------------- mid ----
-// 17..64 rows (decode at larger batches).  Per byte of W there are now enough
+// 17..128 rows (decode at larger batches, short prompts).  Per byte of W there are now enough
 // MFMAs that the activations must be shared: a workgroup owns 64 output
 // channels (one 16-channel tile per wave) and a slice of K; the activations of
 // a k-step go through LDS once for the four waves, W streams from global
@@ -424,7 +424,7 @@ gemm_mid_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float* _
   if (epilogue == EPI_SILU_PAIR) {
     // the workgroup's 64 rows are one group: waves 0,1 hold gate rows, waves 2,3 their up rows
     __syncthreads();
-    float* ex = reinterpret_cast<float*>(&As[0]);           // [2 waves][MT][4][64] floats <= 8 KB
+    float* ex = reinterpret_cast<float*>(&As[0]);           // [2 waves][MT][4][64] floats: 2 KB a row tile
     if (wave >= 2) {
 #pragma unroll
       for (int u = 0; u < MT; ++u)
@@ -465,14 +465,16 @@ gemm_mid_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float* _
   }
 }
 
-constexpr int MID_KS = 256;
+constexpr int MID_KS = 256;       // k per step up to 64 rows; half of it above, where the rows in LDS are twice as many
+constexpr int MID_ROWS = 128;
 
 template <int MT>
 static int launch_mid(const bf16* A, const bf16* W, float* C, int M, int N, int K, int n_split, int epilogue,
                       hipStream_t st) {
-  const int steps = (K + MID_KS - 1) / MID_KS, per = (steps + n_split - 1) / n_split;
+  constexpr int KS = MT > 4 ? MID_KS / 2 : MID_KS;
+  const int steps = (K + KS - 1) / KS, per = (steps + n_split - 1) / n_split;
   dim3 grid((N + 63) / 64, n_split);
-  gemm_mid_kernel<MT, MID_KS><<<grid, 256, 0, st>>>(A, W, C, M, N, K, per, epilogue);
+  gemm_mid_kernel<MT, KS><<<grid, 256, 0, st>>>(A, W, C, M, N, K, per, epilogue);
   TL_LAUNCH_CHECK("gemm_mid");
   return 0;
 }
@@ -806,13 +808,13 @@ extern "C" int tl_gemm_bf16_variant(const void* A, const void* W, void* C, int M
   TL_REQUIRE(false, "gemm_bf16: unknown variant %d", variant);
 }
 
-// 17..64 rows.  n_split == 1: C as in tl_gemm_bf16 (all three epilogues).  n_split > 1: C is
+// 17..128 rows.  n_split == 1: C as in tl_gemm_bf16 (all three epilogues).  n_split > 1: C is
 // float [n_split][M][N] and receives partial sums (epilogue must be 0); every split gets at
 // least one k-step of 256.
 extern "C" int tl_gemm_mid_bf16(const void* A, const void* W, void* C, int M, int N, int K, int n_split,
                                 int epilogue, hipStream_t st) {
-  TL_REQUIRE(M > 0 && M <= 64 && N > 0 && K > 0 && K % 8 == 0, "gemm_mid: bad sizes M=%d N=%d K=%d (M at most 64, "
-             "K a multiple of 8)", M, N, K);
+  TL_REQUIRE(M > 0 && M <= MID_ROWS && N > 0 && K > 0 && K % 8 == 0, "gemm_mid: bad sizes M=%d N=%d K=%d (M at most "
+             "%d, K a multiple of 8)", M, N, K, MID_ROWS);
   TL_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "gemm_mid: operands must be 16-byte aligned");
   TL_REQUIRE(n_split >= 1 && n_split <= (K + MID_KS - 1) / MID_KS && n_split <= 65535,
              "gemm_mid: %d splits do not fit K=%d (one step of %d at least each)", n_split, K, MID_KS);
@@ -826,7 +828,11 @@ extern "C" int tl_gemm_mid_bf16(const void* A, const void* W, void* C, int M, in
   if (M <= 16) return launch_mid<1>(a, w, c, M, N, K, n_split, epilogue, st);
   if (M <= 32) return launch_mid<2>(a, w, c, M, N, K, n_split, epilogue, st);
   if (M <= 48) return launch_mid<3>(a, w, c, M, N, K, n_split, epilogue, st);
-  return launch_mid<4>(a, w, c, M, N, K, n_split, epilogue, st);
+  if (M <= 64) return launch_mid<4>(a, w, c, M, N, K, n_split, epilogue, st);
+  if (M <= 80) return launch_mid<5>(a, w, c, M, N, K, n_split, epilogue, st);
+  if (M <= 96) return launch_mid<6>(a, w, c, M, N, K, n_split, epilogue, st);
+  if (M <= 112) return launch_mid<7>(a, w, c, M, N, K, n_split, epilogue, st);
+  return launch_mid<8>(a, w, c, M, N, K, n_split, epilogue, st);
 }
 
 // q|k|v of a step with one token a sequence (row m is sequence m, at position row_pos[m]):

@@ -352,18 +352,28 @@ def gemm_bf16_norm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumula
     return groups.value
 
 
+MID_ROWS = 128      # most rows of the kernel that shares a k-step's activations through LDS
+
+
 def mid_splits(M: int, N: int, K: int) -> int:
-    """For 17..64 rows: into how many slices K is cut so that some 400
-    workgroups (64 output channels each) are at work; 1 where N alone gives
-    them."""
+    """For 17..MID_ROWS rows: into how many slices K is cut so that some 400
+    workgroups or more (64 output channels each) are at work, a power of two
+    (which shares the k-steps out evenly at the usual sizes; measured best at
+    the 7B sizes); 1 where N alone gives them."""
     blocks = -(-N // 64)
     steps = -(-K // 256)
-    return max(1, min(-(-400 // blocks), steps, 16))
+    want = -(-400 // blocks)
+    S = 1
+    while S < want and S < 16:
+        S *= 2
+    while S > steps:
+        S //= 2
+    return max(1, S)
 
 
 def gemm_mid_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, n_split: int = 1,
                   accumulate: bool = False, silu_pair: bool = False) -> None:
-    """The product for 17..64 rows.  n_split == 1: out as in `gemm_bf16`.
+    """The product for 17..MID_ROWS rows.  n_split == 1: out as in `gemm_bf16`.
     n_split > 1: out is float32 [n_split, M, N] and receives partial sums that
     the next kernel adds up (`add_rmsnorm`, `add_partials`, `rope_commit`)."""
     M, K = a.shape
@@ -407,7 +417,8 @@ def add_partials(x: torch.Tensor, parts: torch.Tensor) -> None:
     _check(lib().tl_add_partials(_p(x), _p(parts), parts.shape[0], n, H, _stream()))
 
 
-LIBRARY_ROWS = 64           # above this many rows the library's product beats ours (measured at the 7B sizes)
+LIBRARY_ROWS = 64           # above this many rows the library's product beats ours (measured at the 7B sizes),
+                            # but for small N up to MID_ROWS rows, where ours wins with K cut into partial sums
 
 
 def gemm_library(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:

@@ -98,8 +98,13 @@ class AttentionMixer(Mixer):
             return
         if self.own_kv:
             tag = f"_{run.index}" if run.kv_read_later else ""
-            qkv = ws.get("attn_qkv", (n, (nq + 2 * nkv) * d), torch.float32)
-            self.qkv(y, qkv)
+            parts = self.qkv.partial(y, ctx, "attn_qkv_parts")
+            if parts is not None:               # K cut into partial sums: the first slice takes the others
+                qkv = parts[0]
+                ops.add_partials(qkv, parts[1:])
+            else:
+                qkv = ws.get("attn_qkv", (n, (nq + 2 * nkv) * d), torch.float32)
+                self.qkv(y, qkv)
             k = ws.get("attn_k" + tag, (n, nkv, d), ctx.dtype)
             if ops.uses_transposed_values(ctx.dtype, d, ctx.all_single):
                 # the matrix cores read values along the keys: only the transposed copy is made, by tiles

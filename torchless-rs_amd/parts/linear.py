@@ -22,18 +22,20 @@ class Linear:
         second half of the norm that made `a`, a factor per row (at most 16 rows)."""
         if factor is not None:
             ops.gemm_bf16_norm(a, self.weight, out, accumulate, factor=factor)
-        elif self.mid(a):
+        elif self.mid(a) and a.shape[0] <= ops.LIBRARY_ROWS:
             ops.gemm_mid_bf16(a, self.weight, out, 1, accumulate)
         else:
             ops.gemm(a, self.weight, out, accumulate)
 
     def mid(self, a: torch.Tensor) -> bool:
-        """17..64 rows of bfloat16: the kernel that shares the activations."""
-        return 16 < a.shape[0] <= 64 and ops.bf16_gemm_ok(a, self.weight)
+        """17..MID_ROWS rows of bfloat16: the kernel that shares the activations.
+        (Above LIBRARY_ROWS rows it beats the library only with K cut into
+        partial sums, which `partial` does.)"""
+        return 16 < a.shape[0] <= ops.MID_ROWS and ops.bf16_gemm_ok(a, self.weight)
 
     def partial(self, a: torch.Tensor, ctx, name: str):
         """The product as partial sums [S, M, N] (float32) for a reader that adds
-        them up, where that pays (17..64 rows and K worth cutting); else None."""
+        them up, where that pays (17..MID_ROWS rows and K worth cutting); else None."""
         if not self.mid(a):
             return None
         S = ops.mid_splits(a.shape[0], self.out_features, self.in_features)
