@@ -343,7 +343,7 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
 // result is written at once.
 constexpr int DC_WAVES = 4;
 
-template <int DPAD>   // multiple of 32
+template <int DPAD, bool LEAN>   // DPAD: multiple of 32; LEAN: d == DPAD, loads without guards at fixed offsets
 __global__ void __launch_bounds__(DC_WAVES * 64)
 attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
                    const int* __restrict__ table, int table_stride, int ring_pages,
@@ -382,10 +382,20 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
   for (int vb = 0; vb < VB; ++vb) o[vb] = f32x4{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
 
-  // the split's groups of 32 keys go round the waves
-  for (int gi = 2 * my_lo + wave; gi < 2 * my_hi; gi += DC_WAVES) {
+  // the split's groups of 32 keys go round the waves; a wave's pages are two apart, and the id of
+  // its next page is looked up while it works on this one
+  static_assert(DC_WAVES == 4, "a wave's groups are two pages apart");
+  const int* trow = table + (size_t)b * table_stride;
+  const int gi0 = 2 * my_lo + wave;
+  int ring = (gi0 / 2) % ring_pages;
+  int page_nxt = gi0 < 2 * my_hi ? trow[ring] : 0;
+  for (int gi = gi0; gi < 2 * my_hi; gi += DC_WAVES) {
     const int pg = gi / 2, grp = gi % 2;
-    const int page = table[(size_t)b * table_stride + pg % ring_pages];
+    const int page = page_nxt;
+    ring += 2;
+    if (ring >= ring_pages) ring -= ring_pages;
+    if (ring >= ring_pages) ring -= ring_pages;          // (a ring of one page)
+    if (gi + DC_WAVES < 2 * my_hi) page_nxt = trow[ring];
     const bf16* kbase = pages + (size_t)page * page_elems + (size_t)kvh * head_elems;
     const bf16* vbase = kbase + (size_t)nkv * head_elems;
     {
@@ -395,19 +405,33 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
       // the two blocks are 8 consecutive keys, j0 + 8 kg .. + 7
       // all loads of the group first: keys (two blocks) and values
       bf16x8 kreg[2][KB], vreg[VB];
+      if constexpr (LEAN) {
+        // a uniform base for the group plus this lane's offset in bytes; the rest are constants
+        const bf16* kgrp = kbase + grp * 32 * DPAD;
+        const bf16* vgrp = vbase + grp * 32;
+        unsigned k_lane = ((8 * (li / 4) + (li % 4)) * DPAD + 8 * kg) * 2, v_lane = (li * PAGE + 8 * kg) * 2;
+        asm volatile("" : "+v"(k_lane), "+v"(v_lane));     // (worked out here, not kept in 24 registers)
 #pragma unroll
-      for (int bs = 0; bs < 2; ++bs) {
-        const bf16* krow = kbase + (size_t)(grp * 32 + 8 * (li / 4) + 4 * bs + (li % 4)) * d;
+        for (int bs = 0; bs < 2; ++bs)
 #pragma unroll
-        for (int kb = 0; kb < KB; ++kb) {
-          const int k = kb * 32 + 8 * kg;
-          kreg[bs][kb] = (k + 8 <= d) ? ld8(krow + k) : z8();
+          for (int kb = 0; kb < KB; ++kb) kreg[bs][kb] = ld8_at(kgrp, k_lane + (bs * 4 * DPAD + kb * 32) * 2);
+#pragma unroll
+        for (int vb = 0; vb < VB; ++vb) vreg[vb] = ld8_at(vgrp, v_lane + vb * 16 * PAGE * 2);
+      } else {
+#pragma unroll
+        for (int bs = 0; bs < 2; ++bs) {
+          const bf16* krow = kbase + (size_t)(grp * 32 + 8 * (li / 4) + 4 * bs + (li % 4)) * d;
+#pragma unroll
+          for (int kb = 0; kb < KB; ++kb) {
+            const int k = kb * 32 + 8 * kg;
+            kreg[bs][kb] = (k + 8 <= d) ? ld8(krow + k) : z8();
+          }
         }
-      }
 #pragma unroll
-      for (int vb = 0; vb < VB; ++vb) {
-        const int dv = vb * 16 + li;
-        vreg[vb] = (dv < d) ? ld8(vbase + (size_t)dv * PAGE + grp * 32 + 8 * kg) : z8();
+        for (int vb = 0; vb < VB; ++vb) {
+          const int dv = vb * 16 + li;
+          vreg[vb] = (dv < d) ? ld8(vbase + (size_t)dv * PAGE + grp * 32 + 8 * kg) : z8();
+        }
       }
       f32x4 s[2];
 #pragma unroll
@@ -443,18 +467,24 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
       l = l * alpha + psum;
       m = m_new;
       // O^T[dv][head] += V^T[dv][keys] P^T[keys][head]; values lie as [d][PAGE] in the page
+      if (j0 + 31 > p) {           // rows past the sequence's end were never written: 0 * garbage
+        typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+        u32x4 keep;                // this lane's 8 keys are 4 pairs of 16 bits
 #pragma unroll
-      for (int vb = 0; vb < VB; ++vb) {
-        bf16x8 a = vreg[vb];
-        if (j0 + 31 > p) {         // rows past the sequence's end were never written: 0 * garbage
+        for (int w2 = 0; w2 < 4; ++w2)
+          keep[w2] = (j0 + 8 * kg + 2 * w2 <= p ? 0x0000ffffu : 0u) | (j0 + 8 * kg + 2 * w2 + 1 <= p ? 0xffff0000u : 0u);
 #pragma unroll
-          for (int e = 0; e < 8; ++e)
-            if (j0 + 8 * kg + e > p) a[e] = (bf16)0.f;
-        }
-#pragma unroll
-        for (int r = 0; r < 4; ++r) o[vb][r] *= alpha;
-        o[vb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pb, o[vb], 0, 0, 0);
+        for (int vb = 0; vb < VB; ++vb)
+          vreg[vb] = __builtin_bit_cast(bf16x8, __builtin_bit_cast(u32x4, vreg[vb]) & keep);
       }
+      if (__ballot(alpha != 1.0f) != 0ull) {      // the running maximum moved in some lane
+#pragma unroll
+        for (int vb = 0; vb < VB; ++vb)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) o[vb][r] *= alpha;
+      }
+#pragma unroll
+      for (int vb = 0; vb < VB; ++vb) o[vb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg[vb], pb, o[vb], 0, 0, 0);
     }
   }
   // o[vb][r] = O[dv = 16 vb + 4 kg + r][head li]; m, l are per head li (equal in the 4 kg lanes).
@@ -613,9 +643,14 @@ static int launch_decode(const bf16* q, const bf16* pages, const int* table, int
                          float scale, int n_splits, float* part, bf16* out, hipStream_t st) {
   const int g = nq / nkv, head_groups = (g + 15) / 16;
   dim3 grid(B * nkv * head_groups, n_splits);
-  attn_decode_kernel<DPAD><<<grid, DC_WAVES * 64, 0, st>>>(q, pages, table, table_stride, ring_pages,
-                                                            row_pos, nq, nkv, d, window, scale, n_splits,
-                                                            head_groups, part, out);
+  if (d == DPAD)
+    attn_decode_kernel<DPAD, true><<<grid, DC_WAVES * 64, 0, st>>>(q, pages, table, table_stride, ring_pages,
+                                                                    row_pos, nq, nkv, d, window, scale, n_splits,
+                                                                    head_groups, part, out);
+  else
+    attn_decode_kernel<DPAD, false><<<grid, DC_WAVES * 64, 0, st>>>(q, pages, table, table_stride, ring_pages,
+                                                                     row_pos, nq, nkv, d, window, scale, n_splits,
+                                                                     head_groups, part, out);
   TL_LAUNCH_CHECK("attn_decode");
   if (n_splits > 1) {
     attn_decode_combine_kernel<<<B * nq, 64, 0, st>>>(part, n_splits, d, out);
