@@ -89,7 +89,7 @@ struct RowFactors {
 };
 
 // ---------------------------------------------------------------- skinny ----
-template <int NT, int MT, int SK_WAVES>
+template <int NT, int MT, int SK_WAVES, bool FULLK>      // FULLK: K % 64 == 0, no load needs a guard (and a branch)
 __global__ void __launch_bounds__(SK_WAVES * 64)
 gemm_skinny_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float* __restrict__ C, int M,
                    int N, int K, int epilogue, NormSplit ns) {
@@ -119,7 +119,7 @@ gemm_skinny_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float
   // this lane's 16 consecutive k of a step: two chunks of 8
   auto load_step = [&](int s, bf16x8 (&wv)[NT][2], bf16x8 (&av)[MT][2]) {
     const int k = s * 64 + kg * 16;
-    const bool ok0 = k + 8 <= K, ok1 = k + 16 <= K;
+    const bool ok0 = FULLK || k + 8 <= K, ok1 = FULLK || k + 16 <= K;
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       wv[t][0] = ok0 ? load8(wrow[t] + k) : zero8();
@@ -215,7 +215,10 @@ template <int NT, int MT, int SK_WAVES = 8>
 static int launch_skinny(const bf16* A, const bf16* W, float* C, int M, int N, int K, int epilogue,
                          hipStream_t st, NormSplit ns = NormSplit{}) {
   const int grid = (N + 16 * NT - 1) / (16 * NT);
-  gemm_skinny_kernel<NT, MT, SK_WAVES><<<grid, SK_WAVES * 64, 0, st>>>(A, W, C, M, N, K, epilogue, ns);
+  if (K % 64 == 0)
+    gemm_skinny_kernel<NT, MT, SK_WAVES, true><<<grid, SK_WAVES * 64, 0, st>>>(A, W, C, M, N, K, epilogue, ns);
+  else
+    gemm_skinny_kernel<NT, MT, SK_WAVES, false><<<grid, SK_WAVES * 64, 0, st>>>(A, W, C, M, N, K, epilogue, ns);
   TL_LAUNCH_CHECK("gemm_skinny");
   return 0;
 }
@@ -349,8 +352,8 @@ gemm_qkv_rope_commit_kernel(const bf16* __restrict__ A, const bf16* __restrict__
 // memory into registers.  With n_split > 1 the slices of K go to different
 // workgroups, which write partial sums P[split][M][N]; the kernel that reads
 // them next adds them up (always in the order of the splits).
-template <int MT, int KS>      // KS: k per step (a multiple of 64); everything of a step is in flight at once
-__global__ void __launch_bounds__(256)
+template <int MT, int KS, bool FULLK>   // KS: k per step (a multiple of 64), everything of a step is in flight at once;
+__global__ void __launch_bounds__(256)  // FULLK: K % KS == 0, no load needs a guard (and a branch)
 gemm_mid_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float* __restrict__ C, int M,
                 int N, int K, int steps_per_split, int epilogue) {
   constexpr int ROWS = MT * 16, LD = KS + 8, SUB = KS / 64;
@@ -369,7 +372,7 @@ gemm_mid_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float* _
     for (int i = 0; i < PER; ++i) {
       const int c = tid + 256 * i;
       const int row = c / CPR, k = s * KS + (c % CPR) * 8;
-      areg[i] = (c < CHUNKS && k + 8 <= K) ? load8(A + (size_t)min(row, M - 1) * K + k) : zero8();
+      areg[i] = (c < CHUNKS && (FULLK || k + 8 <= K)) ? load8(A + (size_t)min(row, M - 1) * K + k) : zero8();
     }
   };
   auto stash_a = [&]() {
@@ -384,8 +387,8 @@ gemm_mid_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float* _
 #pragma unroll
     for (int j = 0; j < SUB; ++j) {
       const int k = s * KS + j * 64 + kg * 16;
-      w[j][0] = (k + 8 <= K) ? load8(wrow + k) : zero8();
-      w[j][1] = (k + 16 <= K) ? load8(wrow + k + 8) : zero8();
+      w[j][0] = (FULLK || k + 8 <= K) ? load8(wrow + k) : zero8();
+      w[j][1] = (FULLK || k + 16 <= K) ? load8(wrow + k + 8) : zero8();
     }
   };
 
@@ -474,7 +477,10 @@ static int launch_mid(const bf16* A, const bf16* W, float* C, int M, int N, int 
   constexpr int KS = MT > 4 ? MID_KS / 2 : MID_KS;
   const int steps = (K + KS - 1) / KS, per = (steps + n_split - 1) / n_split;
   dim3 grid((N + 63) / 64, n_split);
-  gemm_mid_kernel<MT, KS><<<grid, 256, 0, st>>>(A, W, C, M, N, K, per, epilogue);
+  if (K % KS == 0)
+    gemm_mid_kernel<MT, KS, true><<<grid, 256, 0, st>>>(A, W, C, M, N, K, per, epilogue);
+  else
+    gemm_mid_kernel<MT, KS, false><<<grid, 256, 0, st>>>(A, W, C, M, N, K, per, epilogue);
   TL_LAUNCH_CHECK("gemm_mid");
   return 0;
 }
