@@ -597,3 +597,47 @@ def test_steps_of_65_to_128_rows_at_7b_layer_sizes(tmp_path):
         assert rel_err(lg[i:i + 1], plain.forward(w, cfg, many[i], dtype=torch.float32)[[3]]) < TOL["bfloat16"]
     for s in slots:
         eng.free(s)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_configurations(tmp_path, seed):
+    """Configurations drawn at random (head sizes in steps of 16 up to 256, any heads and groups,
+    widths and vocabularies that are no powers of two, with and without a window): unequal
+    prompts in one step with every row wanted, then the last tokens one by one, in both dtypes."""
+    import random
+    from torchless_rs_amd import write_random_model
+    from torchless_rs_amd.engine import Engine, SeqInput, load_model
+    rng = random.Random(1000 + seed)
+    d = rng.choice([16, 32, 48, 64, 80, 96, 112, 128, 160, 192, 224, 256])
+    nkv = rng.choice([1, 2, 3, 4])
+    nq = nkv * rng.choice([1, 2, 3, 5, 8, 17] if d <= 64 else [1, 2, 4])
+    cfg = {"architectures": ["MistralForCausalLM"], "model_type": "mistral",
+           "num_hidden_layers": rng.choice([1, 2, 3]), "hidden_size": rng.choice([40, 72, 96, 136, 200, 264]),
+           "num_attention_heads": nq, "num_key_value_heads": nkv, "head_dim": d,
+           "intermediate_size": rng.choice([64, 96, 160, 224, 352]), "vocab_size": rng.choice([130, 257, 384, 1000]),
+           "rope_theta": rng.choice([500.0, 10000.0, 1e6]), "sliding_window": rng.choice([None, 7, 64, 70, 150]),
+           "rms_norm_eps": rng.choice([1e-5, 1e-6, 1e-4]), "max_position_embeddings": 1024,
+           "tie_word_embeddings": False, "hidden_act": "silu"}
+    mdir = write_random_model(str(tmp_path / "m"), cfg, seed=seed, std=0.05, norm_std=0.1, dtype=torch.bfloat16)
+    cfgd, w = read_model_dir(mdir)
+    lens = [rng.choice([1, 5, 33, 64, 65, 100, 129, 200]) for _ in range(rng.choice([1, 2, 3, 5]))]
+    ids = prompts(cfg["vocab_size"], lens, seed=100 + seed)
+    wants = [plain.forward(w, cfgd, p, dtype=torch.float32) for p in ids]
+    for dtype in DTYPES:
+        eng = Engine(load_model(mdir, dtype), max_tokens=64 * (sum(-(-n // 64) for n in lens) + 2))
+        slots = [eng.alloc() for _ in ids]
+        tail = [min(len(p) - 1, rng.choice([0, 1, 7, 32])) for p in ids]
+        heads = [len(p) - t for p, t in zip(ids, tail)]
+        lg = eng.step([SeqInput(s, p[:h], list(range(h))) for s, p, h in zip(slots, ids, heads)]).clone()
+        worst, o = 0.0, 0
+        for i, h in enumerate(heads):
+            worst = max(worst, rel_err(lg[o:o + h], wants[i][:h]))
+            o += h
+        for t in range(max(tail)):
+            live = [i for i in range(len(ids)) if t < tail[i]]
+            lg = eng.step([SeqInput(slots[i], [ids[i][heads[i] + t]], [0]) for i in live]).clone()
+            for r, i in enumerate(live):
+                worst = max(worst, rel_err(lg[r:r + 1], wants[i][heads[i] + t:heads[i] + t + 1]))
+        for s in slots:
+            eng.free(s)
+        assert worst < TOL[dtype], (cfg, lens, tail, dtype, worst)
