@@ -692,6 +692,10 @@ extern "C" int tl_attn_prefill_bf16(const void* q, const void* k_new, const void
   TL_REQUIRE(vt_cols > 0 && vt_cols % 64 == 0 && ((uintptr_t)vt_new % 16 == 0),
              "attn_prefill: the transposed values need a multiple of 64 columns (%d) and 16-byte alignment",
              vt_cols);
+  // (a thread's offsets into the step's keys and transposed values are 32 bits)
+  TL_REQUIRE((long long)vt_cols * 2 * 256 < (1LL << 32) && (long long)nkv * d * 2 * 64 < (1LL << 32),
+             "attn_prefill: %d columns of transposed values (or %d KV heads of %d) are too many for one step",
+             vt_cols, nkv, d);
   TL_BY_DPAD(launch_prefill, (const bf16*)q, (const bf16*)k_new, (const bf16*)vt_new, vt_cols, tile_off,
              (const bf16*)pages, table, table_stride, ring_pages, row_pos, cu_seqlens, n_cached, B,
              n_tiles, nq, nkv, d, window, scale, (bf16*)out, st);
