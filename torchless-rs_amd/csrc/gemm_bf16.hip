@@ -141,6 +141,19 @@ gemm_skinny_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float
       }
   };
 
+  // What the accumulating epilogue adds to and scales by is asked for now, where a thread has
+  // one element of it at most: the answers are there when the sums are.
+  constexpr int NB = 16 * NT;
+  constexpr bool one_each = NB * 16 * MT <= SK_WAVES * 64;
+  const bool writer = MT == 1 && ns.norm_w != nullptr;          // with EPI_ACCUMULATE only (checked on the host)
+  float c_old = 0.f, w_norm = 0.f;
+  if (one_each && epilogue == EPI_ACCUMULATE) {
+    const int nl = threadIdx.x % NB, m = threadIdx.x / NB;
+    if ((int)threadIdx.x < NB * 16 * MT && n0 + nl < N && m < M) {
+      c_old = C[(size_t)m * N + n0 + nl];
+      if (writer) w_norm = ns.norm_w[n0 + nl];
+    }
+  }
   bf16x8 w0[NT][2], a0[MT][2], w1[NT][2], a1[MT][2];
   int s = s0;
   if (s < s1) load_step(s, w0, a0);
@@ -164,7 +177,6 @@ gemm_skinny_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float
 #pragma unroll
       for (int r = 0; r < 4; ++r) red[wave][((t * MT + u) * 4 + r) * 64 + lane] = acc[t][u][r];
   __syncthreads();
-  constexpr int NB = 16 * NT;
   auto total = [&](int nl, int m) {
     const int t = nl / 16, u = m / 16;
     const int idx = ((t * MT + u) * 4 + (nl % 4)) * 64 + ((nl % 16) / 4) * 16 + (m % 16);
@@ -190,7 +202,6 @@ gemm_skinny_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float
     }
     return;
   }
-  const bool writer = MT == 1 && ns.norm_w != nullptr;          // with EPI_ACCUMULATE only (checked on the host)
   for (int e = threadIdx.x; e < NB * 16 * MT; e += SK_WAVES * 64) {
     const int nl = e % NB, m = e / NB;
     const float v = total(nl, m);
@@ -198,9 +209,9 @@ gemm_skinny_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float
     float xn = 0.f;
     if (n < N && m < M) {
       float* c = C + (size_t)m * N + n;
-      xn = (epilogue == EPI_ACCUMULATE) ? *c + v : v;
+      xn = (epilogue == EPI_ACCUMULATE) ? (one_each ? c_old : *c) + v : v;
       *c = xn;
-      if (writer) ns.xt[(size_t)m * N + n] = (bf16)(xn * ns.norm_w[n]);
+      if (writer) ns.xt[(size_t)m * N + n] = (bf16)(xn * (one_each ? w_norm : ns.norm_w[n]));
     }
     if (writer) {                  // whole waves get here: NB lanes in a row share m
       float q = xn * xn;
