@@ -350,7 +350,8 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
                    const int* __restrict__ row_pos, int nq, int nkv, int d, int window, float scale,
                    int n_splits, int head_groups, float* __restrict__ part, bf16* __restrict__ out) {
   constexpr int KB = DPAD / 32, VB = DPAD / 16;
-  __shared__ float red_o[VB * 4 * 64];
+  constexpr bool APART = DPAD <= 128;        // room in LDS for every wave's scaled O^T: one barrier instead of four
+  __shared__ float red_o[(APART ? DC_WAVES : 1) * VB * 4 * 64];
   __shared__ float red_ml[DC_WAVES][2][16];
   const int g = nq / nkv;
   const int hg = blockIdx.x % head_groups;
@@ -498,18 +499,35 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
 #pragma unroll
   for (int w = 0; w < DC_WAVES; ++w) mm = fmaxf(mm, red_ml[w][0][li]);
   const float f = (m == -INFINITY) ? 0.f : __expf(m - mm);
-  for (int w = 0; w < DC_WAVES; ++w) {
-    if (wave == w) {
+  if constexpr (APART) {
 #pragma unroll
-      for (int vb = 0; vb < VB; ++vb)
+    for (int vb = 0; vb < VB; ++vb)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          float* dst = &red_o[(vb * 4 + r) * 64 + lane];
-          *dst = (w == 0) ? o[vb][r] * f : *dst + o[vb][r] * f;
-        }
-    }
+      for (int r = 0; r < 4; ++r) red_o[wave * (VB * 4 * 64) + (vb * 4 + r) * 64 + lane] = o[vb][r] * f;
     __syncthreads();
+  } else {
+    for (int w = 0; w < DC_WAVES; ++w) {
+      if (wave == w) {
+#pragma unroll
+        for (int vb = 0; vb < VB; ++vb)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            float* dst = &red_o[(vb * 4 + r) * 64 + lane];
+            *dst = (w == 0) ? o[vb][r] * f : *dst + o[vb][r] * f;
+          }
+      }
+      __syncthreads();
+    }
   }
+  // the waves' shares in their order (the sum that the one-after-the-other way makes)
+  auto o_sum = [&](int idx) {
+    float v = red_o[idx];
+    if constexpr (APART) {
+#pragma unroll
+      for (int w = 1; w < DC_WAVES; ++w) v += red_o[w * (VB * 4 * 64) + idx];
+    }
+    return v;
+  };
   for (int e = threadIdx.x; e < 16 * DPAD; e += DC_WAVES * 64) {
     const int hd = e / DPAD, dv = e % DPAD;
     if (hg * 16 + hd >= g || dv >= d) continue;
@@ -525,11 +543,11 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
     const int idx = ((dv / 16) * 4 + (dv % 4)) * 64 + ((dv % 16) / 4) * 16 + hd;
     const size_t bh = (size_t)b * nq + kvh * g + hg * 16 + hd;
     if (n_splits == 1) {                                // nothing to merge with
-      out[bh * d + dv] = (bf16)(red_o[idx] / ll);
+      out[bh * d + dv] = (bf16)(o_sum(idx) / ll);
       continue;
     }
     float* dst = part + (bh * n_splits + split) * (d + 2);
-    dst[2 + dv] = red_o[idx];
+    dst[2 + dv] = o_sum(idx);
     if (dv == 0) {
       dst[0] = mh;
       dst[1] = ll;
