@@ -1,0 +1,32 @@
+"""The rules that choose a kernel's shape from the sizes: pure functions, tested without a GPU."""
+from torchless_rs_amd.kernels import ops
+
+
+def test_mid_splits_are_powers_of_two_that_fit():
+    for M in (17, 64, 128):
+        for N in (72, 4096, 6144, 28672, 32000):
+            for K in (48, 256, 1000, 4096, 14336):
+                S = ops.mid_splits(M, N, K)
+                steps = -(-K // 256)
+                assert S >= 1 and S & (S - 1) == 0, (M, N, K, S)
+                assert S <= max(1, steps) and S <= 16, (M, N, K, S)
+    # the 7B sizes: narrow outputs are cut in 8, the wide one is not cut
+    assert ops.mid_splits(64, 4096, 4096) == 8 and ops.mid_splits(64, 6144, 4096) == 8
+    assert ops.mid_splits(128, 4096, 14336) == 8 and ops.mid_splits(64, 28672, 4096) == 1
+    assert ops.mid_splits(20, 72, 48) == 1                  # one step of K: nothing to cut
+
+
+def test_decode_splits_follow_batch_and_length():
+    assert ops.decode_groups(8, 32, 8) == 64 and ops.decode_groups(1, 34, 2) == 4      # 17 heads a group: two tiles
+    assert ops.decode_splits(64, 32, 8, 32) == 1            # enough workgroups without a cut
+    assert ops.decode_splits(8, 32, 8, 65) == 8             # 64 groups: eight parts reach 512 workgroups
+    assert ops.decode_splits(1, 32, 8, 64) == 16            # at least four pages a part
+    assert ops.decode_splits(1, 32, 8, 1) == 1
+    for B in (1, 3, 8, 64):
+        for pages in (1, 4, 5, 64, 1100):
+            S = ops.decode_splits(B, 32, 8, pages)
+            assert 1 <= S <= max(1, -(-pages // ops.SPLIT_PAGES))
+
+
+def test_row_thresholds():
+    assert ops.LIBRARY_ROWS == 64 and ops.MID_ROWS == 128 and ops.MID_ROWS > ops.LIBRARY_ROWS
