@@ -47,6 +47,8 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64")
+    ap.add_argument("--no-tiled-copies", action="store_true",
+                    help="keep no second copies of q|k|v, o and down in the layout that single-token steps stream")
     ap.add_argument("--only", choices=["prefill", "decode"], default=None,
                     help="measure one phase only and print its line to stderr (for profiling)")
     args = ap.parse_args()
@@ -70,9 +72,10 @@ def main() -> int:
     t0 = time.time()
     tensors = random_tensors(model_spec_for(cfg).weight_specs(), seed=5, std=0.02,
                              dtype=torch.bfloat16, device=dev)
-    model = model_from_tensors(cfg, tensors, "bfloat16", dev)
+    model = model_from_tensors(cfg, tensors, "bfloat16", dev, tiled_copies=not args.no_tiled_copies)
     del tensors
     torch.cuda.synchronize()
+    resident_gib = round(torch.cuda.memory_allocated() / 2 ** 30, 2)     # weights and their tiled copies
     print(f"[bench] weights ready in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
 
     L, H, I, V = args.layers, cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
@@ -187,7 +190,8 @@ def main() -> int:
                    "intermediate_size": I, "vocab_size": V, "sliding_window": W,
                    "rope_theta": cfg.rope_theta, "rms_norm_eps": cfg.rms_norm_eps,
                    "global_batch": args.batch, "seq_len": args.context, "parallelism": "none",
-                   "sampling": "greedy"},
+                   "sampling": "greedy", "tiled_weight_copies": not args.no_tiled_copies,
+                   "weights_resident_gib": resident_gib},
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4)},

@@ -641,3 +641,40 @@ def test_random_configurations(tmp_path, seed):
         for s in slots:
             eng.free(s)
         assert worst < TOL[dtype], (cfg, lens, tail, dtype, worst)
+
+
+def test_tiled_weight_copies_change_no_bit(tmp_path):
+    """Sizes at which q|k|v, o and down all have their tiled copies: single-token steps read
+    them, and give the bits they give from the weights as stored, and the plain logits."""
+    from torchless_rs_amd import write_random_model
+    from torchless_rs_amd.engine import Engine, SeqInput, load_model
+    cfg = {"architectures": ["MistralForCausalLM"], "model_type": "mistral", "num_hidden_layers": 2,
+           "hidden_size": 128, "num_attention_heads": 4, "num_key_value_heads": 2, "head_dim": 32,
+           "intermediate_size": 192, "vocab_size": 300, "rope_theta": 10000.0, "sliding_window": 40,
+           "rms_norm_eps": 1e-5, "max_position_embeddings": 256, "tie_word_embeddings": False, "hidden_act": "silu"}
+    mdir = write_random_model(str(tmp_path / "m"), cfg, seed=5, std=0.05, norm_std=0.1, dtype=torch.bfloat16)
+    cfgd, w = read_model_dir(mdir)
+    ids = prompts(cfg["vocab_size"], [70, 9, 33], seed=77)
+    wants = [plain.forward(w, cfgd, p, dtype=torch.float32) for p in ids]
+    tail = 20
+    runs = {}
+    for tiled in (True, False):
+        model = load_model(mdir, "bfloat16", tiled_copies=tiled)
+        for blk in model.blocks:
+            copies = [blk.mixer.qkv.own_tiles, blk.mixer.o.tiles, blk.ffn.down.tiles]
+            assert all((c is not None) == tiled for c in copies)
+            assert blk.mixer.qkv.tiles is None and blk.ffn.gate_up.tiles is None
+        eng = Engine(model, max_tokens=64 * 6)
+        slots = [eng.alloc() for _ in ids]
+        heads = [max(1, len(p) - tail) for p in ids]
+        outs = [eng.step([SeqInput(s, p[:h], [h - 1]) for s, p, h in zip(slots, ids, heads)]).clone()]
+        for t in range(tail):
+            live = [i for i in range(len(ids)) if heads[i] + t < len(ids[i])]
+            outs.append(eng.step([SeqInput(slots[i], [ids[i][heads[i] + t]], [0]) for i in live]).clone())
+            for r, i in enumerate(live):
+                assert rel_err(outs[-1][r:r + 1], wants[i][heads[i] + t:heads[i] + t + 1]) < TOL["bfloat16"]
+        for s in slots:
+            eng.free(s)
+        runs[tiled] = outs
+    for a, b in zip(runs[True], runs[False]):
+        assert torch.equal(a, b)

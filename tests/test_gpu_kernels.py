@@ -712,6 +712,95 @@ def test_qkv_rope_commit_with_row_factor(ops):
         assert rel_err(pages[pg, 1].reshape(nkv, d, 64)[:, :, p % 64], full[b, nq + nkv:]) < KTOL["bfloat16"]
 
 
+# ---- the tiled copy of a weight that steps of at most 16 rows stream from ---------------------
+
+def tiled_by_formula(w, rows=None):
+    """[N/16, K/64, 2, 16, 4, 8] with (T, s, c, r, g, e) = w[rows[16 T + r], 64 s + 16 g + 8 c + e]."""
+    N, K = w.shape
+    src = w if rows is None else w[rows.long()]
+    return src.view(N // 16, 16, K // 64, 4, 2, 8).permute(0, 2, 4, 1, 3, 5).contiguous()
+
+
+@pytest.mark.parametrize("N,K", [(16, 64), (48, 192), (4112, 320)])
+def test_tile_weights(ops, N, K):
+    w = rnd(N, K, seed=61, dtype=torch.bfloat16).to(DEV)
+    assert torch.equal(ops.tile_weights(w), tiled_by_formula(w))
+    rows = torch.randperm(N, generator=torch.Generator().manual_seed(62)).to(torch.int32).to(DEV)
+    assert torch.equal(ops.tile_weights(w, rows), tiled_by_formula(w, rows))
+    for bad in (w[:, : K - 8].contiguous(), w[: N - 8].contiguous()):
+        with pytest.raises(ops.KernelError, match="multiple of 16"):
+            ops.tile_weights(bad)
+    assert ops.tiles_fit(N, K) and not ops.tiles_fit(N + 8, K) and not ops.tiles_fit(N, K + 32)
+
+
+@pytest.mark.parametrize("M", [1, 7, 16])
+@pytest.mark.parametrize("N,K", [(16, 64), (48, 192), (4112, 320), (96, 4096)])
+def test_products_from_the_tiled_copy_give_the_same_bits(ops, M, N, K):
+    """The same values meet in the same MFMAs in the same order, wherever they were read from."""
+    a = rnd(M, K, seed=63, dtype=torch.bfloat16).to(DEV)
+    w = rnd(N, K, seed=64, dtype=torch.bfloat16).to(DEV)
+    tiles = ops.tile_weights(w)
+    x0 = rnd(M, N, seed=65).to(DEV)
+    for accumulate in (False, True):
+        got, want = x0.clone(), x0.clone()
+        ops.gemm_bf16(a, w, want, accumulate=accumulate)
+        ops.gemm_bf16(a, w, got, accumulate=accumulate, tiles=tiles)
+        assert torch.equal(got, want)
+        assert rel_err(got, (x0.double().cpu() if accumulate else 0) + a.double().cpu() @ w.double().cpu().t()) < 1e-5
+    # with both halves of a norm around it
+    g = (1 + 0.2 * rnd(N, seed=66)).to(DEV)
+    res = []
+    for t in (None, tiles):
+        x = x0.clone()
+        xt = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ssq = torch.full((16, N // 16), float("nan"), device=DEV)
+        groups = ops.gemm_bf16_norm(a, w, x, accumulate=True, norm_weight=g, xt=xt, ssq_out=ssq, tiles=t)
+        res.append((x, xt, ssq[:M].clone(), groups))
+    assert res[0][3] == res[1][3] == N // 16
+    for u, v in zip(res[0][:3], res[1][:3]):
+        assert torch.equal(u, v)
+    ssq_in = (torch.rand(16, 3, generator=torch.Generator().manual_seed(67)) * K).to(DEV)
+    factor = ops.RowFactor(ssq_in, 3, K, 1e-5)
+    o1, o2 = torch.empty(M, N, device=DEV), torch.empty(M, N, device=DEV)
+    ops.gemm_bf16_norm(a, w, o1, factor=factor)
+    ops.gemm_bf16_norm(a, w, o2, factor=factor, tiles=tiles)
+    assert torch.equal(o1, o2)
+    # a copy of another weight's shape is refused
+    with pytest.raises(ops.KernelError, match="tiles"):
+        ops.gemm_bf16(a, w, o1, tiles=tiles.view(-1)[: tiles.numel() // 2].clone())
+
+
+@pytest.mark.parametrize("nq,nkv,d,K,lens", [(6, 2, 48, 64, [0, 63, 64, 300]), (4, 4, 16, 320, [5]), (3, 1, 256, 128, [7, 200]),
+                                             (8, 2, 128, 1024, [9, 64, 127, 128, 640, 2, 3, 4, 5, 6, 7, 8, 70, 71, 72, 73])])
+def test_qkv_rope_commit_from_the_tiled_copy(ops, nq, nkv, d, K, lens):
+    from torchless_rs_amd.parts.position import Rotary
+    n = len(lens)
+    c = paged_case(ops, "bfloat16", nq, nkv, d, None, lens_cached=lens, lens_new=[1] * n, seed=19, n_pages=60)
+    y = rnd(n, K, seed=20, dtype=torch.bfloat16).to(DEV)
+    w = rnd((nq + 2 * nkv) * d, K, seed=21, dtype=torch.bfloat16, scale=0.2).to(DEV)
+    inv = Rotary(d, 10000.0).inv_freq(DEV)
+    rows = ops.qkv_tile_rows(nq, nkv, d, DEV)
+    assert sorted(rows.tolist()) == list(range((nq + 2 * nkv) * d))
+    head0 = rows[:16].tolist()                       # a tile of a rotated head: 8 channels and their partners
+    assert head0 == list(range(8)) + list(range(d // 2, d // 2 + 8))
+    v0 = (nq + nkv) * d
+    assert rows[v0:v0 + 16].tolist() == list(range(v0, v0 + 16))
+    tiles = ops.tile_weights(w, rows)
+    ssq_in = (torch.rand(16, 4, generator=torch.Generator().manual_seed(22)) * K).to(DEV)
+    for factor in (None, ops.RowFactor(ssq_in, 4, K, 1e-6)):
+        for kv_half in (None, False, True):
+            out = []
+            for t in (None, tiles):
+                q = torch.full((n, nq, d), float("nan"), dtype=torch.bfloat16, device=DEV)
+                pages = c["pages"].clone()
+                ops.qkv_rope_commit(y, w, c["row_pos"], inv, c["table"], c["ring"], nq, nkv, d, q, pages,
+                                    factor=factor, kv_half=kv_half, tiles=t)
+                out.append((q, torch.nan_to_num(pages.float(), nan=-7.0)))
+            assert torch.equal(out[0][0], out[1][0])
+            assert torch.equal(out[0][1], out[1][1])
+    assert not torch.equal(out[1][1], torch.nan_to_num(c["pages"].float(), nan=-7.0))
+
+
 # ---- 17..128 rows: shared activations, K cut into partial sums (above 64 rows the k-step is 128) --
 
 @pytest.mark.parametrize("M", [17, 32, 33, 48, 50, 64, 5, 65, 80, 97, 112, 128])

@@ -7,7 +7,9 @@
 //    between them and every lane keeps several 16-byte loads in flight; the
 //    partial sums meet in LDS.  The activations are the other operand, read
 //    through the caches.  A row's result does not depend on M.  The epilogue
-//    may carry the halves of an RMSNorm (NormSplit).
+//    may carry the halves of an RMSNorm (NormSplit).  It can also read W from a
+//    copy laid out in tiles (see tile_weights_kernel): a wave's loads are then one
+//    run of consecutive bytes, which the memory serves faster than 16 rows apart.
 //  * gemm_qkv_rope_commit: the skinny product for the fused q|k|v projection of
 //    single-token steps, with rotation and the write into the cache's pages.
 //  * gemm_mid: 17..128 rows.  The activations of a k-step are shared by the four
@@ -88,8 +90,29 @@ struct RowFactors {
   }
 };
 
+// ----------------------------------------------------------- tiled copy ----
+// The copy of W [N, K] that the kernels for at most 16 rows stream from, when N % 16 == 0 and
+// K % 64 == 0: [N/16 tiles][K/64 steps][2 halves][16 rows][4 groups][8], where element
+// (tile T, step s, half c, row r, group g, e) is W[rows[16 T + r]][64 s + 16 g + 8 c + e]
+// (`rows`: a permutation of the rows, or null for none).  One MFMA operand of a wave (row r
+// = lane % 16, group g = lane / 16, 8 values) is then 1 KB of consecutive memory, a step 2 KB,
+// and a tile's steps follow each other.
+constexpr int TILE_STEP = 1024;        // elements of one tile's step
+
+__global__ void __launch_bounds__(256)
+tile_weights_kernel(const bf16* __restrict__ W, const int* __restrict__ rows, int N, int K, bf16* __restrict__ Wt) {
+  const size_t chunks = (size_t)N * K / 8;
+  for (size_t c = (size_t)blockIdx.x * 256 + threadIdx.x; c < chunks; c += (size_t)gridDim.x * 256) {
+    const int g = c % 4, r = (c / 4) % 16, half = (c / 64) % 2;
+    const size_t step = (c / 128) % (K / 64), tile = c / 128 / (K / 64);
+    const int row = rows ? rows[tile * 16 + r] : (int)(tile * 16 + r);
+    *reinterpret_cast<bf16x8*>(Wt + c * 8) = load8(W + (size_t)row * K + step * 64 + 16 * g + 8 * half);
+  }
+}
+
 // ---------------------------------------------------------------- skinny ----
-template <int NT, int MT, int SK_WAVES, bool FULLK>      // FULLK: K % 64 == 0, no load needs a guard (and a branch)
+// TILED: W is the tiled copy (N % 16 == 0, K % 64 == 0, hence FULLK)
+template <int NT, int MT, int SK_WAVES, bool FULLK, bool TILED = false>      // FULLK: K % 64 == 0, no load needs a guard (and a branch)
 __global__ void __launch_bounds__(SK_WAVES * 64)
 gemm_skinny_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float* __restrict__ C, int M,
                    int N, int K, int epilogue, NormSplit ns) {
@@ -106,7 +129,9 @@ gemm_skinny_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float
   const bf16* wrow[NT];
   const bf16* arow[MT];
 #pragma unroll
-  for (int t = 0; t < NT; ++t) wrow[t] = W + (size_t)min(n0 + t * 16 + li, N - 1) * K;
+  for (int t = 0; t < NT; ++t)
+    wrow[t] = TILED ? W + (size_t)(n0 / 16 + t) * 16 * K + li * 32 + kg * 8
+                    : W + (size_t)min(n0 + t * 16 + li, N - 1) * K;
 #pragma unroll
   for (int u = 0; u < MT; ++u) arow[u] = A + (size_t)min(u * 16 + li, M - 1) * K;
 
@@ -122,8 +147,13 @@ gemm_skinny_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float
     const bool ok0 = FULLK || k + 8 <= K, ok1 = FULLK || k + 16 <= K;
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-      wv[t][0] = ok0 ? load8(wrow[t] + k) : zero8();
-      wv[t][1] = ok1 ? load8(wrow[t] + k + 8) : zero8();
+      if constexpr (TILED) {
+        wv[t][0] = load8(wrow[t] + (size_t)s * TILE_STEP);
+        wv[t][1] = load8(wrow[t] + (size_t)s * TILE_STEP + TILE_STEP / 2);
+      } else {
+        wv[t][0] = ok0 ? load8(wrow[t] + k) : zero8();
+        wv[t][1] = ok1 ? load8(wrow[t] + k + 8) : zero8();
+      }
     }
 #pragma unroll
     for (int u = 0; u < MT; ++u) {
@@ -222,10 +252,19 @@ gemm_skinny_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float
   }
 }
 
+static bool tiles_fit(int N, int K) { return N % 16 == 0 && K % 64 == 0; }
+
 template <int NT, int MT, int SK_WAVES = 8>
 static int launch_skinny(const bf16* A, const bf16* W, float* C, int M, int N, int K, int epilogue,
-                         hipStream_t st, NormSplit ns = NormSplit{}) {
+                         hipStream_t st, NormSplit ns = NormSplit{}, const bf16* Wt = nullptr) {
   const int grid = (N + 16 * NT - 1) / (16 * NT);
+  if constexpr (NT == 1 && MT == 1 && SK_WAVES == 8) {
+    if (Wt != nullptr && tiles_fit(N, K)) {
+      gemm_skinny_kernel<NT, MT, SK_WAVES, true, true><<<grid, SK_WAVES * 64, 0, st>>>(A, Wt, C, M, N, K, epilogue, ns);
+      TL_LAUNCH_CHECK("gemm_skinny");
+      return 0;
+    }
+  }
   if (K % 64 == 0)
     gemm_skinny_kernel<NT, MT, SK_WAVES, true><<<grid, SK_WAVES * 64, 0, st>>>(A, W, C, M, N, K, epilogue, ns);
   else
@@ -246,8 +285,11 @@ static int launch_skinny(const bf16* A, const bf16* W, float* C, int M, int N, i
 // the compute units (7B: 384 tiles are one and a half a unit, 256 + 256 are two for all).
 // The sums and the rotation are those of the unfused kernels, bit for bit
 // (a' = a c - b s; b' = a s + b c; src/kernels/mod.rs:603-605 of the reference).
+// TILED: W is the tiled copy whose tile (head, t) holds the 16 channels named above in that
+// order (`tl_qkv_tile_rows`), so a half tile is rows np*sub.. and 8 + np*sub.. of its tile.
 constexpr int QKV_WAVES = 8;
 
+template <bool TILED>
 __global__ void __launch_bounds__(QKV_WAVES * 64)
 gemm_qkv_rope_commit_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, int M, int K,
                             const int* __restrict__ row_pos, const float* __restrict__ inv_freq,
@@ -277,7 +319,16 @@ gemm_qkv_rope_commit_kernel(const bf16* __restrict__ A, const bf16* __restrict__
   const bool rotated = head < nq + nkv;
   const bool loads = li < 2 * np;               // rows of the MFMA tile that hold a channel
   const int ch = rotated ? (li < np ? np * tt + li : half + np * tt + li - np) : 2 * np * tt + li;
-  const bf16* wrow = W + ((size_t)head * d + (loads ? ch : 0)) * K;
+  const bf16* wrow;
+  if constexpr (TILED) {
+    // the tile that holds this (half) tile's channels, and this lane's row in it
+    const int sub = np == 8 ? 0 : tt % 2;
+    const int tile = head * (d / 16) + (np == 8 ? tt : tt / 2);
+    const int r = rotated ? (li < np ? np * sub + li : 8 + np * sub + li - np) : 2 * np * sub + li;
+    wrow = W + (size_t)tile * 16 * K + (loads ? r : 0) * 32 + kg * 8;
+  } else {
+    wrow = W + ((size_t)head * d + (loads ? ch : 0)) * K;
+  }
   const bf16* arow = A + (size_t)min(li, M - 1) * K;
   const int steps = (K + 63) / 64;
   const int per = (steps + QKV_WAVES - 1) / QKV_WAVES;
@@ -287,8 +338,13 @@ gemm_qkv_rope_commit_kernel(const bf16* __restrict__ A, const bf16* __restrict__
   auto load_step = [&](int s, bf16x8 (&wv)[2], bf16x8 (&av)[2]) {
     const int k = s * 64 + kg * 16;
     const bool ok0 = k + 8 <= K, ok1 = k + 16 <= K;
-    wv[0] = (ok0 && loads) ? load8(wrow + k) : zero8();
-    wv[1] = (ok1 && loads) ? load8(wrow + k + 8) : zero8();
+    if constexpr (TILED) {
+      wv[0] = loads ? load8(wrow + (size_t)s * TILE_STEP) : zero8();
+      wv[1] = loads ? load8(wrow + (size_t)s * TILE_STEP + TILE_STEP / 2) : zero8();
+    } else {
+      wv[0] = (ok0 && loads) ? load8(wrow + k) : zero8();
+      wv[1] = (ok1 && loads) ? load8(wrow + k + 8) : zero8();
+    }
     av[0] = ok0 ? load8(arow + k) : zero8();
     av[1] = ok1 ? load8(arow + k + 8) : zero8();
   };
@@ -757,12 +813,14 @@ static int launch_big(const bf16* A, const bf16* W, float* C, int M, int N, int 
 using namespace tl;
 
 // epilogue: 0 store float, 1 accumulate into float, 2 silu(gate) * up into bfloat16 [M, N/2]
-// (W's rows in groups of 64: 32 gate rows and their 32 up rows; N a multiple of 64)
-extern "C" int tl_gemm_bf16(const void* A, const void* W, void* C, int M, int N, int K, int epilogue,
+// (W's rows in groups of 64: 32 gate rows and their 32 up rows; N a multiple of 64).
+// Wt (or null): the tiled copy of W, see tl_gemm_bf16_norm.
+extern "C" int tl_gemm_bf16(const void* A, const void* W, const void* Wt, void* C, int M, int N, int K, int epilogue,
                             hipStream_t st) {
   TL_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_bf16: bad sizes M=%d N=%d K=%d", M, N, K);
   TL_REQUIRE(K % 8 == 0, "gemm_bf16: K=%d must be a multiple of 8", K);
-  TL_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "gemm_bf16: operands must be 16-byte aligned");
+  TL_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0) && ((uintptr_t)Wt % 16 == 0),
+             "gemm_bf16: operands must be 16-byte aligned");
   TL_REQUIRE(epilogue >= 0 && epilogue <= 2, "gemm_bf16: unknown epilogue %d", epilogue);
   TL_REQUIRE(epilogue != EPI_SILU_PAIR || N % 64 == 0, "gemm_bf16: the paired epilogue needs N=%d to be "
              "a multiple of 64", N);
@@ -773,7 +831,7 @@ extern "C" int tl_gemm_bf16(const void* A, const void* W, void* C, int M, int N,
   const bool wide = N >= 16384 || epilogue == EPI_SILU_PAIR;     // many rows: 64 a workgroup
   if (M <= 16) {
     if (wide && (M > 4 || epilogue == EPI_SILU_PAIR)) return launch_skinny<4, 1, 4>(a, w, c, M, N, K, epilogue, st);
-    return launch_skinny<1, 1, 8>(a, w, c, M, N, K, epilogue, st);
+    return launch_skinny<1, 1, 8>(a, w, c, M, N, K, epilogue, st, NormSplit{}, (const bf16*)Wt);
   }
   if (M <= 32) {
     if (wide) return launch_skinny<4, 2, 4>(a, w, c, M, N, K, epilogue, st);
@@ -856,7 +914,9 @@ extern "C" int tl_gemm_mid_bf16(const void* A, const void* W, void* C, int M, in
 // W is [(nq + 2 nkv) d, K]; q receives [M, nq, d], the pages k and v of the new position.
 // With ssq_in, row m's sums are multiplied by rsqrt(sum_j ssq_in[m][j] * inv_h + eps) first.
 // kv_half: 1 halves the tiles of k and v heads, 0 does not, -1 lets the launcher choose.
-extern "C" int tl_gemm_qkv_rope_commit(const void* A, const void* W, int M, int K, const int* row_pos,
+// Wt (or null): the tiled copy of W with the rows of `tl_qkv_tile_rows`, read instead of W
+// when K % 64 == 0.
+extern "C" int tl_gemm_qkv_rope_commit(const void* A, const void* W, const void* Wt, int M, int K, const int* row_pos,
                                        const float* inv_freq, const int* table, int table_stride,
                                        int ring_pages, int nq, int nkv, int d, void* q, void* pages,
                                        const float* ssq_in, int n_part, float inv_h, float eps,
@@ -886,9 +946,16 @@ extern "C" int tl_gemm_qkv_rope_commit(const void* A, const void* W, int M, int 
   const int grid = kv_half ? mixed : full;
   NormSplit ns{};
   ns.ssq_in = ssq_in; ns.n_part = n_part; ns.inv_h = inv_h; ns.eps = eps;
-  gemm_qkv_rope_commit_kernel<<<grid, QKV_WAVES * 64, 0, st>>>((const bf16*)A, (const bf16*)W, M, K, row_pos,
-                                                              inv_freq, table, table_stride, ring_pages, nq,
-                                                              nkv, d, (bf16*)q, (bf16*)pages, ns, kv_half);
+  if (Wt != nullptr && K % 64 == 0) {
+    TL_REQUIRE((uintptr_t)Wt % 16 == 0, "qkv_rope_commit: operands must be 16-byte aligned");
+    gemm_qkv_rope_commit_kernel<true><<<grid, QKV_WAVES * 64, 0, st>>>(
+        (const bf16*)A, (const bf16*)Wt, M, K, row_pos, inv_freq, table, table_stride, ring_pages, nq, nkv, d,
+        (bf16*)q, (bf16*)pages, ns, kv_half);
+  } else {
+    gemm_qkv_rope_commit_kernel<false><<<grid, QKV_WAVES * 64, 0, st>>>(
+        (const bf16*)A, (const bf16*)W, M, K, row_pos, inv_freq, table, table_stride, ring_pages, nq, nkv, d,
+        (bf16*)q, (bf16*)pages, ns, kv_half);
+  }
   TL_LAUNCH_CHECK("gemm_qkv_rope_commit");
   return 0;
 }
@@ -897,8 +964,10 @@ extern "C" int tl_gemm_qkv_rope_commit(const void* A, const void* W, int M, int 
 // ssq_in [16][n_part] (or null): a factor per row on the results.  norm_w [N], xt [M][N],
 // ssq_out [16][workgroups] (or all null): with the accumulate epilogue, also write
 // xt = bfloat16(C * norm_w) and the workgroups' sums of C^2; *n_groups receives the number
-// of workgroups, which is the n_part of the product that reads xt.
-extern "C" int tl_gemm_bf16_norm(const void* A, const void* W, void* C, int M, int N, int K, int epilogue,
+// of workgroups, which is the n_part of the product that reads xt.  Wt (or null): the tiled
+// copy of W (rows in their own order), read instead of W by the kernel with 16 channels a
+// workgroup when N % 16 == 0 and K % 64 == 0.
+extern "C" int tl_gemm_bf16_norm(const void* A, const void* W, const void* Wt, void* C, int M, int N, int K, int epilogue,
                                  const float* ssq_in, int n_part, float inv_h, float eps,
                                  const float* norm_w, void* xt, float* ssq_out, int ssq_capacity,
                                  int* n_groups, hipStream_t st) {
@@ -923,5 +992,31 @@ extern "C" int tl_gemm_bf16_norm(const void* A, const void* W, void* C, int M, i
   ns.ssq_in = ssq_in; ns.n_part = n_part; ns.inv_h = inv_h; ns.eps = eps;
   ns.norm_w = norm_w; ns.xt = (bf16*)xt; ns.ssq_out = ssq_out;
   if (four) return launch_skinny<4, 1, 4>((const bf16*)A, (const bf16*)W, (float*)C, M, N, K, epilogue, st, ns);
-  return launch_skinny<1, 1, 8>((const bf16*)A, (const bf16*)W, (float*)C, M, N, K, epilogue, st, ns);
+  TL_REQUIRE((uintptr_t)Wt % 16 == 0, "gemm_bf16_norm: operands must be 16-byte aligned");
+  return launch_skinny<1, 1, 8>((const bf16*)A, (const bf16*)W, (float*)C, M, N, K, epilogue, st, ns, (const bf16*)Wt);
+}
+
+// Wt [N/16][K/64][2][16][4][8] = the tiled copy of W [N, K] (N % 16 == 0, K % 64 == 0) with its
+// rows taken in the order `rows` [N] (null: as they are).
+extern "C" int tl_tile_weights(const void* W, const int* rows, int N, int K, void* Wt, hipStream_t st) {
+  TL_REQUIRE(N > 0 && K > 0 && tiles_fit(N, K), "tile_weights: N=%d must be a multiple of 16 and K=%d of 64", N, K);
+  TL_REQUIRE(((uintptr_t)W % 16 == 0) && ((uintptr_t)Wt % 16 == 0), "tile_weights: operands must be 16-byte aligned");
+  const size_t chunks = (size_t)N * K / 8;
+  const int grid = (chunks + 255) / 256 < 8192 ? (int)((chunks + 255) / 256) : 8192;
+  tile_weights_kernel<<<grid, 256, 0, st>>>((const bf16*)W, rows, N, K, (bf16*)Wt);
+  TL_LAUNCH_CHECK("tile_weights");
+  return 0;
+}
+
+// The order of W's rows in the tiled copy that tl_gemm_qkv_rope_commit reads: tile t of a q or
+// k head holds channels 8t..8t+7 and d/2+8t..d/2+8t+7, v heads keep theirs.  rows: [(nq + 2 nkv) d], host.
+extern "C" int tl_qkv_tile_rows(int nq, int nkv, int d, int* rows) {
+  TL_REQUIRE(nq > 0 && nkv > 0 && d >= 16 && d % 16 == 0, "qkv_tile_rows: bad heads nq=%d nkv=%d d=%d", nq, nkv, d);
+  for (int head = 0; head < nq + 2 * nkv; ++head)
+    for (int t = 0; t < d / 16; ++t)
+      for (int r = 0; r < 16; ++r) {
+        const int ch = head < nq + nkv ? (r < 8 ? 8 * t + r : d / 2 + 8 * t + r - 8) : 16 * t + r;
+        rows[(head * (d / 16) + t) * 16 + r] = head * d + ch;
+      }
+  return 0;
 }

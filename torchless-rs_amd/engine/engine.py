@@ -56,27 +56,28 @@ def require_gpu(device) -> torch.device:
     return device
 
 
-def load_model(model_dir: str, dtype="bfloat16", device="cuda:0") -> Model:
+def load_model(model_dir: str, dtype="bfloat16", device="cuda:0", tiled_copies: bool = True) -> Model:
     """A model from a folder with config.json and safetensors; the class of
-    the configuration and the parts follow from config.json's architecture."""
+    the configuration and the parts follow from config.json's architecture.
+    `tiled_copies`: see `Model.load_weights`."""
     from ..models import model_spec_for
     from ..kernels.build import load as load_kernels
     device = require_gpu(device)
     load_kernels()                                   # fail here, loudly, if it cannot be had
     cfg = load_config(model_dir)
     model = Model(model_spec_for(cfg), cfg, resolve_dtype(dtype), device)
-    model.load_weights(ModelFiles(model_dir))
+    model.load_weights(ModelFiles(model_dir), tiled_copies)
     return model
 
 
 def model_from_tensors(config: ModelConfig, tensors: Dict[str, torch.Tensor], dtype="bfloat16",
-                       device="cuda:0") -> Model:
+                       device="cuda:0", tiled_copies: bool = True) -> Model:
     from ..models import model_spec_for
     from ..kernels.build import load as load_kernels
     device = require_gpu(device)
     load_kernels()
     model = Model(model_spec_for(config), config, resolve_dtype(dtype), device)
-    model.load_weights(TensorDict(tensors))
+    model.load_weights(TensorDict(tensors), tiled_copies)
     return model
 
 

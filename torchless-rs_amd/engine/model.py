@@ -42,9 +42,18 @@ class Model:
         self.graph_safe = all(p.graph_safe for p in [self.embedding, self.final_norm, self.head] + self.blocks)
 
     # ---- weights -----------------------------------------------------------
-    def load_weights(self, source) -> None:
+    def load_weights(self, source, tiled_copies: bool = True) -> None:
         """`source`: anything with names/shape/dtype/tensor (a model folder's
-        files, or tensors in memory)."""
+        files, or tensors in memory).  `tiled_copies`: may the parts keep second
+        copies of weights in the layout that single-token steps stream fastest?"""
+        from ..parts.linear import Linear
+        before, Linear.tiled_copies = Linear.tiled_copies, bool(tiled_copies)
+        try:
+            self._load_parts(source)
+        finally:
+            Linear.tiled_copies = before
+
+    def _load_parts(self, source) -> None:
         spec = self.spec
         t = bind_weights(spec.weight_specs(), source, self.dtype, self.device, spec.ignore_tensors)
 

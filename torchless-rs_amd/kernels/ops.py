@@ -273,17 +273,57 @@ def sample(logits: torch.Tensor, temperature: float, top_k: int, top_p: float, s
 EPI_STORE, EPI_ACCUMULATE, EPI_SILU_PAIR = 0, 1, 2
 
 
+def tiles_fit(N: int, K: int) -> bool:
+    """Can a weight [N, K] have a tiled copy?"""
+    return N % 16 == 0 and K % 64 == 0
+
+
+def tile_weights(w: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The copy of w [N, K] (bfloat16, N % 16 == 0, K % 64 == 0) that the products for at most
+    16 rows stream from: [N/16, K/64, 2, 16, 4, 8] with element (T, s, c, r, g, e) =
+    w[rows[16 T + r], 64 s + 16 g + 8 c + e], so that what a wave loads at a time lies in one
+    run of memory.  `rows` (int32 [N], on the device): a permutation of the rows; None: none."""
+    N, K = w.shape
+    _req(w, "tile_weights.w", torch.bfloat16)
+    if not tiles_fit(N, K):
+        raise KernelError(f"tile_weights: N={N} must be a multiple of 16 and K={K} of 64")
+    if rows is not None:
+        _req(rows, "tile_weights.rows", torch.int32, (N,))
+    out = torch.empty((N // 16, K // 64, 2, 16, 4, 8), dtype=torch.bfloat16, device=w.device)
+    _check(lib().tl_tile_weights(_p(w), _p(rows), N, K, _p(out), _stream()))
+    return out
+
+
+def qkv_tile_rows(nq: int, nkv: int, d: int, device) -> torch.Tensor:
+    """The order of the rows of w = q|k|v in the tiled copy that `qkv_rope_commit` reads
+    (a tile of a q or k head holds both halves of 8 rotated pairs)."""
+    n = (nq + 2 * nkv) * d
+    buf = (ctypes.c_int * n)()
+    _check(lib().tl_qkv_tile_rows(int(nq), int(nkv), int(d), buf))
+    return torch.tensor(list(buf), dtype=torch.int32, device=device)
+
+
+def _req_tiles(tiles: Optional[torch.Tensor], N: int, K: int) -> None:
+    if tiles is not None:
+        _req(tiles, "gemm.tiles", torch.bfloat16, (N // 16, K // 64, 2, 16, 4, 8))
+        if not tiles_fit(N, K):
+            raise KernelError(f"gemm.tiles: a weight [{N}, {K}] has no tiled copy")
+
+
 def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False,
-              variant: Optional[int] = None, silu_pair: bool = False) -> None:
+              variant: Optional[int] = None, silu_pair: bool = False,
+              tiles: Optional[torch.Tensor] = None) -> None:
     """out[M,N] (+)= a[M,K] @ w[N,K]^T on the matrix cores: bfloat16 operands,
     float32 accumulation.  K must be a multiple of 8.  With `silu_pair`, w's
     rows come in groups of 64 (32 gate rows and the 32 up rows that belong to
     them) and out is bfloat16 [M, N/2] = silu(gate) * up.  `variant` (tests
-    and tuning) forces one kernel."""
+    and tuning) forces one kernel.  `tiles`: `tile_weights(w)`, read instead of
+    w by the kernel for at most 16 rows and 16 channels a workgroup."""
     M, K = a.shape
     N = w.shape[0]
     _req(a, "gemm.a", torch.bfloat16)
     _req(w, "gemm.w", torch.bfloat16, (N, K))
+    _req_tiles(tiles, N, K)
     if silu_pair:
         if accumulate or N % 64:
             raise KernelError("gemm: the paired epilogue stores, and needs N to be a multiple of 64")
@@ -293,7 +333,7 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: b
         _req(out, "gemm.out", torch.float32, (M, N))
         epi = EPI_ACCUMULATE if accumulate else EPI_STORE
     if variant is None:
-        _check(lib().tl_gemm_bf16(_p(a), _p(w), _p(out), M, N, K, epi, _stream()))
+        _check(lib().tl_gemm_bf16(_p(a), _p(w), _p(tiles), _p(out), M, N, K, epi, _stream()))
     else:
         _check(lib().tl_gemm_bf16_variant(_p(a), _p(w), _p(out), M, N, K, epi, int(variant), _stream()))
 
@@ -315,16 +355,17 @@ def norm_split_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
 def gemm_bf16_norm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False,
                    silu_pair: bool = False, factor: Optional[RowFactor] = None,
                    norm_weight: Optional[torch.Tensor] = None, xt: Optional[torch.Tensor] = None,
-                   ssq_out: Optional[torch.Tensor] = None) -> int:
+                   ssq_out: Optional[torch.Tensor] = None, tiles: Optional[torch.Tensor] = None) -> int:
     """`gemm_bf16` for at most 16 rows with the halves of an RMSNorm around it.
     `factor`: every row of the result is multiplied by its rsqrt(mean(x^2) + eps).
     `norm_weight`, `xt`, `ssq_out` (with `accumulate`): out += product, xt =
     bfloat16(out * norm_weight), ssq_out[m, g] = the sum of out[m, :]^2 over workgroup g's
-    channels.  Returns the number of workgroups (the reader's n_part)."""
+    channels.  `tiles`: see `gemm_bf16`.  Returns the number of workgroups (the reader's n_part)."""
     M, K = a.shape
     N = w.shape[0]
     _req(a, "gemm.a", torch.bfloat16)
     _req(w, "gemm.w", torch.bfloat16, (N, K))
+    _req_tiles(tiles, N, K)
     if silu_pair:
         if accumulate or N % 64:
             raise KernelError("gemm: the paired epilogue stores, and needs N to be a multiple of 64")
@@ -346,7 +387,7 @@ def gemm_bf16_norm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumula
         _req(ssq_out, "gemm.ssq_out", torch.float32)
         cap = ssq_out.numel()
     groups = ctypes.c_int(0)
-    _check(lib().tl_gemm_bf16_norm(_p(a), _p(w), _p(out), M, N, K, epi, _p(ssq_in), n_part,
+    _check(lib().tl_gemm_bf16_norm(_p(a), _p(w), _p(tiles), _p(out), M, N, K, epi, _p(ssq_in), n_part,
                                    ctypes.c_float(inv_h), ctypes.c_float(eps), _p(norm_weight), _p(xt),
                                    _p(ssq_out), cap, ctypes.byref(groups), _stream()))
     return groups.value
@@ -447,16 +488,17 @@ def bf16_gemm_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
             and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
 
-def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
+def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False,
+         tiles: Optional[torch.Tensor] = None) -> None:
     """out[M,N] (+)= a[M,K] @ w[N,K]^T with float32 accumulation.  The kernel
     follows from the operand types: bfloat16 x bfloat16 goes to the matrix
     cores (our kernels up to LIBRARY_ROWS rows, the library's above), anything
-    with float32 in it to the plain FMA kernel."""
+    with float32 in it to the plain FMA kernel.  `tiles`: see `gemm_bf16`."""
     if bf16_gemm_ok(a, w):
         if a.shape[0] > LIBRARY_ROWS:
             gemm_library(a, w, out, accumulate)
         else:
-            gemm_bf16(a, w, out, accumulate)
+            gemm_bf16(a, w, out, accumulate, tiles=tiles)
     else:
         gemm_plain(a, w, out, accumulate)
 
@@ -489,14 +531,17 @@ def qkv_rope_commit_ok(a: torch.Tensor, w: torch.Tensor, d: int, pages: torch.Te
 
 def qkv_rope_commit(a: torch.Tensor, w: torch.Tensor, row_pos, inv_freq, table, ring_pages: int, nq: int,
                     nkv: int, d: int, q: torch.Tensor, pages: torch.Tensor,
-                    factor: Optional[RowFactor] = None, kv_half: Optional[bool] = None) -> None:
+                    factor: Optional[RowFactor] = None, kv_half: Optional[bool] = None,
+                    tiles: Optional[torch.Tensor] = None) -> None:
     """For a step with one token a sequence (at most 16): the product a @ w^T with w = q|k|v,
     the rotation of q and k, q into its buffer and k, v into the pages, in one kernel; the
     same bits as `gemm` and then `rope_commit`.  `factor`: see `gemm_bf16_norm`.  `kv_half`
-    (tests): force or forbid the smaller tiles for k and v that the launcher may choose."""
+    (tests): force or forbid the smaller tiles for k and v that the launcher may choose.
+    `tiles`: `tile_weights(w, qkv_tile_rows(nq, nkv, d))`, read instead of w."""
     n, K = a.shape
     _req(a, "qkv_rope_commit.a", torch.bfloat16)
     _req(w, "qkv_rope_commit.w", torch.bfloat16, ((nq + 2 * nkv) * d, K))
+    _req_tiles(tiles, (nq + 2 * nkv) * d, K)
     _req(row_pos, "qkv_rope_commit.row_pos", torch.int32, (n,))
     _req(inv_freq, "qkv_rope_commit.inv_freq", torch.float32, (d // 2,))
     _req(q, "qkv_rope_commit.q", torch.bfloat16, (n, nq, d))
@@ -512,7 +557,7 @@ def qkv_rope_commit(a: torch.Tensor, w: torch.Tensor, row_pos, inv_freq, table, 
         if factor.ssq.numel() < factor.n_part * 16 or factor.n_part < 1:
             raise KernelError(f"qkv_rope_commit.factor: {factor.ssq.numel()} floats for {factor.n_part} workgroups")
         ssq_in, n_part, inv_h, eps = factor.ssq, factor.n_part, 1.0 / factor.size, factor.eps
-    _check(lib().tl_gemm_qkv_rope_commit(_p(a), _p(w), n, K, _p(row_pos), _p(inv_freq), _p(table),
+    _check(lib().tl_gemm_qkv_rope_commit(_p(a), _p(w), _p(tiles), n, K, _p(row_pos), _p(inv_freq), _p(table),
                                          table.shape[1], int(ring_pages), nq, nkv, d, _p(q), _p(pages),
                                          _p(ssq_in), n_part, ctypes.c_float(inv_h), ctypes.c_float(eps),
                                          -1 if kv_half is None else int(kv_half), _stream()))
@@ -645,7 +690,7 @@ def measure_ceilings(device="cuda:0", gib: float = 8.0) -> dict:
     buf = torch.empty(n_bytes // 4, dtype=torch.float32, device=device).normal_()
     sink = torch.zeros(256 * 32, dtype=torch.float32, device=device)
     best_read = 0.0
-    for blocks in (256 * 4, 256 * 8, 256 * 16, 256 * 32):
+    for blocks in (256, 256 * 2, 256 * 4, 256 * 8, 256 * 16, 256 * 32):     # one workgroup a compute unit is the fastest
         for _ in range(3):
             torch.cuda.synchronize()
             t = time.perf_counter()

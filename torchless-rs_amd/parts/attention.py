@@ -66,8 +66,13 @@ class AttentionMixer(Mixer):
             ws += [tensors[p + "k_proj.weight"], tensors[p + "v_proj.weight"]]
         if len({w.dtype for w in ws}) > 1:
             ws = [w.to(torch.float32) for w in ws]
-        self.qkv = Linear(torch.cat(ws, dim=0))
-        self.o = Linear(tensors[p + "o_proj.weight"])
+        fused = torch.cat(ws, dim=0)
+        # single-token steps stream q|k|v and o from tiled copies; the fused q|k|v kernel has its own order of rows
+        rows = None
+        if self.own_kv and self.d % 16 == 0 and fused.is_cuda and fused.dtype == torch.bfloat16:
+            rows = ops.qkv_tile_rows(self.nq, self.nkv, self.d, fused.device)
+        self.qkv = Linear(fused, tiled=True, tile_rows=rows)
+        self.o = Linear(tensors[p + "o_proj.weight"], tiled=True)
 
     def forward(self, ctx, run, y: torch.Tensor, x: torch.Tensor) -> None:
         n, nq, nkv, d = y.shape[0], self.nq, self.nkv, self.d
@@ -85,7 +90,8 @@ class AttentionMixer(Mixer):
             # one token a sequence: k and v go straight into the pages, then everything is read there
             if fused:
                 ops.qkv_rope_commit(y, self.qkv.weight, ctx.row_pos, inv_freq, table, group.ring_pages,
-                                    nq, nkv, d, q, pages, factor=factor)     # product, rotation and commit in one
+                                    nq, nkv, d, q, pages, factor=factor,     # product, rotation and commit in one
+                                    tiles=self.qkv.own_tiles)
             else:
                 qkv = self.qkv.partial(y, ctx, "attn_qkv_parts")     # partial sums, added up by the rotation
                 if qkv is None:

@@ -42,7 +42,7 @@ class SwiGLU(FeedForward):
         self.paired = (compute_dtype == torch.bfloat16 and g.dtype == torch.bfloat16 and self.I % 32 == 0
                        and self.H % 8 == 0)
         self.gate_up = Linear(interleave_pairs(g, u) if self.paired else torch.cat([g, u], dim=0))
-        self.down = Linear(tensors[p + "down_proj.weight"])
+        self.down = Linear(tensors[p + "down_proj.weight"], tiled=True)
 
     def forward(self, ctx, y: torch.Tensor, x: torch.Tensor) -> None:
         n = y.shape[0]

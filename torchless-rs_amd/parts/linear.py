@@ -10,22 +10,37 @@ from ..kernels import ops
 
 
 class Linear:
-    """A weight [N, K] resident on the device in its stored width."""
+    """A weight [N, K] resident on the device in its stored width.  With `tiled` it
+    also keeps the tiled copy (`ops.tile_weights`) that the products of steps of at
+    most 16 rows read instead: memory spent for the rate at which decoding streams
+    the weights (`Linear.tiled_copies` switches all of them off).  `tile_rows`: the
+    copy's own order of rows, for a kernel that wants one; then only that kernel
+    reads it (`own_tiles`)."""
 
-    def __init__(self, weight: torch.Tensor):
+    tiled_copies = True
+
+    def __init__(self, weight: torch.Tensor, tiled: bool = False, tile_rows: torch.Tensor = None):
         assert weight.dim() == 2
         self.weight = weight.contiguous()
         self.out_features, self.in_features = self.weight.shape
+        self.tiles = self.own_tiles = None
+        if (tiled and Linear.tiled_copies and self.weight.is_cuda and self.weight.dtype == torch.bfloat16
+                and ops.tiles_fit(self.out_features, self.in_features)):
+            copy = ops.tile_weights(self.weight, tile_rows)
+            if tile_rows is None:
+                self.tiles = copy
+            else:
+                self.own_tiles = copy
 
     def __call__(self, a: torch.Tensor, out: torch.Tensor, accumulate: bool = False, factor=None) -> None:
         """out[M, N] (+)= a[M, K] @ W^T; out is float32.  `factor` (`ops.RowFactor`): the
         second half of the norm that made `a`, a factor per row (at most 16 rows)."""
         if factor is not None:
-            ops.gemm_bf16_norm(a, self.weight, out, accumulate, factor=factor)
+            ops.gemm_bf16_norm(a, self.weight, out, accumulate, factor=factor, tiles=self.tiles)
         elif self.mid(a) and a.shape[0] <= ops.LIBRARY_ROWS:
             ops.gemm_mid_bf16(a, self.weight, out, 1, accumulate)
         else:
-            ops.gemm(a, self.weight, out, accumulate)
+            ops.gemm(a, self.weight, out, accumulate, tiles=self.tiles)
 
     def mid(self, a: torch.Tensor) -> bool:
         """17..MID_ROWS rows of bfloat16: the kernel that shares the activations.
@@ -56,7 +71,7 @@ class Linear:
             xt = ctx.workspace.get("prenormed_y", (a.shape[0], self.out_features), torch.bfloat16)
             ssq = ctx.workspace.get(name + "_ssq", (16, -(-self.out_features // 16)), torch.float32)
             groups = ops.gemm_bf16_norm(a, self.weight, x, accumulate=True, norm_weight=norm.weight, xt=xt,
-                                        ssq_out=ssq)
+                                        ssq_out=ssq, tiles=self.tiles)
             ctx.prenormed = (norm, xt, ops.RowFactor(ssq, groups, norm.size, norm.eps))
             return
         parts = self.partial(a, ctx, name)
