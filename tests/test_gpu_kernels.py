@@ -715,10 +715,10 @@ def test_qkv_rope_commit_with_row_factor(ops):
 # ---- the tiled copy of a weight that steps of at most 16 rows stream from ---------------------
 
 def tiled_by_formula(w, rows=None):
-    """[N/16, K/64, 2, 16, 4, 8] with (T, s, c, r, g, e) = w[rows[16 T + r], 64 s + 16 g + 8 c + e]."""
+    """[N/16, K/64, 2, 4, 16, 8] with (T, s, c, g, r, e) = w[rows[16 T + r], 64 s + 16 g + 8 c + e]."""
     N, K = w.shape
     src = w if rows is None else w[rows.long()]
-    return src.view(N // 16, 16, K // 64, 4, 2, 8).permute(0, 2, 4, 1, 3, 5).contiguous()
+    return src.view(N // 16, 16, K // 64, 4, 2, 8).permute(0, 2, 4, 3, 1, 5).contiguous()
 
 
 @pytest.mark.parametrize("N,K", [(16, 64), (48, 192), (4112, 320)])

@@ -92,18 +92,18 @@ struct RowFactors {
 
 // ----------------------------------------------------------- tiled copy ----
 // The copy of W [N, K] that the kernels for at most 16 rows stream from, when N % 16 == 0 and
-// K % 64 == 0: [N/16 tiles][K/64 steps][2 halves][16 rows][4 groups][8], where element
-// (tile T, step s, half c, row r, group g, e) is W[rows[16 T + r]][64 s + 16 g + 8 c + e]
+// K % 64 == 0: [N/16 tiles][K/64 steps][2 halves][4 groups][16 rows][8], where element
+// (tile T, step s, half c, group g, row r, e) is W[rows[16 T + r]][64 s + 16 g + 8 c + e]
 // (`rows`: a permutation of the rows, or null for none).  One MFMA operand of a wave (row r
-// = lane % 16, group g = lane / 16, 8 values) is then 1 KB of consecutive memory, a step 2 KB,
-// and a tile's steps follow each other.
+// = lane % 16, group g = lane / 16, 8 values) is then 1 KB of consecutive memory in the order of
+// the lanes, a step 2 KB, and a tile's steps follow each other.
 constexpr int TILE_STEP = 1024;        // elements of one tile's step
 
 __global__ void __launch_bounds__(256)
 tile_weights_kernel(const bf16* __restrict__ W, const int* __restrict__ rows, int N, int K, bf16* __restrict__ Wt) {
   const size_t chunks = (size_t)N * K / 8;
   for (size_t c = (size_t)blockIdx.x * 256 + threadIdx.x; c < chunks; c += (size_t)gridDim.x * 256) {
-    const int g = c % 4, r = (c / 4) % 16, half = (c / 64) % 2;
+    const int r = c % 16, g = (c / 16) % 4, half = (c / 64) % 2;
     const size_t step = (c / 128) % (K / 64), tile = c / 128 / (K / 64);
     const int row = rows ? rows[tile * 16 + r] : (int)(tile * 16 + r);
     *reinterpret_cast<bf16x8*>(Wt + c * 8) = load8(W + (size_t)row * K + step * 64 + 16 * g + 8 * half);
@@ -130,7 +130,7 @@ gemm_skinny_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float
   const bf16* arow[MT];
 #pragma unroll
   for (int t = 0; t < NT; ++t)
-    wrow[t] = TILED ? W + (size_t)(n0 / 16 + t) * 16 * K + li * 32 + kg * 8
+    wrow[t] = TILED ? W + (size_t)(n0 / 16 + t) * 16 * K + kg * 128 + li * 8
                     : W + (size_t)min(n0 + t * 16 + li, N - 1) * K;
 #pragma unroll
   for (int u = 0; u < MT; ++u) arow[u] = A + (size_t)min(u * 16 + li, M - 1) * K;
@@ -325,7 +325,7 @@ gemm_qkv_rope_commit_kernel(const bf16* __restrict__ A, const bf16* __restrict__
     const int sub = np == 8 ? 0 : tt % 2;
     const int tile = head * (d / 16) + (np == 8 ? tt : tt / 2);
     const int r = rotated ? (li < np ? np * sub + li : 8 + np * sub + li - np) : 2 * np * sub + li;
-    wrow = W + (size_t)tile * 16 * K + (loads ? r : 0) * 32 + kg * 8;
+    wrow = W + (size_t)tile * 16 * K + kg * 128 + (loads ? r : 0) * 8;
   } else {
     wrow = W + ((size_t)head * d + (loads ? ch : 0)) * K;
   }
@@ -996,7 +996,7 @@ extern "C" int tl_gemm_bf16_norm(const void* A, const void* W, const void* Wt, v
   return launch_skinny<1, 1, 8>((const bf16*)A, (const bf16*)W, (float*)C, M, N, K, epilogue, st, ns, (const bf16*)Wt);
 }
 
-// Wt [N/16][K/64][2][16][4][8] = the tiled copy of W [N, K] (N % 16 == 0, K % 64 == 0) with its
+// Wt [N/16][K/64][2][4][16][8] = the tiled copy of W [N, K] (N % 16 == 0, K % 64 == 0) with its
 // rows taken in the order `rows` [N] (null: as they are).
 extern "C" int tl_tile_weights(const void* W, const int* rows, int N, int K, void* Wt, hipStream_t st) {
   TL_REQUIRE(N > 0 && K > 0 && tiles_fit(N, K), "tile_weights: N=%d must be a multiple of 16 and K=%d of 64", N, K);

@@ -280,16 +280,16 @@ def tiles_fit(N: int, K: int) -> bool:
 
 def tile_weights(w: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The copy of w [N, K] (bfloat16, N % 16 == 0, K % 64 == 0) that the products for at most
-    16 rows stream from: [N/16, K/64, 2, 16, 4, 8] with element (T, s, c, r, g, e) =
+    16 rows stream from: [N/16, K/64, 2, 4, 16, 8] with element (T, s, c, g, r, e) =
     w[rows[16 T + r], 64 s + 16 g + 8 c + e], so that what a wave loads at a time lies in one
-    run of memory.  `rows` (int32 [N], on the device): a permutation of the rows; None: none."""
+    run of memory, lane after lane.  `rows` (int32 [N], on the device): a permutation of the rows; None: none."""
     N, K = w.shape
     _req(w, "tile_weights.w", torch.bfloat16)
     if not tiles_fit(N, K):
         raise KernelError(f"tile_weights: N={N} must be a multiple of 16 and K={K} of 64")
     if rows is not None:
         _req(rows, "tile_weights.rows", torch.int32, (N,))
-    out = torch.empty((N // 16, K // 64, 2, 16, 4, 8), dtype=torch.bfloat16, device=w.device)
+    out = torch.empty((N // 16, K // 64, 2, 4, 16, 8), dtype=torch.bfloat16, device=w.device)
     _check(lib().tl_tile_weights(_p(w), _p(rows), N, K, _p(out), _stream()))
     return out
 
@@ -305,7 +305,7 @@ def qkv_tile_rows(nq: int, nkv: int, d: int, device) -> torch.Tensor:
 
 def _req_tiles(tiles: Optional[torch.Tensor], N: int, K: int) -> None:
     if tiles is not None:
-        _req(tiles, "gemm.tiles", torch.bfloat16, (N // 16, K // 64, 2, 16, 4, 8))
+        _req(tiles, "gemm.tiles", torch.bfloat16, (N // 16, K // 64, 2, 4, 16, 8))
         if not tiles_fit(N, K):
             raise KernelError(f"gemm.tiles: a weight [{N}, {K}] has no tiled copy")
 
