@@ -801,6 +801,59 @@ def test_qkv_rope_commit_from_the_tiled_copy(ops, nq, nkv, d, K, lens):
     assert not torch.equal(out[1][1], torch.nan_to_num(c["pages"].float(), nan=-7.0))
 
 
+# ---- many channels against at most 16 rows: whole rows of the weights, 1 KB a load --------------
+
+@pytest.mark.parametrize("M", [1, 5, 16])
+@pytest.mark.parametrize("N,K", [(64, 512), (192, 1536), (128, 2560), (320, 1024), (64, 3584)])
+def test_gemm_rows_kernel(ops, M, N, K):
+    variant = 2
+    a = rnd(M, K, seed=71, dtype=torch.bfloat16).to(DEV)
+    w = rnd(N, K, seed=72, dtype=torch.bfloat16, scale=0.3).to(DEV)
+    want = a.double().cpu() @ w.double().cpu().t()
+    out = torch.full((M, N), float("nan"), device=DEV)
+    ops.gemm_bf16(a, w, out, variant=variant)
+    assert rel_err(out, want) < 1e-5
+    x0 = rnd(M, N, seed=73).to(DEV)
+    acc = x0.clone()
+    ops.gemm_bf16(a, w, acc, accumulate=True, variant=variant)
+    assert rel_err(acc, x0.double().cpu() + want) < 1e-5
+    # a row's result does not depend on the rows beside it
+    alone = torch.empty(1, N, device=DEV)
+    ops.gemm_bf16(a[M - 1:].contiguous(), w, alone, variant=variant)
+    assert torch.equal(alone[0], out[M - 1])
+    h = torch.full((M, N // 2), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.gemm_bf16(a, w, h, silu_pair=True, variant=2)
+    full = want.view(M, N // 64, 2, 32)
+    assert rel_err(h, (plain.silu(full[:, :, 0]) * full[:, :, 1]).reshape(M, N // 2)) < KTOL["bfloat16"]
+    with pytest.raises(ops.KernelError, match="gemm_rows"):
+        ops.gemm_bf16(a[:, : K - 64].contiguous(), w[:, : K - 64].contiguous(), out, variant=variant)
+
+
+def test_wide_products_of_few_rows_take_the_rows_kernel(ops):
+    """The dispatcher sends gate|up (paired epilogue, with the norm's factor) and a head-sized product
+    to the kernel that reads whole rows, and gets what the other kernels get."""
+    M, K, N = 6, 1024, 16384 + 64
+    a = rnd(M, K, seed=74, dtype=torch.bfloat16).to(DEV)
+    w = rnd(N, K, seed=75, dtype=torch.bfloat16, scale=0.2).to(DEV)
+    want = a.double().cpu() @ w.double().cpu().t()
+    got, forced, other = (torch.empty(M, N, device=DEV) for _ in range(3))
+    ops.gemm_bf16(a, w, got)
+    ops.gemm_bf16(a, w, forced, variant=2)
+    ops.gemm_bf16(a, w, other, variant=411)
+    assert torch.equal(got, forced)
+    assert rel_err(got, want) < 1e-5 and rel_err(other, want) < 1e-5
+    ssq = (torch.rand(16, 5, generator=torch.Generator().manual_seed(76)) * K).to(DEV)
+    factor = ops.RowFactor(ssq, 5, K, 1e-5)
+    r = torch.rsqrt(ssq[:M].double().sum(1).cpu() / K + 1e-5)
+    h = torch.full((M, N // 2), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.gemm_bf16_norm(a, w, h, silu_pair=True, factor=factor)
+    full = (want * r[:, None]).view(M, N // 64, 2, 32)
+    assert rel_err(h, (plain.silu(full[:, :, 0]) * full[:, :, 1]).reshape(M, N // 2)) < KTOL["bfloat16"]
+    out = torch.empty(M, N, device=DEV)
+    ops.gemm_bf16_norm(a, w, out, factor=factor)
+    assert rel_err(out, want * r[:, None]) < 1e-5
+
+
 # ---- 17..128 rows: shared activations, K cut into partial sums (above 64 rows the k-step is 128) --
 
 @pytest.mark.parametrize("M", [17, 32, 33, 48, 50, 64, 5, 65, 80, 97, 112, 128])

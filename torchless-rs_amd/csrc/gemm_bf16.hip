@@ -10,6 +10,9 @@
 //    may carry the halves of an RMSNorm (NormSplit).  It can also read W from a
 //    copy laid out in tiles (see tile_weights_kernel): a wave's loads are then one
 //    run of consecutive bytes, which the memory serves faster than 16 rows apart.
+//  * gemm_rows: at most 16 rows against many channels (gate|up, the head) when K is a multiple
+//    of 512: W is read 1 KB of a row at a time, which the memory serves fastest, and turned
+//    into MFMA operands in LDS.
 //  * gemm_qkv_rope_commit: the skinny product for the fused q|k|v projection of
 //    single-token steps, with rotation and the write into the cache's pages.
 //  * gemm_mid: 17..128 rows.  The activations of a k-step are shared by the four
@@ -270,6 +273,126 @@ static int launch_skinny(const bf16* A, const bf16* W, float* C, int M, int N, i
   else
     gemm_skinny_kernel<NT, MT, SK_WAVES, false><<<grid, SK_WAVES * 64, 0, st>>>(A, W, C, M, N, K, epilogue, ns);
   TL_LAUNCH_CHECK("gemm_skinny");
+  return 0;
+}
+
+// ------------------------------------------------------- rows, 1 KB at a time ----
+// At most 16 rows of activations against many channels (gate|up, the head), from the weights as
+// stored.  The memory serves a load fastest when a wave's 64 lanes take 1 KB of one row, not
+// sixteen pieces of sixteen rows, so that is how W is read here: a workgroup owns 64 channels,
+// its 4 waves split K in chunks of 512; a wave reads 16 rows x 512 k with 16 loads, turns them in
+// its own 16 KB of LDS into MFMA operands (channel = lane % 16), and multiplies them with the
+// activations of that chunk, which it keeps in registers for the workgroup's 4 groups of 16
+// channels.  No barrier until the waves' sums meet; the epilogues are those of gemm_skinny
+// (store, accumulate, silu(gate) * up in groups of 64 rows, a factor per row).
+constexpr int ROWS_CHUNK = 512;                          // k a load instruction takes of one row
+constexpr int ROWS_LDS = 4 * 16 * ROWS_CHUNK * 2;        // bytes: a tile of 16 rows x 512 k for each wave
+constexpr int NRB = 4;                                   // groups of 16 channels a workgroup
+
+__global__ void __launch_bounds__(256, 2)
+gemm_rows_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float* __restrict__ C, int M, int N,
+                 int K, int epilogue, NormSplit ns) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char rows_smem[];
+  __shared__ float rs[16];
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64, li = lane % 16, kg = lane / 16;
+  const int n0 = blockIdx.x * (16 * NRB);
+  bf16* T = reinterpret_cast<bf16*>(rows_smem) + wave * (16 * ROWS_CHUNK);
+  const int chunks = K / ROWS_CHUNK;
+  const int c0 = wave * chunks / 4, c1 = (wave + 1) * chunks / 4;       // this wave's chunks of K
+  const bf16* alane = A + (size_t)min(li, M - 1) * K + kg * 8;          // + chunk * 512 + j * 32
+
+  f32x4 acc[NRB];
+#pragma unroll
+  for (int t = 0; t < NRB; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  bf16x8 wcur[16], areg[16];
+  auto load_w = [&](int c, int rb, bf16x8 (&w)[16]) {
+    // a uniform base and 32-bit offsets in bytes, worked out anew each time (kept across the loop,
+    // sixteen 64-bit addresses would take the registers that the loads in flight need)
+    const bf16* base = W + (size_t)(n0 + rb * 16) * K + (size_t)c * ROWS_CHUNK;
+    unsigned off = lane * 16, row_bytes = 2u * K;
+    asm volatile("" : "+v"(off), "+v"(row_bytes));
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+      w[i] = *reinterpret_cast<const bf16x8*>(reinterpret_cast<const char*>(base) + (off + i * row_bytes));
+  };
+  const bool scaled = ns.ssq_in != nullptr;
+  RowFactors rf;
+  if (c0 < c1) load_w(c0, 0, wcur);
+  if (scaled) rf.fetch(ns);
+  for (int c = c0; c < c1; ++c) {
+#pragma unroll
+    for (int j = 0; j < 16; ++j) areg[j] = load8(alane + (size_t)c * ROWS_CHUNK + j * 32);
+#pragma unroll
+    for (int rb = 0; rb < NRB; ++rb) {
+      // row i's chunk of 8 values q goes to place q ^ i of the row: the reads below, 16 rows at the
+      // same q, then fall on 16 different groups of banks
+#pragma unroll
+      for (int i = 0; i < 16; ++i) *reinterpret_cast<bf16x8*>(&T[i * ROWS_CHUNK + ((lane ^ i) * 8)]) = wcur[i];
+      __builtin_amdgcn_wave_barrier();
+      // the next 16 rows are asked for as soon as these have left their registers; a wave spends
+      // most of its time waiting for them, with other waves' loads under way meanwhile
+      if (rb < NRB - 1) load_w(c, rb + 1, wcur);
+      else if (c + 1 < c1) load_w(c + 1, 0, wcur);
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        const bf16x8 wf = *reinterpret_cast<const bf16x8*>(&T[li * ROWS_CHUNK + (((4 * j + kg) ^ li) * 8)]);
+        acc[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, areg[j], acc[rb], 0, 0, 0);
+      }
+      __builtin_amdgcn_wave_barrier();
+    }
+  }
+  if (scaled) rf.finish(ns, rs);
+  __syncthreads();                                     // every wave is done with its tile: the sums take its place
+  float* red = reinterpret_cast<float*>(rows_smem);   // [4 waves][NRB tiles][4][64]
+#pragma unroll
+  for (int t = 0; t < NRB; ++t)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) red[wave * (NRB * 256) + (t * 4 + r) * 64 + lane] = acc[t][r];   // D[n = 4 kg + r][m = li] of tile t
+  __syncthreads();
+  auto total = [&](int nl, int m) {
+    const int idx = ((nl / 16) * 4 + (nl % 4)) * 64 + ((nl % 16) / 4) * 16 + m;
+    float v = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) v += red[w * (NRB * 256) + idx];
+    return scaled ? v * rs[m] : v;
+  };
+  if (epilogue == EPI_SILU_PAIR) {                     // the 64 rows are 32 gate rows and their 32 up rows
+    bf16* H = reinterpret_cast<bf16*>(C);
+    const int NH = N / 2;
+    for (int e = threadIdx.x; e < 32 * 16; e += 256) {
+      const int j = e % 32, m = e / 32;
+      if (m < M) {
+        const float g = total(j, m), u = total(32 + j, m);
+        H[(size_t)m * NH + n0 / 2 + j] = (bf16)((g / (1.0f + expf(-g))) * u);
+      }
+    }
+    return;
+  }
+  for (int e = threadIdx.x; e < 16 * NRB * 16; e += 256) {
+    const int nl = e % (16 * NRB), m = e / (16 * NRB);
+    if (m < M) {
+      float* c = C + (size_t)m * N + n0 + nl;
+      *c = (epilogue == EPI_ACCUMULATE) ? *c + total(nl, m) : total(nl, m);
+    }
+  }
+}
+
+static bool rows_fit(int M, int N, int K) { return M <= 16 && N % 64 == 0 && K % ROWS_CHUNK == 0; }
+
+static int launch_rows(const bf16* A, const bf16* W, float* C, int M, int N, int K, int epilogue, hipStream_t st,
+                       NormSplit ns = NormSplit{}) {
+  static bool raised = false;
+  if (!raised) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_rows_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, ROWS_LDS);
+    if (e != hipSuccess) {
+      set_error("gemm_rows: cannot have %d bytes of LDS: %s", ROWS_LDS, hipGetErrorString(e));
+      return 2;
+    }
+    raised = true;
+  }
+  gemm_rows_kernel<<<N / (16 * NRB), 256, ROWS_LDS, st>>>(A, W, C, M, N, K, epilogue, ns);
+  TL_LAUNCH_CHECK("gemm_rows");
   return 0;
 }
 
@@ -830,6 +953,7 @@ extern "C" int tl_gemm_bf16(const void* A, const void* W, const void* Wt, void* 
   float* c = (float*)C;
   const bool wide = N >= 16384 || epilogue == EPI_SILU_PAIR;     // many rows: 64 a workgroup
   if (M <= 16) {
+    if (wide && rows_fit(M, N, K)) return launch_rows(a, w, c, M, N, K, epilogue, st);
     if (wide && (M > 4 || epilogue == EPI_SILU_PAIR)) return launch_skinny<4, 1, 4>(a, w, c, M, N, K, epilogue, st);
     return launch_skinny<1, 1, 8>(a, w, c, M, N, K, epilogue, st, NormSplit{}, (const bf16*)Wt);
   }
@@ -849,7 +973,7 @@ extern "C" int tl_gemm_bf16(const void* A, const void* W, const void* Wt, void* 
   return 0;
 }
 
-// For tests and tuning: force one kernel whatever M is.  variant 0: tiled; 1: big; else NT*100 + MT*10 + waves/4.
+// For tests and tuning: force one kernel whatever M is.  variant 0: tiled; 1: big; 2: rows; else NT*100 + MT*10 + waves/4.
 extern "C" int tl_gemm_bf16_variant(const void* A, const void* W, void* C, int M, int N, int K,
                                     int epilogue, int variant, hipStream_t st) {
   TL_REQUIRE(M > 0 && N > 0 && K > 0 && K % 8 == 0, "gemm_bf16: bad sizes M=%d N=%d K=%d", M, N, K);
@@ -865,6 +989,11 @@ extern "C" int tl_gemm_bf16_variant(const void* A, const void* W, void* C, int M
     return 0;
   }
   if (variant == 1) return launch_big(a, w, c, M, N, K, epilogue, st);
+  if (variant == 2) {
+    TL_REQUIRE(rows_fit(M, N, K), "gemm_rows: M=%d N=%d K=%d (at most 16 rows, N a multiple of 64, K of %d)", M, N,
+               K, ROWS_CHUNK);
+    return launch_rows(a, w, c, M, N, K, epilogue, st);
+  }
   const int mt = (variant / 10) % 10;
   TL_REQUIRE(M <= 16 * mt, "gemm_skinny: variant %d takes at most %d rows, not %d", variant, 16 * mt, M);
   TL_REQUIRE(epilogue != EPI_SILU_PAIR || variant / 100 == 4, "gemm_skinny: the paired epilogue needs 64 rows "
@@ -982,6 +1111,7 @@ extern "C" int tl_gemm_bf16_norm(const void* A, const void* W, const void* Wt, v
   TL_REQUIRE(!writer || (epilogue == EPI_ACCUMULATE && xt != nullptr && ssq_out != nullptr),
              "gemm_bf16_norm: the next norm's half goes with the accumulate epilogue, xt and ssq_out");
   const bool wide = N >= 16384 || epilogue == EPI_SILU_PAIR;
+  const bool rows = wide && !writer && rows_fit(M, N, K);        // many channels, K in chunks of 512: whole rows, 1 KB a load
   const bool four = wide && (M > 4 || epilogue == EPI_SILU_PAIR);
   const int groups = four ? (N + 63) / 64 : (N + 15) / 16;
   if (n_groups) *n_groups = groups;
@@ -991,6 +1121,7 @@ extern "C" int tl_gemm_bf16_norm(const void* A, const void* W, const void* Wt, v
   NormSplit ns{};
   ns.ssq_in = ssq_in; ns.n_part = n_part; ns.inv_h = inv_h; ns.eps = eps;
   ns.norm_w = norm_w; ns.xt = (bf16*)xt; ns.ssq_out = ssq_out;
+  if (rows) return launch_rows((const bf16*)A, (const bf16*)W, (float*)C, M, N, K, epilogue, st, ns);
   if (four) return launch_skinny<4, 1, 4>((const bf16*)A, (const bf16*)W, (float*)C, M, N, K, epilogue, st, ns);
   TL_REQUIRE((uintptr_t)Wt % 16 == 0, "gemm_bf16_norm: operands must be 16-byte aligned");
   return launch_skinny<1, 1, 8>((const bf16*)A, (const bf16*)W, (float*)C, M, N, K, epilogue, st, ns, (const bf16*)Wt);
