@@ -643,14 +643,16 @@ def test_random_configurations(tmp_path, seed):
         assert worst < TOL[dtype], (cfg, lens, tail, dtype, worst)
 
 
-def test_tiled_weight_copies_change_no_bit(tmp_path):
+@pytest.mark.parametrize("H,nq,nkv,d,I", [(128, 4, 2, 32, 192), (512, 8, 2, 64, 320)])
+def test_tiled_weight_copies_change_no_bit(tmp_path, H, nq, nkv, d, I):
     """Sizes at which q|k|v, o and down all have their tiled copies: single-token steps read
-    them, and give the bits they give from the weights as stored, and the plain logits."""
+    them, and give the bits they give from the weights as stored, and the plain logits.  (At
+    the second size gate|up of such steps is read in whole rows, 1 KB a load.)"""
     from torchless_rs_amd import write_random_model
     from torchless_rs_amd.engine import Engine, SeqInput, load_model
     cfg = {"architectures": ["MistralForCausalLM"], "model_type": "mistral", "num_hidden_layers": 2,
-           "hidden_size": 128, "num_attention_heads": 4, "num_key_value_heads": 2, "head_dim": 32,
-           "intermediate_size": 192, "vocab_size": 300, "rope_theta": 10000.0, "sliding_window": 40,
+           "hidden_size": H, "num_attention_heads": nq, "num_key_value_heads": nkv, "head_dim": d,
+           "intermediate_size": I, "vocab_size": 300, "rope_theta": 10000.0, "sliding_window": 40,
            "rms_norm_eps": 1e-5, "max_position_embeddings": 256, "tie_word_embeddings": False, "hidden_act": "silu"}
     mdir = write_random_model(str(tmp_path / "m"), cfg, seed=5, std=0.05, norm_std=0.1, dtype=torch.bfloat16)
     cfgd, w = read_model_dir(mdir)
