@@ -5,7 +5,9 @@ The reference has one cache per sequence and re-uses it by setting `pos = 0`
 taken from the front and given back at the end (src/model/batching.rs:190,
 227-234, 549-555).  Here ids are handed out from a free list, an id is never
 held twice, and giving back an id that is not held is an error.  The lists
-themselves live in the host library (csrc/host/books.cpp).
+themselves live in the host library (csrc/host/books.cpp); the pages' list
+there starts in a fixed shuffled order, so that a sequence's pages lie
+scattered over the pool.
 """
 from __future__ import annotations
 

@@ -32,15 +32,26 @@ int fail(int code, const char* fmt, ...) {
 }
 
 // Ids 0..n-1.  take() returns the id that was given back last (a freed id is used again at
-// once, so re-use is exercised), else the lowest id that was never taken.
+// once, so re-use is exercised), else the lowest id that was never taken; with `scattered`,
+// else the next of a fixed shuffle of the ids.  Pages are handed out scattered: a sequence's
+// pages one after the other in memory put the workgroups of a decode step, which start on pages
+// a power of two apart, on the same memory channels (attention over 8 x 4,096 keys: 32.1 against
+// 30.7 us in a pool that is just large enough, 31.2 against 27.5 in a pool of 3 GB).
 struct FreeList {
   int n;
   std::string what;
   std::vector<int> free_;
   std::vector<uint8_t> held;
-  FreeList(int n_, const char* what_) : n(n_), what(what_), held(n_, 0) {
+  FreeList(int n_, const char* what_, bool scattered = false) : n(n_), what(what_), held(n_, 0) {
     free_.reserve(n);
     for (int i = n - 1; i >= 0; --i) free_.push_back(i);
+    if (scattered) {                          // Fisher-Yates with a fixed generator: the same order in every run
+      uint64_t x = 0x9E3779B97F4A7C15ull;
+      for (int i = n - 1; i > 0; --i) {
+        x ^= x << 13; x ^= x >> 7; x ^= x << 17;
+        std::swap(free_[i], free_[(int)(x % (uint64_t)(i + 1))]);
+      }
+    }
   }
   int n_free() const { return (int)free_.size(); }
   bool holds(long i) const { return i >= 0 && i < n && held[i]; }
@@ -80,7 +91,7 @@ struct Group {
   int ring_pages;
   FreeList pool;
   std::vector<std::vector<int>> pages;      // by slot
-  Group(int ring, int n_pages, int max_slots) : ring_pages(ring), pool(n_pages, "page"), pages(max_slots) {}
+  Group(int ring, int n_pages, int max_slots) : ring_pages(ring), pool(n_pages, "page", true), pages(max_slots) {}
   int pages_needed(long length) const { return (int)std::min<long>((length + PAGE - 1) / PAGE, ring_pages); }
 };
 
