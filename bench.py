@@ -1,7 +1,8 @@
 """Decode and prefill throughput of the Mistral-7B-v0.1 shape on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 8192] [--layers L]
-                    [--shape 7b-v0.1|7b-v0.3|nemo-12b]
+                    [--shape 7b-v0.1|7b-v0.3|nemo-12b] [--only decode|prefill] [--prefill-tokens T]
+                    [--no-points] [--no-tiled-copies]
 
 One JSON line: decoded tokens a second of the default run (batch 8 at the
 context length of the configuration), the prefill of one 2,048-token prompt,
