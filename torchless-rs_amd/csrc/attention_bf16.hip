@@ -12,6 +12,8 @@
 // for that, and the prefill kernel transposes the step's own value rows on
 // their way into LDS.
 #include "common.hpp"
+#include "no_alloc.h"
+#include <mutex>
 
 namespace tl {
 
@@ -735,4 +737,56 @@ extern "C" int tl_attn_decode_bf16(const void* q, const void* pages, const int* 
   TL_BY_DPAD(launch_decode, (const bf16*)q, (const bf16*)pages, table, table_stride, ring_pages, row_pos,
              B, nq, nkv, d, window, scale, n_splits, part, (bf16*)out, st);
   return 1;
+}
+
+// ---- the entry point that allocates nothing (declared in no_alloc.h) --------
+// The partial results of the splits lie in this array instead of a buffer of the
+// caller's.  In host code its name is only a stand-in: the address that kernels
+// and copies take is looked up per device, once, and kept.
+static __device__ __align__(256) unsigned char scratch[TL_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int MAX_DEVICES = 64;
+std::mutex scratch_lock;
+float* scratch_of_device[MAX_DEVICES] = {};
+
+// The device address of `scratch` on the current device (0 and an error message if it cannot be had).
+float* static_scratch() {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
+    set_error("attn_decode_static: no current device (%s, device %d)", hipGetErrorString(e), dev);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> hold(scratch_lock);
+  if (scratch_of_device[dev] == nullptr) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr) {
+      set_error("attn_decode_static: the scratch array has no address on device %d: %s", dev,
+                hipGetErrorString(e));
+      return nullptr;
+    }
+    scratch_of_device[dev] = static_cast<float*>(ptr);
+  }
+  return scratch_of_device[dev];
+}
+}  // namespace
+
+extern "C" size_t tl_static_scratch_bytes(void) { return TL_STATIC_SCRATCH_BYTES; }
+
+extern "C" int tl_attn_decode_bf16_static(const void* q, const void* pages, const int* table, int table_stride,
+                                          int ring_pages, const int* row_pos, int B, int nq, int nkv, int d,
+                                          int window, float scale, int n_splits, void* out, hipStream_t st) {
+  TL_REQUIRE(B > 0 && nq > 0 && nkv > 0 && d > 0 && n_splits > 0,
+             "attn_decode_static: bad sizes B=%d nq=%d nkv=%d d=%d splits=%d", B, nq, nkv, d, n_splits);
+  const unsigned long long need = 4ull * (unsigned long long)B * (unsigned long long)nq *
+                                  (unsigned long long)n_splits * (unsigned long long)(d + 2);
+  TL_REQUIRE(n_splits == 1 || need <= TL_STATIC_SCRATCH_BYTES,
+             "attn_decode_static: the partial results of B=%d, %d heads, %d splits, head size %d take %llu "
+             "bytes, the static scratch holds %u", B, nq, n_splits, d, need, (unsigned)TL_STATIC_SCRATCH_BYTES);
+  float* part = static_scratch();
+  if (part == nullptr) return 2;
+  return tl_attn_decode_bf16(q, pages, table, table_stride, ring_pages, row_pos, B, nq, nkv, d, window, scale,
+                             n_splits, part, out, st);
 }
