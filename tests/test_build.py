@@ -1,0 +1,48 @@
+"""Which built library is loaded (no GPU, nothing compiled): only one that was made from the sources
+as they are, and from the temporary directory only out of a folder that is this user's alone."""
+import os
+
+import pytest
+
+from torchless_rs_amd.kernels import build
+
+
+def test_a_library_older_than_its_sources_is_built_again(tmp_path):
+    lib = str(tmp_path / "lib.so")
+    open(lib, "w").close()
+    calls = []
+
+    def rebuild():
+        calls.append(1)
+        return "fresh"
+
+    assert build._current_or_rebuilt(lib, "abc", rebuild, "lib") == "fresh"         # no stamp at all
+    build._write_stamp(lib, "abc")
+    assert build._current_or_rebuilt(lib, "abc", rebuild, "lib") == lib and len(calls) == 1
+    assert build._current_or_rebuilt(lib, "abd", rebuild, "lib") == "fresh" and len(calls) == 2
+    assert build._current_or_rebuilt(None, "abc", rebuild, "lib") == "fresh"
+
+    def cannot():
+        raise build.ExtensionMissing("hipcc not found")
+
+    with pytest.raises(build.ExtensionMissing, match="older than its sources"):
+        build._current_or_rebuilt(lib, "abd", cannot, "lib")
+
+
+def test_the_digest_follows_sources_and_flags(tmp_path):
+    f = tmp_path / "k.hip"
+    f.write_text("a")
+    d0 = build._digest([str(f)], ["-O3"])
+    assert d0 == build._digest([str(f)], ["-O3"]) and d0 != build._digest([str(f)], ["-O2"])
+    f.write_text("b")
+    assert d0 != build._digest([str(f)], ["-O3"])
+    assert build.kernels_digest() != build.host_digest()
+
+
+def test_a_shared_folder_under_tmp_is_not_trusted(tmp_path):
+    mine = tmp_path / "mine"
+    mine.mkdir(mode=0o700)
+    assert build._own_private_dir(str(mine))
+    os.chmod(mine, 0o777)
+    assert not build._own_private_dir(str(mine))
+    assert not build._own_private_dir(str(tmp_path / "absent"))

@@ -1,12 +1,38 @@
 """The cache's bookkeeping (no GPU): no slot or page lost, held twice or freed
 twice; windows hold a ring of pages; a step gets all its pages or none."""
+import ctypes
 import random
 
 import pytest
 import torch
 
-from torchless_rs_amd.cache import (PAGE, Cache, CacheFull, CacheMisuse, FreeList, KVRequest,
-                                    StateRequest, pages_for)
+from torchless_rs_amd.cache import PAGE, Cache, CacheFull, CacheMisuse, KVRequest, StateRequest, pages_for
+from torchless_rs_amd.cache import native
+
+
+class FreeList:
+    """The host library's free list (the one its books of slots and pages are made of), by itself."""
+
+    def __init__(self, n, what):
+        self.h = ctypes.c_void_p(native.lib().tl_freelist_new(n, what.encode()))
+
+    def __del__(self):
+        native.lib().tl_freelist_delete(self.h)
+
+    @property
+    def n_free(self):
+        return native.lib().tl_freelist_n_free(self.h)
+
+    def take(self):
+        out = ctypes.c_int(-1)
+        native.check(native.lib().tl_freelist_take(self.h, ctypes.byref(out)))
+        return out.value
+
+    def give_back(self, i):
+        native.check(native.lib().tl_freelist_give_back(self.h, int(i)))
+
+    def check(self):
+        native.check(native.lib().tl_freelist_check(self.h))
 
 
 def test_free_list():
@@ -131,3 +157,34 @@ def test_state_is_zeroed_when_a_slot_is_taken():
     c.state[0][s] += 5
     c.free_slot(s)
     assert c.alloc_slot() == s and float(c.state[0][s].abs().sum()) == 0
+
+
+def test_a_dropped_cache_is_freed_without_the_cycle_collector():
+    """Nothing in the cache points back at it: dropping the last reference frees its storage at
+    once, also when the collector is switched off or the objects are frozen out of its sight."""
+    import gc
+    import weakref
+    gc.collect()
+    gc.disable()
+    try:
+        c = Cache({0: KVRequest(2, 16, None)}, {0: StateRequest((4,))}, 64 * 4, torch.float32, "cpu",
+                  max_slots=2, allocate=True)
+        s = c.alloc_slot()
+        c.prepare([(s, 70)])
+        c.commit([(s, 70)])
+        storage, state, books = weakref.ref(c.groups[0].storage), weakref.ref(c.state[0]), weakref.ref(c._books)
+        del c
+        assert storage() is None and state() is None and books() is None
+    finally:
+        gc.enable()
+
+
+def test_a_closed_cache_gives_its_storage_back_and_refuses_use():
+    import weakref
+    c = Cache({0: KVRequest(2, 16, None)}, {}, 64 * 4, torch.float32, "cpu", allocate=True)
+    storage = weakref.ref(c.groups[0].storage)
+    c.close()
+    assert storage() is None
+    with pytest.raises(CacheMisuse, match="closed"):
+        c.alloc_slot()
+    c.close()                                               # twice is harmless

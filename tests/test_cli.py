@@ -38,6 +38,14 @@ def test_help_and_usage(capsys):
     assert main(["m", "one two"]) == 1
 
 
+def test_a_failed_run_is_an_error_line_and_exit_1(tmp_path, capsys):
+    """What `generate` raises (here: a folder that holds no model, or no GPU) comes out as the
+    other errors do, not as a traceback."""
+    assert main([str(tmp_path / "no_such_model"), "1 2 3"]) == 1
+    err = capsys.readouterr().err
+    assert err.startswith("Error: ") and "Traceback" not in err
+
+
 def test_ids_and_sampling_names():
     assert parse_ids("1, 5 17") == [1, 5, 17]
     assert SamplingConfig().temperature == 1.0                            # sampler/mod.rs:46-54

@@ -48,6 +48,7 @@ def test_round_trip_through_dict():
     ({"num_attention_heads": 5}, "head_dim"),                 # 64 / 5 and no head_dim
     ({"num_key_value_heads": 3}, "num_key_value_heads"),       # 4 % 3
     ({"head_dim": 15}, "even"),
+    ({"head_dim": 258}, "up to 256"),                           # beyond what the attention kernels take
     ({"hidden_act": "gelu"}, "hidden_act"),
     ({"rope_scaling": {"type": "linear", "factor": 2}}, "rope_scaling"),
     ({"quantization_config": {"quant_method": "gptq"}}, "quantized"),

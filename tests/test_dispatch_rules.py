@@ -28,5 +28,13 @@ def test_decode_splits_follow_batch_and_length():
             assert 1 <= S <= max(1, -(-pages // ops.SPLIT_PAGES))
 
 
-def test_row_thresholds():
-    assert ops.LIBRARY_ROWS == 64 and ops.MID_ROWS == 128 and ops.MID_ROWS > ops.LIBRARY_ROWS
+def test_rows_choose_the_kernel():
+    """Which product runs follows from the number of rows alone: the fused kernels up to 16, the one
+    that shares activations to MID_ROWS, cut into partial sums where few channels leave the chip idle."""
+    import torch
+    from torchless_rs_amd.parts.linear import Linear
+    lin = Linear(torch.zeros(4096, 4096, dtype=torch.bfloat16))
+    rows = lambda m: torch.zeros(m, 4096, dtype=torch.bfloat16)
+    assert [lin.mid(rows(m)) for m in (1, 16, 17, ops.MID_ROWS, ops.MID_ROWS + 1)] == [False, False, True, True, False]
+    assert not lin.mid(torch.zeros(32, 4096))                        # float32 rows: the plain kernel
+    assert ops.LIBRARY_ROWS < ops.MID_ROWS                           # between them only narrow outputs are ours

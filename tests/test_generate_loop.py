@@ -169,3 +169,35 @@ def test_running_ahead_steps():
     assert eng.steps == [[2, 1], [1, 1], [1, 1]]             # 3 tokens each: the last is never fed
     out = generate(AheadEngine(), DrawingSampler(), [[1]], max_tokens=5, run_ahead=False)
     assert out[0].tokens == [2, 3, 4, 5, 6]
+
+
+@pytest.mark.parametrize("fail_at", [0, 3])
+def test_an_exception_leaves_nothing_held(fail_at):
+    """`on_token` (or a step) that raises: the batch's slots are given back, and the engine serves
+    the next call as if nothing had happened."""
+    eng, smp = StrawEngine(), ArgmaxSampler()
+    seen = []
+
+    def on_token(i, t):
+        seen.append((i, t))
+        if len(seen) > fail_at:
+            raise RuntimeError("the caller's callback failed")
+
+    with pytest.raises(RuntimeError, match="callback failed"):
+        generate(eng, smp, [[1, 2], [10], [20]], max_tokens=5, on_token=on_token)
+    assert not eng.held and sorted(eng.free_slots) == [0, 1, 2, 3]
+    out = generate(eng, smp, [[1, 2], [10]], max_tokens=2)
+    assert [r.tokens for r in out] == [[3, 4], [11, 12]] and not eng.held
+
+
+def test_a_failing_step_leaves_nothing_held():
+    class Failing(StrawEngine):
+        def step(self, batch):
+            if len(self.steps) == 2:
+                raise ValueError("no room")
+            return super().step(batch)
+
+    eng = Failing()
+    with pytest.raises(ValueError, match="no room"):
+        generate(eng, ArgmaxSampler(), [[1], [5, 6]], max_tokens=6)
+    assert not eng.held

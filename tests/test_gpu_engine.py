@@ -296,21 +296,26 @@ def test_temperature_generation_follows_the_seeded_draws(zoo):
     eng, z = engine_for(zoo, "B", "float32"), zoo["B"]
     ps = z["prompts"]
     cfg = SamplingConfig(temperature=0.8, seed=4)
+
+    def follows_the_plain_draws(prompts, results):
+        for i, (p, r) in enumerate(zip(prompts, results)):
+            ids = list(p)
+            for step, t in enumerate(r.tokens):
+                lg = plain.forward(z["w"], z["cfg"], ids)[-1]
+                want = plain.sample(lg, philox_uniform(4, step, i), 0.8)
+                if t != want:                                       # the draw fell on a boundary
+                    cum = plain.sample_distribution(lg, 0.8).cumsum(0)
+                    assert abs(float(cum[min(t, want)]) - philox_uniform(4, step, i)) < 1e-5
+                ids.append(t)
+
     out = generate_until_eos(eng, ps, cfg, max_tokens=16)
-    again = generate_until_eos(eng, ps[::-1], cfg, max_tokens=16)[::-1]
-    for i, (p, r) in enumerate(zip(ps, out)):
-        ids = list(p)
-        for step, t in enumerate(r.tokens):
-            lg = plain.forward(z["w"], z["cfg"], ids)[-1]
-            want = plain.sample(lg, philox_uniform(4, step, i), 0.8)
-            if t != want:                                       # the draw fell on a boundary
-                cum = plain.sample_distribution(lg, 0.8).cumsum(0)
-                assert abs(float(cum[min(t, want)]) - philox_uniform(4, step, i)) < 1e-5
-            ids.append(t)
-    # a request's draws are keyed by its own index, so another order of the batch gives other tokens,
-    # but the same requests in the same order give the same tokens
+    follows_the_plain_draws(ps, out)
+    # a request's draws are keyed by its own index: the batch in another order draws with other
+    # numbers (and follows the plain implementation with those), the same order gives the same tokens
+    again = generate_until_eos(eng, ps[::-1], cfg, max_tokens=16)
+    follows_the_plain_draws(ps[::-1], again)
+    assert [r.tokens for r in again[::-1]] != [r.tokens for r in out]
     assert [r.tokens for r in generate_until_eos(eng, ps, cfg, max_tokens=16)] == [r.tokens for r in out]
-    assert len(again) == len(out)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -467,9 +472,22 @@ def test_trace_replay(zoo, dtype, tmp_path):
                 fed[i] += 1
             step += 1
     out = replay(z["dir"], dtype, lines, tmp_path, max_tokens=64 * 8)
-    assert sorted(int(f[:-4]) for f in os.listdir(out)) == sorted(expect)
+    assert sorted(int(f[:-4]) for f in os.listdir(out) if f.endswith(".f32")) == sorted(expect)
     for st, want in expect.items():
         assert rel_err(read_logits(out, st, V), want) < TOL[dtype], st
+    # the index says which row of a step's file is which request's position
+    with open(os.path.join(out, "index.json")) as f:
+        index = json.load(f)
+    assert index["vocab"] == V and sorted(int(k) for k in index["steps"]) == sorted(expect)
+    fed_before = {}
+    for l in lines:
+        rows = []
+        for e in l["entries"]:
+            rows += [(e["id"], fed_before.get(e["id"], 0) + w) for w in e["want"]]
+            fed_before[e["id"]] = fed_before.get(e["id"], 0) + len(e["tokens"])
+        if rows:
+            got = index["steps"][str(l["step"])]
+            assert [(r["id"], r["position"]) for r in got] == rows and [r["row"] for r in got] == list(range(len(rows)))
 
 
 def test_command_line(zoo):

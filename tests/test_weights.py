@@ -62,8 +62,37 @@ def test_malformed_files(tmp_path):
     _write_raw(p, {"t": {"dtype": "F32", "shape": [4], "data_offsets": [0, 8]}}, b"\0" * 8)
     with pytest.raises(SafetensorsError, match="need"):
         SafetensorsFile(p)
+    # a negative shape whose product would pass the count of bytes; offsets that are no integers
+    _write_raw(p, {"t": {"dtype": "U8", "shape": [-2, -3], "data_offsets": [0, 6]}}, b"\0" * 8)
+    with pytest.raises(SafetensorsError, match="negative dimension"):
+        SafetensorsFile(p)
+    _write_raw(p, {"t": {"dtype": "U8", "shape": [4], "data_offsets": [0.0, 4.0]}}, b"\0" * 8)
+    with pytest.raises(SafetensorsError, match="must be integers"):
+        SafetensorsFile(p)
+    _write_raw(p, {"t": {"dtype": "U8", "shape": [4], "data_offsets": [0, 4]},
+                   "u": {"dtype": "U8", "shape": [4], "data_offsets": [2, 6]}}, b"\0" * 8)
+    with pytest.raises(SafetensorsError, match="overlaps"):
+        SafetensorsFile(p)
     with pytest.raises(SafetensorsError, match="neither"):
         ModelFiles(str(tmp_path / "nothing"))
+
+
+def test_an_index_cannot_name_files_outside_the_folder(tmp_path):
+    inside, outside = tmp_path / "model", tmp_path / "elsewhere"
+    inside.mkdir()
+    outside.mkdir()
+    write_safetensors(str(outside / "x.safetensors"), {"a": torch.ones(2)})
+    for shard in ("../elsewhere/x.safetensors", str(outside / "x.safetensors"), "sub/x.safetensors", ".."):
+        (inside / "model.safetensors.index.json").write_text(json.dumps({"weight_map": {"a": shard}}))
+        with pytest.raises(SafetensorsError, match="plain file name"):
+            ModelFiles(str(inside))
+    os.symlink(str(outside / "x.safetensors"), str(inside / "link.safetensors"))
+    (inside / "model.safetensors.index.json").write_text(json.dumps({"weight_map": {"a": "link.safetensors"}}))
+    with pytest.raises(SafetensorsError, match="outside"):
+        ModelFiles(str(inside))
+    (inside / "model.safetensors.index.json").write_text(json.dumps({"weight_map": {"a": 3}}))
+    with pytest.raises(SafetensorsError, match="file names"):
+        ModelFiles(str(inside))
 
 
 def test_sharded_folder(tmp_path):

@@ -34,16 +34,31 @@ def generate_until_eos(engine: Engine, prompts: Sequence[Sequence[int]], config:
 def generate(model_dir: str, prompts: Sequence[Sequence[int]], max_tokens: int = 16,
              temperature: float = 0.7, top_k: Optional[int] = None, top_p: Optional[float] = None,
              seed: int = 0, stop_ids: Optional[Sequence[int]] = None, dtype: str = "bfloat16",
-             max_seq_len: Optional[int] = None, device: str = "cuda:0") -> List[GenerationResult]:
+             max_seq_len: Optional[int] = None, device: str = "cuda:0",
+             freeze_gc: bool = False) -> List[GenerationResult]:
     """Load the model folder and generate for every prompt.  `stop_ids` None
-    means config.json's eos_token_id, if it has one."""
+    means config.json's eos_token_id, if it has one.  The engine made for the call is closed
+    when it ends, its cache given back.  `freeze_gc`: see `Engine`."""
     model = load_model(model_dir, dtype, device)
     if stop_ids is None:
         stop_ids = list(getattr(model.config, "eos_token_ids", []) or [])
     longest = max(len(p) for p in prompts) + max_tokens
-    if max_seq_len is not None and longest > max_seq_len:
-        raise ValueError(f"a request needs {longest} positions, --max-seq-len allows {max_seq_len}")
+    # the longest sequence allowed: the model's max_position_embeddings unless the caller sets
+    # another limit, which may exceed it with a warning (src/main.rs:111-137 of the reference)
+    trained = getattr(model.config, "max_position_embeddings", None)
+    if max_seq_len is not None and trained and max_seq_len > trained:
+        import sys
+        sys.stderr.write(f"WARNING: --max-seq-len {max_seq_len} exceeds the model's trained context "
+                         f"length ({trained}).\n")
+    limit = max_seq_len if max_seq_len is not None else trained
+    if limit is not None and longest > limit:
+        raise ValueError(f"a request needs {longest} positions, " +
+                         (f"--max-seq-len allows {limit}" if max_seq_len is not None else
+                          f"the model's max_position_embeddings is {limit}; raise --max-seq-len to go beyond"))
     per_seq = -(-longest // 64) * 64
-    engine = Engine(model, max_tokens=per_seq * len(prompts), max_slots=len(prompts))
-    cfg = SamplingConfig(temperature=temperature, top_k=top_k, top_p=top_p, seed=seed)
-    return generate_until_eos(engine, prompts, cfg, max_tokens, stop_ids)
+    engine = Engine(model, max_tokens=per_seq * len(prompts), max_slots=len(prompts), freeze_gc=freeze_gc)
+    try:
+        cfg = SamplingConfig(temperature=temperature, top_k=top_k, top_p=top_p, seed=seed)
+        return generate_until_eos(engine, prompts, cfg, max_tokens, stop_ids)
+    finally:
+        engine.close()

@@ -63,101 +63,131 @@ def _ints(values) -> np.ndarray:
     return np.ascontiguousarray(np.asarray(values, dtype=np.int32))
 
 
+class _Books:
+    """Owner of the host library's books of one cache.  The views below hold this object and
+    never the cache itself, so that a dropped cache is freed at once, without the cycle collector."""
+
+    def __init__(self, max_slots: int, n_pages: int, rings, pages):
+        self.max_slots, self.n_pages = int(max_slots), int(n_pages)
+        rings, pages = _ints(rings), _ints(pages)
+        self.h = ctypes.c_void_p(native.lib().tl_books_new(self.max_slots, len(rings), rings.ctypes.data,
+                                                           pages.ctypes.data))
+
+    def close(self) -> None:
+        h, self.h = getattr(self, "h", None), None
+        if h:
+            native.lib().tl_books_delete(h)
+
+    __del__ = close
+
+    def held_slots(self) -> List[int]:
+        buf = np.empty(self.max_slots, dtype=np.int32)
+        n = native.lib().tl_books_held_slots(self.h, buf.ctypes.data, buf.size)
+        return buf[:n].tolist()
+
+    def holds(self, slot: int) -> bool:
+        return bool(native.lib().tl_books_holds(self.h, int(slot)))
+
+    @property
+    def free_slots(self) -> int:
+        return native.lib().tl_books_free_slots(self.h)
+
+
 class _Pool:
     """What is free and held of a group's pages (the books are the host library's)."""
 
-    def __init__(self, cache: "Cache", group: int, n: int):
-        self._c, self._g, self.n = cache, group, n
+    def __init__(self, books: _Books, group: int, n: int):
+        self._b, self._g, self.n = books, group, n
 
     @property
     def n_free(self) -> int:
-        return native.lib().tl_books_free_pages(self._c._h, self._g)
+        return native.lib().tl_books_free_pages(self._b.h, self._g)
 
     @property
     def n_held(self) -> int:
         return self.n - self.n_free
 
     def holds(self, page: int) -> bool:
-        return bool(native.lib().tl_books_page_held(self._c._h, self._g, int(page)))
+        return bool(native.lib().tl_books_page_held(self._b.h, self._g, int(page)))
 
 
 class _Slots:
-    def __init__(self, cache: "Cache", n: int):
-        self._c, self.n = cache, n
+    def __init__(self, books: _Books):
+        self._b, self.n = books, books.max_slots
 
     @property
     def n_free(self) -> int:
-        return native.lib().tl_books_free_slots(self._c._h)
+        return self._b.free_slots
 
     @property
     def n_held(self) -> int:
         return self.n - self.n_free
 
     def holds(self, slot: int) -> bool:
-        return bool(native.lib().tl_books_holds(self._c._h, int(slot)))
+        return self._b.holds(slot)
 
 
 class _PagesOfSlot:
     """group.pages_of_slot[slot] -> the slot's pages, in the order of the ring (a copy)."""
 
-    def __init__(self, cache: "Cache", group: int):
-        self._c, self._g = cache, group
+    def __init__(self, books: _Books, group: int):
+        self._b, self._g = books, group
 
     def __getitem__(self, slot: int) -> List[int]:
-        buf = np.empty(self._c.n_pages, dtype=np.int32)
-        n = native.lib().tl_books_pages(self._c._h, self._g, int(slot), buf.ctypes.data, buf.size)
+        buf = np.empty(self._b.n_pages, dtype=np.int32)
+        n = native.lib().tl_books_pages(self._b.h, self._g, int(slot), buf.ctypes.data, buf.size)
         if n < 0:
             raise KeyError(slot)
         return buf[:n].tolist()
 
     def __contains__(self, slot: int) -> bool:
-        return self._c.slots.holds(slot)
+        return self._b.holds(slot)
 
     def __iter__(self):
-        return iter(self._c.held_slots())
+        return iter(self._b.held_slots())
 
     def __len__(self) -> int:
-        return len(self._c.held_slots())
+        return len(self._b.held_slots())
 
 
 class _Lengths:
     """cache.length[slot] -> positions the slot holds; behaves as a read-only dict."""
 
-    def __init__(self, cache: "Cache"):
-        self._c = cache
+    def __init__(self, books: _Books):
+        self._b = books
 
     def __getitem__(self, slot: int) -> int:
-        n = native.lib().tl_books_length(self._c._h, int(slot))
+        n = native.lib().tl_books_length(self._b.h, int(slot))
         if n < 0:
             raise KeyError(slot)
         return n
 
     def __contains__(self, slot: int) -> bool:
-        return self._c.slots.holds(slot)
+        return self._b.holds(slot)
 
     def __iter__(self):
-        return iter(self._c.held_slots())
+        return iter(self._b.held_slots())
 
     def __len__(self) -> int:
-        return self._c.max_slots - self._c.slots.n_free
+        return self._b.max_slots - self._b.free_slots
 
     def values(self):
-        return [self[s] for s in self._c.held_slots()]
+        return [self[s] for s in self._b.held_slots()]
 
 
 class KVGroup:
     """Storage of the runs that share one `KVRequest`."""
 
-    def __init__(self, cache: "Cache", index: int, request: KVRequest, runs: List[int], n_pages: int, dtype,
-                 device, allocate: bool):
+    def __init__(self, index: int, request: KVRequest, runs: List[int], n_pages: int, dtype, device,
+                 allocate: bool):
         self.request = request
         self.runs = list(runs)
         self.layer_of_run = {r: i for i, r in enumerate(self.runs)}
         self.n_pages = n_pages
         # pages one sequence can hold: a ring for a window, else without bound (the pool is the limit)
         self.ring_pages = pages_for(request.window) if request.window else NO_RING
-        self.pool = _Pool(cache, index, n_pages)
-        self.pages_of_slot = _PagesOfSlot(cache, index)
+        self.index = index
+        self.pool = self.pages_of_slot = None        # views of the books, tied by the cache
         self.storage = None
         if allocate:
             # [layer, page, K|V, kv_head, row, head_dim]
@@ -186,15 +216,16 @@ class Cache:
         by_req: Dict[KVRequest, List[int]] = {}
         for run in sorted(kv_requests):
             by_req.setdefault(kv_requests[run], []).append(run)
-        self._h = None
         self.groups: List[KVGroup] = [
-            KVGroup(self, gi, req, runs, self.n_pages, dtype, device, allocate)
+            KVGroup(gi, req, runs, self.n_pages, dtype, device, allocate)
             for gi, (req, runs) in enumerate(by_req.items())]
-        rings, pages = _ints([g.ring_pages for g in self.groups]), _ints([g.n_pages for g in self.groups])
-        self._h = ctypes.c_void_p(native.lib().tl_books_new(self.max_slots, len(self.groups),
-                                                            rings.ctypes.data, pages.ctypes.data))
-        self.slots = _Slots(self, self.max_slots)
-        self.length = _Lengths(self)
+        self._books = _Books(self.max_slots, self.n_pages, [g.ring_pages for g in self.groups],
+                             [g.n_pages for g in self.groups])
+        for g in self.groups:
+            g.pool = _Pool(self._books, g.index, g.n_pages)
+            g.pages_of_slot = _PagesOfSlot(self._books, g.index)
+        self.slots = _Slots(self._books)
+        self.length = _Lengths(self._books)
         self.group_of_run: Dict[int, int] = {
             r: gi for gi, g in enumerate(self.groups) for r in g.runs}
         self.state: Dict[int, Optional[torch.Tensor]] = {}
@@ -203,10 +234,20 @@ class Cache:
             self.state[run] = torch.zeros((self.max_slots,) + tuple(req.shape), dtype=req.dtype,
                                           device=device) if allocate else None
 
-    def __del__(self):
-        h, self._h = getattr(self, "_h", None), None
-        if h:
-            native.lib().tl_books_delete(h)
+    @property
+    def _h(self):
+        """The handle of the books in the host library."""
+        if self._books.h is None:
+            raise CacheMisuse("the cache is closed")
+        return self._books.h
+
+    def close(self) -> None:
+        """Give the device storage and the books back now (the cache cannot be used afterwards).
+        Dropping the last reference does the same."""
+        for g in self.groups:
+            g.storage = None
+        self.state = {run: None for run in self.state}
+        self._books.close()
 
     # ---- slots -----------------------------------------------------------
     def alloc_slot(self) -> int:
@@ -222,9 +263,7 @@ class Cache:
         native.check(native.lib().tl_books_free_slot(self._h, int(slot)))
 
     def held_slots(self) -> List[int]:
-        buf = np.empty(self.max_slots, dtype=np.int32)
-        n = native.lib().tl_books_held_slots(self._h, buf.ctypes.data, buf.size)
-        return buf[:n].tolist()
+        return self._books.held_slots()
 
     # ---- growth ----------------------------------------------------------
     def prepare(self, growth: List[Tuple[int, int]]) -> None:

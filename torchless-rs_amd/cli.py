@@ -135,9 +135,18 @@ def main(argv: Optional[List[str]] = None, prog: str = "torchless") -> int:
     t0 = time.time()
     if opts["--debug"]:
         sys.stderr.write(f"Loading {model_path} ({opts['--dtype']})\n")
-    results = generate(model_path, prompts, max_tokens=max_tokens, temperature=opts["--temperature"],
-                       top_k=opts["--top-k"], top_p=opts["--top-p"], seed=opts["--seed"],
-                       stop_ids=stop_ids, dtype=opts["--dtype"], max_seq_len=opts["--max-seq-len"])
+    try:
+        results = generate(model_path, prompts, max_tokens=max_tokens, temperature=opts["--temperature"],
+                           top_k=opts["--top-k"], top_p=opts["--top-p"], seed=opts["--seed"],
+                           stop_ids=stop_ids, dtype=opts["--dtype"], max_seq_len=opts["--max-seq-len"],
+                           freeze_gc=True)
+    except (ValueError, OSError, RuntimeError, KeyError) as e:
+        # a request beyond --max-seq-len or the cache, a token id outside the vocabulary, a folder
+        # that is not a model, weights that do not fit the configuration, no GPU
+        if opts["--debug"]:
+            raise
+        sys.stderr.write(f"Error: {e}\n")
+        return 1
     dt = time.time() - t0
     for r in results:
         print(" ".join(str(t) for t in r.tokens))

@@ -17,6 +17,8 @@ from typing import Any, Dict, List, Optional
 from .base import ConfigError, ModelConfig, take_bool, take_float, take_int
 
 # keys that are read; anything else in the file is carried in `extra`
+MAX_HEAD_DIM = 256          # the largest head the attention kernels take
+
 _KNOWN = {
     "architectures", "model_type", "hidden_size", "intermediate_size", "num_hidden_layers",
     "num_attention_heads", "num_key_value_heads", "head_dim", "vocab_size",
@@ -63,6 +65,8 @@ class MistralConfig(ModelConfig):
             hd = H // nq
         if hd % 2:
             raise ConfigError(f"config.json: head_dim {hd} must be even for the rotation in pairs")
+        if hd > MAX_HEAD_DIM:
+            raise ConfigError(f"config.json: head_dim {hd} is not served (even sizes up to {MAX_HEAD_DIM})")
         if nq % nkv:
             raise ConfigError(
                 f"config.json: num_attention_heads {nq} is not a multiple of "

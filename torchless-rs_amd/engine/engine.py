@@ -197,7 +197,11 @@ class Engine:
     that live sequences hold at any time, each rounded up to whole pages."""
 
     def __init__(self, model: Model, max_tokens: int, max_slots: Optional[int] = None,
-                 use_graphs: bool = True):
+                 use_graphs: bool = True, freeze_gc: bool = False):
+        """`freeze_gc`: take every object alive now (the model's among them) out of the
+        garbage collector's sight (`gc.freeze()`), so that its passes, a millisecond each every
+        few steps, do not stall decoding.  It acts on the whole process, the caller's objects
+        included: for programs that serve one model until they end (the command line, the bench)."""
         self.model = model
         self.device = model.device
         self.cache: Cache = model.make_cache(max_tokens, max_slots)
@@ -207,10 +211,17 @@ class Engine:
         self.use_graphs = use_graphs
         self.max_graphs = 32
         self._graphs: Dict[tuple, _Graph] = {}
-        # The model's objects live as long as the process: take them out of the collector's
-        # sight, or its passes over them (a millisecond each, every few steps) stall the steps.
-        gc.collect()
-        gc.freeze()
+        if freeze_gc:
+            gc.collect()
+            gc.freeze()
+
+    def close(self) -> None:
+        """Give back the cache's storage, the captured graphs and the workspace now.  The engine
+        cannot step afterwards; the model stays loaded."""
+        self._graphs.clear()
+        self.workspace.clear()
+        self.runs = []
+        self.cache.close()
 
     # ---- slots -----------------------------------------------------------
     def alloc(self) -> int:

@@ -17,7 +17,7 @@ tested without a GPU.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Callable, List, Optional, Sequence
+from typing import Callable, Dict, List, Optional, Sequence
 
 from .engine import SeqInput
 
@@ -96,40 +96,53 @@ def generate(engine, sampler, prompts: Sequence[Sequence[int]], max_tokens: int,
         return bool(r.finish_reason)
 
     for batch in plan_batches(need, engine.fits, max_batch):
-        slots = {i: engine.alloc() for i in batch}
-        live = list(batch)
-        logits = engine.step([SeqInput(slots[i], list(prompts[i]), [len(prompts[i]) - 1]) for i in live])
-        if not run_ahead:
-            while True:
-                ids = sampler.sample(logits, live, [len(results[i].tokens) for i in live])
-                nxt, feed = [], {}
-                for i, t in zip(live, ids):
-                    if accept(i, t):
-                        engine.free(slots.pop(i))
-                    else:
-                        feed[i] = [t]
-                        nxt.append(i)
-                live = nxt
-                if not live:
-                    break
-                logits = engine.step([SeqInput(slots[i], feed[i], [0]) for i in live])
-            continue
-        # run ahead: `order` are the requests whose tokens `drawn` holds (row by row); those of
-        # them that are not known to be finished go into the next step at once
-        order = live
-        drawn = sampler.draw(logits, order, [len(results[i].tokens) for i in order])
-        while order:
-            # a request that is alive and whose budget this token does not use up goes on, unless
-            # the token is a stop id, which the host does not know yet
-            ahead = [i for i in order if i in slots and len(results[i].tokens) + 1 < max_tokens]
-            nxt_drawn = None
-            if ahead:
-                rows = [order.index(i) for i in ahead]
-                logits = engine.step([SeqInput(slots[i], [0], [0]) for i in ahead],
-                                     device_tokens=drawn.device, token_rows=rows)
-                nxt_drawn = sampler.draw(logits, ahead, [len(results[i].tokens) + 1 for i in ahead])
-            for i, t in zip(order, drawn.tokens()):
-                if i in slots and accept(i, t):           # (a request dropped earlier: its row ran for nothing)
-                    engine.free(slots.pop(i))
-            order, drawn = ahead, nxt_drawn
+        slots: Dict[int, int] = {}
+        try:
+            _serve_batch(engine, sampler, prompts, batch, slots, results, accept, max_tokens, run_ahead)
+        finally:
+            # whatever ended the batch (a step that failed, the caller's `on_token`, an interrupt),
+            # nothing of it stays held in the engine
+            for i in list(slots):
+                engine.free(slots.pop(i))
     return results
+
+
+def _serve_batch(engine, sampler, prompts, batch, slots, results, accept, max_tokens, run_ahead) -> None:
+    """One batch from its prompts to its last token.  `slots` (request -> slot) is the caller's: what
+    is still in it when this returns or raises is freed there."""
+    for i in batch:
+        slots[i] = engine.alloc()
+    live = list(batch)
+    logits = engine.step([SeqInput(slots[i], list(prompts[i]), [len(prompts[i]) - 1]) for i in live])
+    if not run_ahead:
+        while True:
+            ids = sampler.sample(logits, live, [len(results[i].tokens) for i in live])
+            nxt, feed = [], {}
+            for i, t in zip(live, ids):
+                if accept(i, t):
+                    engine.free(slots.pop(i))
+                else:
+                    feed[i] = [t]
+                    nxt.append(i)
+            live = nxt
+            if not live:
+                return
+            logits = engine.step([SeqInput(slots[i], feed[i], [0]) for i in live])
+    # run ahead: `order` are the requests whose tokens `drawn` holds (row by row); those of
+    # them that are not known to be finished go into the next step at once
+    order = live
+    drawn = sampler.draw(logits, order, [len(results[i].tokens) for i in order])
+    while order:
+        # a request that is alive and whose budget this token does not use up goes on, unless
+        # the token is a stop id, which the host does not know yet
+        ahead = [i for i in order if i in slots and len(results[i].tokens) + 1 < max_tokens]
+        nxt_drawn = None
+        if ahead:
+            rows = [order.index(i) for i in ahead]
+            logits = engine.step([SeqInput(slots[i], [0], [0]) for i in ahead],
+                                 device_tokens=drawn.device, token_rows=rows)
+            nxt_drawn = sampler.draw(logits, ahead, [len(results[i].tokens) + 1 for i in ahead])
+        for i, t in zip(order, drawn.tokens()):
+            if i in slots and accept(i, t):           # (a request dropped earlier: its row ran for nothing)
+                engine.free(slots.pop(i))
+        order, drawn = ahead, nxt_drawn

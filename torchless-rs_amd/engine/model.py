@@ -46,12 +46,9 @@ class Model:
         """`source`: anything with names/shape/dtype/tensor (a model folder's
         files, or tensors in memory).  `tiled_copies`: may the parts keep second
         copies of weights in the layout that single-token steps stream fastest?"""
-        from ..parts.linear import Linear
-        before, Linear.tiled_copies = Linear.tiled_copies, bool(tiled_copies)
-        try:
+        from ..parts.linear import loading_with
+        with loading_with(tiled_copies):
             self._load_parts(source)
-        finally:
-            Linear.tiled_copies = before
 
     def _load_parts(self, source) -> None:
         spec = self.spec

@@ -12,7 +12,11 @@ A request is given a slot when its id is first seen and gives it back when
 the id appears in `end`.  For a step in which logits are wanted,
 `<out>/<step>.f32` receives them as little-endian float32 [wanted, vocab], in
 the order of the entries and of their `want` lists.  After every step the
-line `done <step>` is printed and flushed.
+line `done <step>` is printed and flushed.  When the input ends (or the run
+fails) `<out>/index.json` lists, for every step that wrote logits, which row
+of its file belongs to which request and position:
+
+    {"vocab": V, "steps": {"0": [{"id": "a", "position": 0, "row": 0}, ...]}}
 """
 from __future__ import annotations
 
@@ -35,8 +39,7 @@ def main(argv=None) -> int:
     args = ap.parse_args(argv)
 
     print("[trace_run] loading torch and the kernels", file=sys.stderr, flush=True)
-    import torch
-    from .engine import Engine, SeqInput, load_model
+    from .engine import Engine, load_model
 
     os.makedirs(args.out, exist_ok=True)
     model = load_model(args.model, args.dtype, "cuda:0")
@@ -44,24 +47,40 @@ def main(argv=None) -> int:
     print("[trace_run] ready", file=sys.stderr, flush=True)
 
     slot_of: Dict[str, int] = {}
+    index: Dict[str, list] = {}
+    try:
+        _replay(engine, args.out, slot_of, index)
+    finally:
+        with open(os.path.join(args.out, "index.json"), "w") as f:
+            json.dump({"vocab": engine.vocab_size, "steps": index}, f)
+    return 0
+
+
+def _replay(engine, out_dir: str, slot_of: Dict[str, int], index: Dict[str, list]) -> None:
+    import torch
+    from .engine import SeqInput
     for line in sys.stdin:
         line = line.strip()
         if not line:
             continue
         rec = json.loads(line)
         step = rec["step"]
-        batch = []
+        batch, rows = [], []
         for e in rec.get("entries", []):
             rid = str(e["id"])
             if rid not in slot_of:
                 slot_of[rid] = engine.alloc()
             batch.append(SeqInput(slot_of[rid], e["tokens"], e.get("want", [])))
+            held = engine.length(slot_of[rid])
+            rows += [{"id": rid, "position": held + int(w), "row": len(rows) + k}
+                     for k, w in enumerate(e.get("want", []))]
         if batch:
             logits = engine.step(batch)
             if logits.shape[0]:
                 arr = logits.detach().to("cpu").numpy().astype("<f4", copy=False)
-                with open(os.path.join(args.out, f"{step}.f32"), "wb") as f:
+                with open(os.path.join(out_dir, f"{step}.f32"), "wb") as f:
                     f.write(np.ascontiguousarray(arr).tobytes())
+                index[str(step)] = rows
             else:
                 torch.cuda.synchronize()
         for rid in rec.get("end", []):
@@ -69,7 +88,6 @@ def main(argv=None) -> int:
             if rid in slot_of:
                 engine.free(slot_of.pop(rid))
         print(f"done {step}", flush=True)
-    return 0
 
 
 if __name__ == "__main__":

@@ -3,13 +3,16 @@ kernels for gfx950 (`libtorchless_hip.so`, hipcc) and the host side of cache
 and step (`libtorchless_host.so`, plain C++, no GPU needed).
 
 `build()` always compiles both.  `load()` and `load_host()` load the library
-that is there and build only if none is.  The libraries go to `csrc/_build/`
-inside the package; if that cannot be written (a read-only checkout), to a
-folder of the user's own under the system's temporary directory.
+that is there if it was built from the sources as they are now (a digest of
+sources and flags is kept beside each library), and build otherwise.  The
+libraries go to `csrc/_build/` inside the package; if that cannot be written
+(a read-only checkout), to a folder of the user's own (mode 0700) under the
+system's temporary directory.
 """
 from __future__ import annotations
 
 import ctypes
+import hashlib
 import os
 import shutil
 import subprocess
@@ -27,6 +30,8 @@ _CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HIPCC_FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
                "-Wno-unused-result"]
+
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-Wall"]
 
 _lib: Optional[ctypes.CDLL] = None
 _host_lib: Optional[ctypes.CDLL] = None
@@ -50,6 +55,41 @@ def host_sources() -> List[str]:
     return sorted(os.path.join(d, f) for f in os.listdir(d) if f.endswith(".cpp"))
 
 
+def _headers() -> List[str]:
+    return sorted(os.path.join(_CSRC, f) for f in os.listdir(_CSRC) if f.endswith((".hpp", ".h")))
+
+
+def _digest(files: List[str], flags: List[str]) -> str:
+    """What a library depends on: the text of its sources and the compiler's flags."""
+    h = hashlib.sha256(" ".join(flags).encode())
+    for f in files:
+        h.update(os.path.basename(f).encode() + b"\0")
+        with open(f, "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()
+
+
+def kernels_digest() -> str:
+    return _digest(sources() + _headers(), HIPCC_FLAGS)
+
+
+def host_digest() -> str:
+    return _digest(host_sources(), HOST_FLAGS)
+
+
+def _write_stamp(lib: str, digest: str) -> None:
+    with open(lib + ".stamp", "w") as f:
+        f.write(digest + "\n")
+
+
+def _is_current(lib: str, digest: str) -> bool:
+    try:
+        with open(lib + ".stamp") as f:
+            return f.read().strip() == digest
+    except OSError:
+        return False
+
+
 def find_cxx() -> str:
     for c in (os.environ.get("CXX"), shutil.which("g++"), shutil.which("c++"), shutil.which("clang++"),
               "/opt/rocm/llvm/bin/clang++"):
@@ -67,17 +107,29 @@ def build_host(verbose: bool = True) -> str:
     lib = os.path.join(out_dir, HOST_LIB_NAME)
     tmp = lib + f".tmp{os.getpid()}"
     t0 = time.time()
-    _run_with_progress([cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", *host_sources(), "-o", tmp],
-                       "the host library")
+    digest = host_digest()
+    _run_with_progress([cxx, *HOST_FLAGS, *host_sources(), "-o", tmp], "the host library")
     os.replace(tmp, lib)
+    _write_stamp(lib, digest)
     if verbose:
         _say(f"built {lib} in {time.time() - t0:.0f} s")
     return lib
 
 
+def _own_private_dir(path: str) -> bool:
+    """Is `path` a folder of this user's that nobody else can write to?"""
+    try:
+        st = os.stat(path)
+    except OSError:
+        return False
+    return (not hasattr(os, "getuid") or st.st_uid == os.getuid()) and not (st.st_mode & 0o022)
+
+
 def _writable_dir(path: str) -> bool:
     try:
-        os.makedirs(path, exist_ok=True)
+        os.makedirs(path, mode=0o700, exist_ok=True)
+        if path.startswith(tempfile.gettempdir() + os.sep) and not _own_private_dir(path):
+            return False                     # a folder under /tmp that someone else made, or may write to
         probe = os.path.join(path, f".probe{os.getpid()}")
         with open(probe, "w"):
             pass
@@ -130,6 +182,7 @@ def build(verbose: bool = True) -> str:
     if out_dir is None:
         raise ExtensionMissing(f"no writable build folder among {build_dirs()}")
     srcs = sources()
+    digest = kernels_digest()
     if verbose:
         _say(f"compiling {len(srcs)} HIP sources for {ARCH} into {out_dir}")
     objs = [os.path.join(out_dir, os.path.basename(s)[:-4] + ".o") for s in srcs]
@@ -147,27 +200,36 @@ def build(verbose: bool = True) -> str:
     tmp = lib + f".tmp{os.getpid()}"
     _run_with_progress([hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", *objs, "-o", tmp], "link")
     os.replace(tmp, lib)
+    _write_stamp(lib, digest)
     if verbose:
         _say(f"built {lib} in {time.time() - t0:.0f} s")
     return lib
 
 
 def built_library(name: str = LIB_NAME) -> Optional[str]:
-    for d in build_dirs():
+    """The library `name` if one is there: in the package's own folder, or in this user's
+    private folder under the temporary directory (never in one that others can write to)."""
+    pkg, tmp = build_dirs()
+    for d in (pkg, tmp):
         p = os.path.join(d, name)
-        if os.path.isfile(p):
+        if os.path.isfile(p) and (d == pkg or _own_private_dir(d)):
             return p
     return None
 
 
-def _warn_if_stale(lib: str, srcs: Optional[List[str]] = None) -> None:
+def _current_or_rebuilt(path: Optional[str], digest: str, rebuild, what: str) -> str:
+    """`path` if it was built from the sources as they are; else a fresh build.  A library that is
+    older than its sources is never loaded: a run would then test other kernels than it shows."""
+    if path is not None and _is_current(path, digest):
+        return path
+    if path is not None:
+        _say(f"{what} at {path} was not built from the present sources; building again")
     try:
-        srcs = srcs or [os.path.join(_CSRC, f) for f in os.listdir(_CSRC) if f.endswith((".hip", ".hpp"))]
-        newest = max(os.path.getmtime(f) for f in srcs)
-        if newest > os.path.getmtime(lib) + 1.0:
-            _say(f"warning: a source is newer than {lib}; build again to pick it up")
-    except OSError:
-        pass
+        return rebuild()
+    except ExtensionMissing as e:
+        if path is None:
+            raise
+        raise ExtensionMissing(f"{path} is older than its sources and cannot be built again: {e}") from None
 
 
 def load() -> ctypes.CDLL:
@@ -176,11 +238,7 @@ def load() -> ctypes.CDLL:
     with _lock:
         if _lib is not None:
             return _lib
-        path = built_library()
-        if path is None:
-            path = build()
-        else:
-            _warn_if_stale(path)
+        path = _current_or_rebuilt(built_library(), kernels_digest(), build, "the kernels' library")
         try:
             _lib = ctypes.CDLL(path)
         except OSError as e:
@@ -194,11 +252,7 @@ def load_host() -> ctypes.CDLL:
     with _lock:
         if _host_lib is not None:
             return _host_lib
-        path = built_library(HOST_LIB_NAME)
-        if path is None:
-            path = build_host()
-        else:
-            _warn_if_stale(path, host_sources())
+        path = _current_or_rebuilt(built_library(HOST_LIB_NAME), host_digest(), build_host, "the host library")
         try:
             _host_lib = ctypes.CDLL(path)
         except OSError as e:

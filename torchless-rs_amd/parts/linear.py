@@ -6,25 +6,40 @@ from __future__ import annotations
 
 import torch
 
+import contextlib
+import contextvars
+
 from ..kernels import ops
+
+# whether weights loaded now may keep tiled copies: set for the extent of one load
+# (`loading_with`), per thread and task, never for the process
+_tiled_copies = contextvars.ContextVar("tiled_copies", default=True)
+
+
+@contextlib.contextmanager
+def loading_with(tiled_copies: bool):
+    """Within this block `Linear(..., tiled=True)` keeps its tiled copy only if `tiled_copies`."""
+    token = _tiled_copies.set(bool(tiled_copies))
+    try:
+        yield
+    finally:
+        _tiled_copies.reset(token)
 
 
 class Linear:
     """A weight [N, K] resident on the device in its stored width.  With `tiled` it
     also keeps the tiled copy (`ops.tile_weights`) that the products of steps of at
     most 16 rows read instead: memory spent for the rate at which decoding streams
-    the weights (`Linear.tiled_copies` switches all of them off).  `tile_rows`: the
+    the weights (a load under `loading_with(False)` makes none).  `tile_rows`: the
     copy's own order of rows, for a kernel that wants one; then only that kernel
     reads it (`own_tiles`)."""
-
-    tiled_copies = True
 
     def __init__(self, weight: torch.Tensor, tiled: bool = False, tile_rows: torch.Tensor = None):
         assert weight.dim() == 2
         self.weight = weight.contiguous()
         self.out_features, self.in_features = self.weight.shape
         self.tiles = self.own_tiles = None
-        if (tiled and Linear.tiled_copies and self.weight.is_cuda and self.weight.dtype == torch.bfloat16
+        if (tiled and _tiled_copies.get() and self.weight.is_cuda and self.weight.dtype == torch.bfloat16
                 and ops.tiles_fit(self.out_features, self.in_features)):
             copy = ops.tile_weights(self.weight, tile_rows)
             if tile_rows is None:

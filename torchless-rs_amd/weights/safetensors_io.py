@@ -59,9 +59,14 @@ class SafetensorsFile:
         self._info: Dict[str, Tuple[str, Tuple[int, ...], int, int]] = {}
         for name, e in header.items():
             try:
-                dt, shape, (b, en) = e["dtype"], tuple(int(s) for s in e["shape"]), e["data_offsets"]
+                dt, dims, (b, en) = e["dtype"], list(e["shape"]), e["data_offsets"]
             except (KeyError, TypeError, ValueError):
                 raise SafetensorsError(f"{path}: malformed entry for tensor {name!r}") from None
+            if any(type(v) is not int for v in dims + [b, en]):
+                raise SafetensorsError(f"{path}: tensor {name!r}: shape and data_offsets must be integers")
+            if any(v < 0 for v in dims):
+                raise SafetensorsError(f"{path}: tensor {name!r} has a negative dimension in {dims}")
+            shape = tuple(dims)
             if dt not in _DTYPES:
                 raise SafetensorsError(f"{path}: tensor {name!r} has unknown dtype {dt!r}")
             n = 1
@@ -75,6 +80,11 @@ class SafetensorsFile:
                     f"{path}: tensor {name!r} holds {en - b} bytes, its shape {list(shape)} and "
                     f"dtype {dt} need {n * _DTYPES[dt][1]}")
             self._info[name] = (dt, shape, int(b), int(en))
+        end = 0
+        for name, (_, _, b, en) in sorted(self._info.items(), key=lambda kv: kv[1][2:]):
+            if b < end and en > b:
+                raise SafetensorsError(f"{path}: the data of tensor {name!r} overlaps another tensor's")
+            end = max(end, en)
         self._mm: Optional[mmap.mmap] = None
 
     def names(self) -> List[str]:
@@ -125,8 +135,15 @@ class ModelFiles:
                     wm = json.load(fh)["weight_map"]
                 except (json.JSONDecodeError, KeyError, TypeError):
                     raise SafetensorsError(f"{index}: no 'weight_map'") from None
+            if not isinstance(wm, dict) or not all(isinstance(v, str) for v in wm.values()):
+                raise SafetensorsError(f"{index}: 'weight_map' must map tensor names to file names")
             for shard in sorted(set(wm.values())):
+                # a shard is a file of this folder: no path, no way out of it
+                if os.path.basename(shard) != shard or shard in ("", ".", ".."):
+                    raise SafetensorsError(f"{index}: shard name {shard!r} is not a plain file name")
                 p = os.path.join(model_dir, shard)
+                if os.path.dirname(os.path.realpath(p)) != os.path.realpath(model_dir):
+                    raise SafetensorsError(f"{index}: shard {shard!r} lies outside {model_dir}")
                 f = SafetensorsFile(p)
                 self._files[p] = f
                 for n in f.names():
