@@ -240,3 +240,76 @@ def generate_greedy(weights, cfg, prompt, max_tokens, stop_ids=(), dtype=torch.f
         out.append(t)
         ids.append(t)
     return out, "length"
+
+
+# --- the same model with the engine's bfloat16 roundings ------------------------
+
+def to_bf16(t: torch.Tensor) -> torch.Tensor:
+    """Round as a float32 value is rounded when it is stored in bfloat16 (nearest even)."""
+    return t.to(torch.float32).to(torch.bfloat16).to(t.dtype)
+
+
+def forward_rounded(weights: dict, cfg: dict, ids, step_rows, library_rows=64) -> torch.Tensor:
+    """`forward` in float64 with a rounding to bfloat16 at every place where the engine's
+    bfloat16 path stores one, and nowhere else: the output of a norm, q and k after the rotation,
+    v, the probabilities as they enter the product with the values (their sum is taken
+    unrounded), the attention's output, silu(gate) * up.  The residual stream, all sums and the
+    softmax are not rounded (the engine keeps them in float32).
+
+    Two roundings depend on how many rows the step had that a row came in (`step_rows[t]`):
+    * up to 16 rows, a norm that follows a product is cut in two around the products next to
+      it: bfloat16(x * w) goes into the product and the results are multiplied by
+      rsqrt(mean(x^2) + eps) (all but the first layer's first norm and the last norm);
+    * above `library_rows` rows, gate and up are themselves stored in bfloat16 before the
+      activation (None: never).
+    (The kernels round a probability against the running maximum of the keys seen so far and
+    scale float32 sums afterwards; here it is rounded against the row's maximum: another
+    realisation of the same rounding.)
+    The formulas are those of the functions above; only the roundings are added."""
+    f64 = torch.float64
+    w = {k: v.to(f64) for k, v in weights.items()}
+    ids = torch.as_tensor(ids)
+    T = ids.shape[0]
+    step_rows = torch.as_tensor(step_rows)
+    split = (step_rows <= 16)[:, None]
+    pre_round = (step_rows > library_rows)[:, None] if library_rows else torch.zeros(T, 1, dtype=torch.bool)
+    positions = torch.arange(T)
+    eps = cfg["rms_norm_eps"]
+    nq = cfg["num_attention_heads"]
+    nkv = cfg.get("num_key_value_heads") or nq
+    d = cfg.get("head_dim") or cfg["hidden_size"] // nq
+    theta = cfg.get("rope_theta", 10000.0)
+
+    def normed(x, weight, may_split):
+        """(input of the products, factor on their results)"""
+        whole = to_bf16(rmsnorm(x, weight, eps))
+        if not may_split:
+            return whole, torch.ones(T, 1, dtype=f64)
+        r = 1.0 / torch.sqrt((x * x).sum(-1, keepdim=True) / x.shape[-1] + eps)
+        return torch.where(split, to_bf16(x * weight), whole), torch.where(split, r, torch.ones_like(r))
+
+    x = embedding(w["model.embed_tokens.weight"], ids)
+    for i in range(cfg["num_hidden_layers"]):
+        p = f"model.layers.{i}."
+        y, r = normed(x, w[p + "input_layernorm.weight"], i > 0)
+        q = (linear(y, w[p + "self_attn.q_proj.weight"]) * r).view(T, nq, d)
+        k = (linear(y, w[p + "self_attn.k_proj.weight"]) * r).view(T, nkv, d)
+        v = (linear(y, w[p + "self_attn.v_proj.weight"]) * r).view(T, nkv, d)
+        q, k, v = to_bf16(rope(q, positions, theta)), to_bf16(rope(k, positions, theta)), to_bf16(v)
+        mask = visible(positions, cfg.get("sliding_window"))
+        ctx = torch.empty_like(q)
+        for h in range(nq):
+            kvh = h // (nq // nkv)
+            s = (q[:, h, :] @ k[:, kvh, :].t()) * (1.0 / math.sqrt(d))
+            s = s.masked_fill(~mask, float("-inf"))
+            e = torch.exp(s - s.max(dim=-1, keepdim=True).values)
+            ctx[:, h, :] = (to_bf16(e) @ v[:, kvh, :]) / e.sum(dim=-1, keepdim=True)
+        x = x + linear(to_bf16(ctx).reshape(T, nq * d), w[p + "self_attn.o_proj.weight"])
+        y, r = normed(x, w[p + "post_attention_layernorm.weight"], True)
+        g = linear(y, w[p + "mlp.gate_proj.weight"]) * r
+        u = linear(y, w[p + "mlp.up_proj.weight"]) * r
+        g, u = torch.where(pre_round, to_bf16(g), g), torch.where(pre_round, to_bf16(u), u)
+        x = x + linear(to_bf16(silu(g) * u), w[p + "mlp.down_proj.weight"])
+    y = to_bf16(rmsnorm(x, w["model.norm.weight"], eps))
+    head = "model.embed_tokens.weight" if cfg.get("tie_word_embeddings") else "lm_head.weight"
+    return linear(y, w[head])

@@ -14,7 +14,7 @@ import torch
 
 import plain_mistral as plain
 from test_gpu_kernels import philox_uniform
-from util import CONFIGS, TOL, make_model_dir, prompts, read_model_dir, rel_err
+from util import CONFIGS, TOL, make_model_dir, prompts, read_model_dir, rel_err, within_the_format
 
 pytestmark = pytest.mark.gpu
 REPO = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -630,7 +630,7 @@ def test_random_configurations(tmp_path, seed):
     nkv = rng.choice([1, 2, 3, 4])
     nq = nkv * rng.choice([1, 2, 3, 5, 8, 17] if d <= 64 else [1, 2, 4])
     cfg = {"architectures": ["MistralForCausalLM"], "model_type": "mistral",
-           "num_hidden_layers": rng.choice([1, 2, 3]), "hidden_size": rng.choice([40, 72, 96, 136, 200, 264]),
+           "num_hidden_layers": rng.choice([1, 2, 3]), "hidden_size": rng.choice([40, 72, 96, 136, 200, 264, 1024, 2048]),
            "num_attention_heads": nq, "num_key_value_heads": nkv, "head_dim": d,
            "intermediate_size": rng.choice([64, 96, 160, 224, 352]), "vocab_size": rng.choice([130, 257, 384, 1000]),
            "rope_theta": rng.choice([500.0, 10000.0, 1e6]), "sliding_window": rng.choice([None, 7, 64, 70, 150]),
@@ -640,25 +640,37 @@ def test_random_configurations(tmp_path, seed):
     cfgd, w = read_model_dir(mdir)
     lens = [rng.choice([1, 5, 33, 64, 65, 100, 129, 200]) for _ in range(rng.choice([1, 2, 3, 5]))]
     ids = prompts(cfg["vocab_size"], lens, seed=100 + seed)
-    wants = [plain.forward(w, cfgd, p, dtype=torch.float32) for p in ids]
+    wants = [plain.forward(w, cfgd, p) for p in ids]
     for dtype in DTYPES:
         eng = Engine(load_model(mdir, dtype), max_tokens=64 * (sum(-(-n // 64) for n in lens) + 2))
         slots = [eng.alloc() for _ in ids]
         tail = [min(len(p) - 1, rng.choice([0, 1, 7, 32])) for p in ids]
         heads = [len(p) - t for p, t in zip(ids, tail)]
         lg = eng.step([SeqInput(s, p[:h], list(range(h))) for s, p, h in zip(slots, ids, heads)]).clone()
-        worst, o = 0.0, 0
+        got, o = [[] for _ in ids], 0
         for i, h in enumerate(heads):
-            worst = max(worst, rel_err(lg[o:o + h], wants[i][:h]))
+            got[i].append(lg[o:o + h])
             o += h
         for t in range(max(tail)):
             live = [i for i in range(len(ids)) if t < tail[i]]
             lg = eng.step([SeqInput(slots[i], [ids[i][heads[i] + t]], [0]) for i in live]).clone()
             for r, i in enumerate(live):
-                worst = max(worst, rel_err(lg[r:r + 1], wants[i][heads[i] + t:heads[i] + t + 1]))
+                got[i].append(lg[r:r + 1])
         for s in slots:
             eng.free(s)
-        assert worst < TOL[dtype], (cfg, lens, tail, dtype, worst)
+        eng.close()
+        got = [torch.cat(g) for g in got]
+        # The engine is held to what the format costs an implementation that shares nothing with
+        # it, on these very requests (float32 sums; bfloat16 roundings where the engine has them),
+        # not to a tolerance fixed for other sizes.
+        if dtype == "float32":
+            worst = max(rel_err(g, x) for g, x in zip(got, wants))
+            cost = max(rel_err(plain.forward(w, cfgd, p, dtype=torch.float32), x) for p, x in zip(ids, wants))
+            assert worst < max(TOL[dtype], 2 * cost), (cfg, lens, tail, worst, cost)
+        else:
+            rows = [[sum(heads)] * h + [sum(1 for t2 in tail if t < t2) for t in range(tl)] for h, tl in zip(heads, tail)]
+            ok, numbers = within_the_format(got, [plain.forward_rounded(w, cfgd, p, r) for p, r in zip(ids, rows)], wants)
+            assert ok, (cfg, lens, tail, numbers)
 
 
 @pytest.mark.parametrize("H,nq,nkv,d,I", [(128, 4, 2, 32, 192), (512, 8, 2, 64, 320)])

@@ -270,3 +270,38 @@ def test_draw():
     p = torch.tensor([0.2, 0.3, 0.5], dtype=D)
     assert [plain.draw(p, r) for r in (0.0, 0.2, 0.21, 0.5, 0.51, 0.999)] == [0, 0, 1, 1, 2, 2]
     assert plain.draw(torch.tensor([0.2, 0.3], dtype=D), 0.9) == 1         # never reached: last index
+
+
+# ---- the variant with the engine's bfloat16 roundings --------------------------------
+
+def test_to_bf16_rounds_to_nearest_even():
+    one = 1.0
+    ulp = 2.0 ** -7                                          # spacing of bfloat16 in [1, 2)
+    x = torch.tensor([one + 0.49 * ulp, one + 0.51 * ulp, one + 0.5 * ulp, one + 1.5 * ulp, -3.0, 0.0], dtype=torch.float64)
+    want = torch.tensor([one, one + ulp, one, one + 2 * ulp, -3.0, 0.0], dtype=torch.float64)   # ties go to the even mantissa
+    assert torch.equal(plain.to_bf16(x), want)
+
+
+def test_rounded_forward_is_the_plain_forward_when_nothing_is_rounded(monkeypatch):
+    """With the rounding taken out, `forward_rounded` must give `forward`'s logits, in both
+    forms of the norm and with and without the rounding of gate and up: its formulas are the
+    plain ones, only the roundings are its own."""
+    cfg, w = _tiny(seed=5, num_hidden_layers=3, head_dim=6, sliding_window=9)
+    ids = torch.randint(0, cfg["vocab_size"], (40,), generator=torch.Generator().manual_seed(3)).tolist()
+    want = plain.forward(w, cfg, ids)
+    monkeypatch.setattr(plain, "to_bf16", lambda t: t)
+    for rows in ([40] * 40, [1] * 40, [100] * 30 + [3] * 10):
+        got = plain.forward_rounded(w, cfg, ids, rows)
+        assert float((got - want).abs().max()) < 1e-10 * float(want.abs().max()), rows
+
+
+def test_rounded_forward_is_near_and_not_equal():
+    cfg, w = _tiny(seed=6)
+    ids = torch.randint(0, cfg["vocab_size"], (30,), generator=torch.Generator().manual_seed(4)).tolist()
+    want = plain.forward(w, cfg, ids)
+    whole, single = plain.forward_rounded(w, cfg, ids, [30] * 30), plain.forward_rounded(w, cfg, ids, [1] * 30)
+    err = lambda a: float((a - want).abs().max() / want.abs().max())
+    assert 1e-4 < err(whole) < 5e-2 and 1e-4 < err(single) < 5e-2
+    assert not torch.equal(whole, single)                   # the norm cut in two rounds elsewhere
+    first = plain.forward_rounded(w, cfg, ids[:1], [30])
+    assert float((whole[:1] - first).abs().max()) < 1e-9       # a row depends on its prefix only

@@ -46,6 +46,27 @@ def rel_err(got: torch.Tensor, want: torch.Tensor) -> float:
     return float((got - want).abs().max() / (want.abs().max() + 1e-30))
 
 
+def rms_err(got: torch.Tensor, want: torch.Tensor) -> float:
+    """Root mean square of the difference as a share of the root mean square of `want`: a far
+    steadier measure of rounding noise than the largest difference."""
+    got, want = got.double().cpu(), want.double().cpu()
+    assert got.shape == want.shape, (got.shape, want.shape)
+    return float(((got - want) ** 2).mean().sqrt() / ((want ** 2).mean().sqrt() + 1e-30))
+
+
+def within_the_format(got, rounded, exact):
+    """Is the engine's bfloat16 result `got` as far from the float64 logits `exact` as the format
+    makes it, and no further?  `rounded`: the plain implementation with the same roundings.
+    (Lists of tensors, one a request.)  The root mean square over all logits may exceed the plain
+    implementation's by a quarter, the largest difference (the maximum of as many draws, which
+    scatters more, most at small widths) by a factor of two.  Returns (ok, the four numbers)."""
+    g, r, x = torch.cat(list(got)), torch.cat(list(rounded)), torch.cat(list(exact))
+    rms, rms_cost = rms_err(g, x), rms_err(r, x)
+    top, top_cost = rel_err(g, x), rel_err(r, x)
+    ok = rms < 1.25 * rms_cost + 1e-4 and top < 2.0 * top_cost + 1e-3
+    return ok, dict(rms=rms, rms_of_roundings=rms_cost, largest=top, largest_of_roundings=top_cost)
+
+
 def make_model_dir(tmp, name: str, dtype=torch.bfloat16) -> str:
     from torchless_rs_amd import write_random_model
     d = os.path.join(str(tmp), f"tiny_{name}_{str(dtype).split('.')[-1]}")
