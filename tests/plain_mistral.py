@@ -15,7 +15,7 @@ import torch
 
 def embedding(table: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
     """Row copy, no scaling.  src/model/modules/embedding.rs:15-21"""
-    return table[ids.long()]
+    return table[ids.long().to(table.device)]
 
 
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
@@ -31,11 +31,11 @@ def linear(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     return x @ w.t()
 
 
-def rope_inv_freq(head_dim: int, theta: float, dtype=torch.float64) -> torch.Tensor:
+def rope_inv_freq(head_dim: int, theta: float, dtype=torch.float64, device=None) -> torch.Tensor:
     """inv_freq[i] = 1 / theta^(i / (d/2)).  src/kernels/mod.rs:572-579"""
     half = head_dim // 2
-    i = torch.arange(half, dtype=dtype)
-    return 1.0 / torch.pow(torch.tensor(theta, dtype=dtype), i / half)
+    i = torch.arange(half, dtype=dtype, device=device)
+    return 1.0 / torch.pow(torch.tensor(theta, dtype=dtype, device=device), i / half)
 
 
 def rope(x: torch.Tensor, positions: torch.Tensor, theta: float) -> torch.Tensor:
@@ -44,7 +44,7 @@ def rope(x: torch.Tensor, positions: torch.Tensor, theta: float) -> torch.Tensor
     src/kernels/mod.rs:582-608"""
     d = x.shape[-1]
     half = d // 2
-    inv = rope_inv_freq(d, theta, x.dtype)
+    inv = rope_inv_freq(d, theta, x.dtype, x.device)
     ang = positions.to(x.dtype)[:, None] * inv[None, :]          # [T, d/2]
     c = torch.cos(ang)[:, None, :]
     s = torch.sin(ang)[:, None, :]
@@ -132,18 +132,34 @@ def block(x, w, prefix, cfg, positions) -> torch.Tensor:
     return x
 
 
+def forward_many(weights, cfg: dict, many_ids, dtype=torch.float64):
+    """Logits [T, V] of each of several whole sequences.  `weights` is read name by name, a
+    layer at a time (so a large model need not be held in `dtype` at once), and the arithmetic
+    runs where its tensors lie.  src/model/mod.rs:430-447"""
+    take = lambda name: weights[name].to(dtype)
+    table = take("model.embed_tokens.weight")
+    xs, positions = [], []
+    for ids in many_ids:
+        ids = torch.as_tensor(ids)
+        xs.append(embedding(table, ids))
+        positions.append(torch.arange(ids.shape[0], device=table.device))
+    for i in range(cfg["num_hidden_layers"]):
+        prefix = f"model.layers.{i}."
+        w = {prefix + n: take(prefix + n) for n in LAYER_TENSORS}
+        xs = [block(x, w, prefix, cfg, pos) for x, pos in zip(xs, positions)]
+    norm = take("model.norm.weight")
+    head = table if cfg.get("tie_word_embeddings") else take("lm_head.weight")
+    return [linear(rmsnorm(x, norm, cfg["rms_norm_eps"]), head) for x in xs]
+
+
+LAYER_TENSORS = ("input_layernorm.weight", "post_attention_layernorm.weight", "self_attn.q_proj.weight",
+                 "self_attn.k_proj.weight", "self_attn.v_proj.weight", "self_attn.o_proj.weight",
+                 "mlp.gate_proj.weight", "mlp.up_proj.weight", "mlp.down_proj.weight")
+
+
 def forward(weights: dict, cfg: dict, ids, dtype=torch.float64) -> torch.Tensor:
     """Logits [T, V] of one whole sequence.  src/model/mod.rs:430-447"""
-    w = {k: v.to(dtype) for k, v in weights.items()}
-    ids = torch.as_tensor(ids)
-    T = ids.shape[0]
-    positions = torch.arange(T)
-    x = embedding(w["model.embed_tokens.weight"], ids)
-    for i in range(cfg["num_hidden_layers"]):
-        x = block(x, w, f"model.layers.{i}.", cfg, positions)
-    x = rmsnorm(x, w["model.norm.weight"], cfg["rms_norm_eps"])
-    head = "model.embed_tokens.weight" if cfg.get("tie_word_embeddings") else "lm_head.weight"
-    return linear(x, w[head])
+    return forward_many(weights, cfg, [ids], dtype)[0]
 
 
 # --- sampling --------------------------------------------------------------
@@ -267,13 +283,15 @@ def forward_rounded(weights: dict, cfg: dict, ids, step_rows, library_rows=64) -
     realisation of the same rounding.)
     The formulas are those of the functions above; only the roundings are added."""
     f64 = torch.float64
-    w = {k: v.to(f64) for k, v in weights.items()}
+    take = lambda name: weights[name].to(f64)            # a layer at a time, where the tensors lie
+    table = take("model.embed_tokens.weight")
+    dev = table.device
     ids = torch.as_tensor(ids)
     T = ids.shape[0]
-    step_rows = torch.as_tensor(step_rows)
+    step_rows = torch.as_tensor(step_rows, device=dev)
     split = (step_rows <= 16)[:, None]
-    pre_round = (step_rows > library_rows)[:, None] if library_rows else torch.zeros(T, 1, dtype=torch.bool)
-    positions = torch.arange(T)
+    pre_round = (step_rows > library_rows)[:, None] if library_rows else torch.zeros(T, 1, dtype=torch.bool, device=dev)
+    positions = torch.arange(T, device=dev)
     eps = cfg["rms_norm_eps"]
     nq = cfg["num_attention_heads"]
     nkv = cfg.get("num_key_value_heads") or nq
@@ -284,13 +302,14 @@ def forward_rounded(weights: dict, cfg: dict, ids, step_rows, library_rows=64) -
         """(input of the products, factor on their results)"""
         whole = to_bf16(rmsnorm(x, weight, eps))
         if not may_split:
-            return whole, torch.ones(T, 1, dtype=f64)
+            return whole, torch.ones(T, 1, dtype=f64, device=dev)
         r = 1.0 / torch.sqrt((x * x).sum(-1, keepdim=True) / x.shape[-1] + eps)
         return torch.where(split, to_bf16(x * weight), whole), torch.where(split, r, torch.ones_like(r))
 
-    x = embedding(w["model.embed_tokens.weight"], ids)
+    x = embedding(table, ids)
     for i in range(cfg["num_hidden_layers"]):
         p = f"model.layers.{i}."
+        w = {p + n: take(p + n) for n in LAYER_TENSORS}
         y, r = normed(x, w[p + "input_layernorm.weight"], i > 0)
         q = (linear(y, w[p + "self_attn.q_proj.weight"]) * r).view(T, nq, d)
         k = (linear(y, w[p + "self_attn.k_proj.weight"]) * r).view(T, nkv, d)
@@ -310,6 +329,5 @@ def forward_rounded(weights: dict, cfg: dict, ids, step_rows, library_rows=64) -
         u = linear(y, w[p + "mlp.up_proj.weight"]) * r
         g, u = torch.where(pre_round, to_bf16(g), g), torch.where(pre_round, to_bf16(u), u)
         x = x + linear(to_bf16(silu(g) * u), w[p + "mlp.down_proj.weight"])
-    y = to_bf16(rmsnorm(x, w["model.norm.weight"], eps))
-    head = "model.embed_tokens.weight" if cfg.get("tie_word_embeddings") else "lm_head.weight"
-    return linear(y, w[head])
+    y = to_bf16(rmsnorm(x, take("model.norm.weight"), eps))
+    return linear(y, table if cfg.get("tie_word_embeddings") else take("lm_head.weight"))
