@@ -52,6 +52,24 @@ def rope(x: torch.Tensor, positions: torch.Tensor, theta: float) -> torch.Tensor
     return torch.cat([a * c - b * s, a * s + b * c], dim=-1)
 
 
+def rope_variant(x: torch.Tensor, positions: torch.Tensor, theta: float, rotary_dim: int,
+                 interleaved: bool) -> torch.Tensor:
+    """Not the reference's rotation, but the family around it that the tests' toy position
+    encodings use: only the first `rotary_dim` channels of a head are rotated (frequencies
+    1 / theta^(i / (rotary_dim/2))), in pairs (i, i + rotary_dim/2), or (2i, 2i+1) when
+    `interleaved`; the other channels pass through.  With rotary_dim = d and halves it is `rope`."""
+    if rotary_dim == 0:
+        return x.clone()
+    head, rest = x[..., :rotary_dim], x[..., rotary_dim:]
+    if interleaved:                       # bring the pairs (2i, 2i+1) to (i, i + r/2), rotate, bring them back
+        order = torch.cat([torch.arange(0, rotary_dim, 2), torch.arange(1, rotary_dim, 2)]).to(x.device)
+        back = torch.argsort(order)
+        head = rope(head[..., order], positions, theta)[..., back]
+    else:
+        head = rope(head, positions, theta)
+    return torch.cat([head, rest], dim=-1)
+
+
 def visible(positions: torch.Tensor, window) -> torch.Tensor:
     """mask[p, j]: key j visible to the query at p iff j <= p, and with a
     window W, not (p >= W and j < p - W + 1).  Causality:

@@ -996,3 +996,92 @@ def test_attention_over_a_long_context(ops, window):
     rows = [0, 63, 64, 4095, 4096, 4097, 40000, L, T - 1]
     assert rel_err(outp[rows], want(rows)) < KTOL["bfloat16"]
     assert torch.isfinite(outp.float()).all()
+
+
+# ---- other rotations than the reference's: a share of the head, interleaved pairs, none ----------
+
+ROTATIONS = [(1.0, False), (1.0, True), (0.5, False), (0.5, True), (0.25, True), (0.0, False)]
+
+
+def rotation_for(ops, d, theta, share, interleaved):
+    r = int(d * share) // 2 * 2
+    if r == 0:
+        return ops.NO_ROTATION, 0
+    inv = plain.rope_inv_freq(r, theta).to(torch.float32).to(DEV)
+    return ops.Rotation(inv, r, interleaved), r
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("share,interleaved", ROTATIONS)
+@pytest.mark.parametrize("nq,nkv,d", [(3, 1, 48), (4, 2, 128), (2, 2, 16)])
+def test_rope_split_and_commit_take_any_rotation(ops, dt, share, interleaved, nq, nkv, d):
+    """`rope_split` against the plain rotation of the same family, and `rope_commit` bit for bit
+    what `rope_split` and `kv_commit` give."""
+    theta, lens = 500.0, [0, 63, 300, 5]
+    rot, r = rotation_for(ops, d, theta, share, interleaved)
+    a = paged_case(ops, dt, nq, nkv, d, None, lens_cached=lens, lens_new=[1] * len(lens), seed=31)
+    n = len(lens)
+    qkv = rnd(n, (nq + 2 * nkv) * d, seed=32).to(DEV)
+    q1, k1, v1 = (torch.empty(n, h, d, dtype=DT[dt], device=DEV) for h in (nq, nkv, nkv))
+    ops.rope_split(qkv, a["row_pos"], rot, nq, nkv, d, q1, k1, v1)
+    x = qkv.double().cpu().view(n, nq + 2 * nkv, d)
+    pos = a["row_pos"].cpu().long()
+    wq = plain.rope_variant(x[:, :nq], pos, theta, r, interleaved)
+    wk = plain.rope_variant(x[:, nq:nq + nkv], pos, theta, r, interleaved)
+    for row, p in enumerate(pos.tolist()):              # float32 angles: off by up to 1.2e-7 * p radians
+        tol = KTOL[dt] + 1.2e-7 * p
+        assert rel_err(q1[row], wq[row]) < tol and rel_err(k1[row], wk[row]) < tol, (row, p)
+    assert torch.equal(v1.cpu(), x[:, nq + nkv:].to(DT[dt]))
+    if r < d:                                        # what is not rotated is copied, not computed
+        assert torch.equal(q1[..., r:].cpu(), x[:, :nq, r:].to(DT[dt]))
+    pages1 = a["pages"].clone()
+    ops.kv_commit(k1, v1, a["row_seq"], a["row_pos"], a["after"], a["table"], a["ring"], pages1)
+    q2, pages2 = torch.full_like(q1, float("nan")), a["pages"].clone()
+    ops.rope_commit(qkv, a["row_pos"], rot, a["table"], a["ring"], nq, nkv, d, q2, pages2)
+    assert torch.equal(q1, q2)
+    assert torch.equal(torch.nan_to_num(pages1.float(), nan=-7.0), torch.nan_to_num(pages2.float(), nan=-7.0))
+
+
+@pytest.mark.parametrize("share,interleaved", ROTATIONS[1:])
+@pytest.mark.parametrize("nq,nkv,d,K,lens", [(6, 2, 48, 64, [0, 63, 64, 300]), (8, 2, 128, 1024, [9, 64, 640, 2, 3, 70, 71]),
+                                             (2, 1, 16, 72, [5, 6])])
+def test_qkv_rope_commit_takes_any_rotation(ops, share, interleaved, nq, nkv, d, K, lens):
+    """The fused kernel of single-token steps, from the weights as stored and from the tiled copy in
+    the order of this rotation's pairs: the bits of the product followed by `rope_commit`."""
+    rot, r = rotation_for(ops, d, 10000.0, share, interleaved)
+    n = len(lens)
+    c = paged_case(ops, "bfloat16", nq, nkv, d, None, lens_cached=lens, lens_new=[1] * n, seed=33, n_pages=60)
+    y = rnd(n, K, seed=34, dtype=torch.bfloat16).to(DEV)
+    w = rnd((nq + 2 * nkv) * d, K, seed=35, dtype=torch.bfloat16, scale=0.2).to(DEV)
+    qkv = torch.empty(n, (nq + 2 * nkv) * d, device=DEV)
+    ops.gemm(y, w, qkv)
+    q1 = torch.empty(n, nq, d, dtype=torch.bfloat16, device=DEV)
+    pages1 = c["pages"].clone()
+    ops.rope_commit(qkv, c["row_pos"], rot, c["table"], c["ring"], nq, nkv, d, q1, pages1)
+    rows = ops.qkv_tile_rows(nq, nkv, d, DEV, rot)
+    assert sorted(rows.tolist()) == list(range((nq + 2 * nkv) * d))
+    if interleaved:
+        assert rows[:16].tolist() == list(range(0, 16, 2)) + list(range(1, 16, 2))
+    tiles = ops.tile_weights(w, rows) if K % 64 == 0 else None
+    for t in (None, tiles):
+        for kv_half in (False, True):
+            q2, pages2 = torch.full_like(q1, float("nan")), c["pages"].clone()
+            ops.qkv_rope_commit(y, w, c["row_pos"], rot, c["table"], c["ring"], nq, nkv, d, q2, pages2,
+                                kv_half=kv_half, tiles=t)
+            assert torch.equal(q1, q2), (t is not None, kv_half)
+            assert torch.equal(torch.nan_to_num(pages1.float(), nan=-7.0), torch.nan_to_num(pages2.float(), nan=-7.0))
+    full = (y.double().cpu() @ w.double().cpu().t()).view(n, nq + 2 * nkv, d)
+    assert rel_err(q1, plain.rope_variant(full[:, :nq], c["row_pos"].cpu().long(), 10000.0, r, interleaved)) < KTOL["bfloat16"]
+
+
+def test_rotations_that_cannot_be_are_refused(ops):
+    qkv = torch.zeros(2, 4 * 16, device=DEV)
+    pos = torch.zeros(2, dtype=torch.int32, device=DEV)
+    q, k, v = (torch.empty(2, h, 16, device=DEV) for h in (2, 1, 1))
+    inv = torch.ones(9, device=DEV)
+    with pytest.raises(ops.KernelError, match="rotated channels"):
+        ops.rope_split(qkv, pos, ops.Rotation(inv, 18), 2, 1, 16, q, k, v)           # more than the head
+    with pytest.raises(ops.KernelError, match="rotated channels"):
+        ops.rope_split(qkv, pos, ops.Rotation(inv[:3].contiguous(), 7), 2, 1, 16, q, k, v)    # odd
+    with pytest.raises(ops.KernelError, match="inv_freq"):
+        ops.rope_split(qkv, pos, ops.Rotation(inv, 8), 2, 1, 16, q, k, v)            # 9 frequencies for 4 pairs

@@ -44,6 +44,12 @@ def test_position_part():
     from torchless_rs_amd.parts import PartSpec, make_part
     rot = make_part("position", PartSpec("rotary", {"head_dim": 48, "theta": 500.0}))
     f = rot.inv_freq(DEV).cpu()
+    r = rot.rotation(DEV)
+    assert (r.rotary_dim, r.interleaved) == (48, False) and r.inv_freq is rot.inv_freq(DEV)
+    assert make_part("position", PartSpec("none", {})).rotation(DEV) is None
+    part = make_part("position", PartSpec("rotary", {"head_dim": 48, "theta": 500.0, "rotary_dim": 16, "interleaved": True}))
+    assert (part.rotation(DEV).rotary_dim, part.rotation(DEV).interleaved) == (16, True)
+    assert rel_err(part.inv_freq(DEV).cpu(), plain.rope_inv_freq(16, 500.0)) < 1e-7
     assert f.shape == (24,) and f[0] == 1.0 and bool((f[1:] < f[:-1]).all())     # kernels/tests.rs:54-69
     assert rel_err(f, plain.rope_inv_freq(48, 500.0)) < 1e-7
     with pytest.raises(ValueError):
@@ -494,3 +500,101 @@ def test_a_toy_position_encoding():
                        "rms_norm_eps": 1e-5}, ids)) > 1e-3           # and it is not the plain rotation
     finally:
         unregister_part("position", "stretched_rotary")
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("rotary_dim,interleaved", [(16, True), (32, True), (16, False), (None, False)])
+def test_other_names_fused_tensors_and_another_rotation_without_a_new_class(dt, rotary_dim, interleaved):
+    """What another architecture with the same mathematics may differ in is data: the tensors'
+    names (also of the norms), q|k|v and gate|up stored as one tensor each, a rotation of a share
+    of the head in interleaved pairs, or no rotation.  The parts are the framework's own, chosen
+    and parameterised by the specification; no class is defined here.  Whole prompts, then tokens
+    one by one (the fused single-token kernels read tiled copies laid out for this rotation)."""
+    from torchless_rs_amd.engine import Engine, SeqInput
+    from torchless_rs_amd.engine.model import Model
+    from torchless_rs_amd.parts import LayerSpec, ModelSpec, PartSpec, Run
+    from torchless_rs_amd.weights import TensorDict, random_tensors
+    H, V, I, nq, nkv, d, L, theta, window, eps = 128, 90, 192, 4, 2, 32, 2, 300.0, 40, 1e-5
+    if rotary_dim is None:
+        position = PartSpec("none", {})
+    else:
+        position = PartSpec("rotary", {"head_dim": d, "theta": theta, "rotary_dim": rotary_dim, "interleaved": interleaved})
+    norm = PartSpec("rmsnorm", {"size": H, "eps": eps})
+    layers = [LayerSpec(prefix=f"h.{i}.",
+                        mixer=PartSpec("attention", {"hidden_size": H, "n_heads": nq, "n_kv_heads": nkv, "head_dim": d,
+                                                     "window": window, "position": position, "prefix": "attn.",
+                                                     "names": {"qkv": "qkv_proj.weight", "o": "dense.weight"}}),
+                        ffn=PartSpec("swiglu", {"hidden_size": H, "intermediate_size": I, "prefix": "ff.",
+                                                "names": {"gate_up": "gate_up_proj.weight", "down": "fc2.weight"}}),
+                        mixer_norm=norm, ffn_norm=norm,
+                        block=PartSpec("pre_norm", {"mixer_norm_name": "ln_1.", "ffn_norm_name": "ln_2."}))
+              for i in range(L)]
+    spec = ModelSpec(hidden_size=H, vocab_size=V,
+                     embedding=PartSpec("tokens", {"vocab_size": V, "hidden_size": H, "name": "wte.weight"}),
+                     embedding_prefix="", layers=layers, schedule=[Run(i) for i in range(L)],
+                     final_norm=norm, final_norm_prefix="ln_f.",
+                     head=PartSpec("linear", {"vocab_size": V, "hidden_size": H, "name": "out.weight"}), head_prefix="")
+    names = set(spec.weight_specs())
+    assert names == {"wte.weight", "ln_f.weight", "out.weight"} | {
+        f"h.{i}.{n}" for i in range(L) for n in ("ln_1.weight", "ln_2.weight", "attn.qkv_proj.weight", "attn.dense.weight",
+                                                   "ff.gate_up_proj.weight", "ff.fc2.weight")}
+    w = random_tensors(spec.weight_specs(), seed=12, std=0.08, norm_std=0.1, dtype=torch.bfloat16)
+    model = Model(spec, None, DT[dt], DEV)
+    model.load_weights(TensorDict(w))
+    eng = Engine(model, max_tokens=64 * 6)
+
+    def plain_forward(ids):
+        wd = {k: v.double() for k, v in w.items()}
+        T, pos = len(ids), torch.arange(len(ids))
+        x = wd["wte.weight"][ids]
+        for i in range(L):
+            p = f"h.{i}."
+            y = plain.rmsnorm(x, wd[p + "ln_1.weight"], eps)
+            qkv = plain.linear(y, wd[p + "attn.qkv_proj.weight"]).view(T, nq + 2 * nkv, d)
+            q, k, v = qkv[:, :nq], qkv[:, nq:nq + nkv], qkv[:, nq + nkv:]
+            q = plain.rope_variant(q, pos, theta, rotary_dim or 0, interleaved)
+            k = plain.rope_variant(k, pos, theta, rotary_dim or 0, interleaved)
+            a = plain.attention_core(q, k, v, pos, window).reshape(T, nq * d)
+            x = x + plain.linear(a, wd[p + "attn.dense.weight"])
+            gu = plain.linear(plain.rmsnorm(x, wd[p + "ln_2.weight"], eps), wd[p + "ff.gate_up_proj.weight"])
+            x = x + plain.linear(plain.silu(gu[:, :I]) * gu[:, I:], wd[p + "ff.fc2.weight"])
+        return plain.linear(plain.rmsnorm(x, wd["ln_f.weight"], eps), wd["out.weight"])
+
+    g = torch.Generator().manual_seed(13)
+    seqs = [torch.randint(0, V, (n,), generator=g).tolist() for n in (70, 9, 33)]
+    wants = [plain_forward(s) for s in seqs]
+    tol = {"float32": 2e-5, "bfloat16": 3e-2}[dt]
+    for tail in (0, 20):
+        slots = [eng.alloc() for _ in seqs]
+        heads = [max(1, len(s) - tail) for s in seqs]
+        lg = eng.step([SeqInput(sl, s[:h], list(range(h))) for sl, s, h in zip(slots, seqs, heads)]).clone()
+        o = 0
+        for i, h in enumerate(heads):
+            assert rel_err(lg[o:o + h], wants[i][:h]) < tol, (tail, i)
+            o += h
+        for t in range(tail):
+            live = [i for i in range(len(seqs)) if heads[i] + t < len(seqs[i])]
+            lg = eng.step([SeqInput(slots[i], [seqs[i][heads[i] + t]], [0]) for i in live]).clone()
+            for r, i in enumerate(live):
+                assert rel_err(lg[r:r + 1], wants[i][heads[i] + t:heads[i] + t + 1]) < tol, (tail, t, i)
+        for sl in slots:
+            eng.free(sl)
+    if dt == "bfloat16":                       # the single-token steps did run the fused kernel on its tiled copy
+        assert all(b.mixer.qkv.own_tiles is not None for b in model.blocks)
+    eng.close()
+
+
+def test_part_parameters_that_cannot_be_are_refused():
+    from torchless_rs_amd.parts import PartSpec, make_part
+    rot = PartSpec("rotary", {"head_dim": 16, "theta": 10.0})
+    base = {"hidden_size": 32, "n_heads": 2, "n_kv_heads": 1, "head_dim": 16, "position": rot}
+    with pytest.raises(ValueError, match="no tensors called"):
+        make_part("mixer", PartSpec("attention", dict(base, names={"query": "wq"})))
+    with pytest.raises(ValueError, match="q alone"):
+        make_part("mixer", PartSpec("attention", dict(base, own_kv=False, names={"qkv": "wqkv"})))
+    with pytest.raises(ValueError, match="no tensors called"):
+        make_part("ffn", PartSpec("swiglu", {"hidden_size": 32, "intermediate_size": 64, "names": {"w1": "x"}}))
+    with pytest.raises(ValueError, match="rotated channels"):
+        make_part("position", PartSpec("rotary", {"head_dim": 16, "theta": 10.0, "rotary_dim": 18}))
+    with pytest.raises(ValueError, match="rotated channels"):
+        make_part("position", PartSpec("rotary", {"head_dim": 16, "theta": 10.0, "rotary_dim": 7}))

@@ -80,6 +80,26 @@ def test_rope_identity_norm_and_pairing():
     assert abs(float(r[0, 0, 0]) - math.cos(1)) < 1e-12 and abs(float(r[0, 0, 2]) - math.sin(1)) < 1e-12
 
 
+def test_rope_variants_reduce_to_the_rotation():
+    """The toy family: all channels in halves is `rope`; interleaved pairs written out by hand;
+    channels behind `rotary_dim` untouched, and the rotated ones as a head of that size."""
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn(5, 3, 12, generator=g, dtype=D)
+    pos = torch.tensor([0, 1, 7, 30, 200])
+    assert torch.equal(plain.rope_variant(x, pos, 100.0, 12, False), plain.rope(x, pos, 100.0))
+    inter = plain.rope_variant(x, pos, 100.0, 12, True)
+    inv = plain.rope_inv_freq(12, 100.0)
+    for i in range(6):
+        ang = pos.to(D) * inv[i]
+        c, s = torch.cos(ang)[:, None], torch.sin(ang)[:, None]
+        a, b = x[..., 2 * i], x[..., 2 * i + 1]
+        assert torch.allclose(inter[..., 2 * i], a * c - b * s) and torch.allclose(inter[..., 2 * i + 1], a * s + b * c)
+    part = plain.rope_variant(x, pos, 100.0, 8, False)
+    assert torch.equal(part[..., 8:], x[..., 8:]) and torch.equal(part[..., :8], plain.rope(x[..., :8], pos, 100.0))
+    assert torch.equal(plain.rope_variant(x, pos, 100.0, 0, False), x)
+    assert not torch.allclose(inter, plain.rope(x, pos, 100.0))
+
+
 def test_rope_scores_depend_on_distance_only():
     g = torch.Generator().manual_seed(0)
     q = torch.randn(1, 1, 16, generator=g, dtype=D)

@@ -74,6 +74,26 @@ __device__ __forceinline__ void rotate_pair(float a, float b, float c, float s, 
   rb = as + bc;
 }
 
+// How q and k are rotated by position: the first `rotary_dim` channels of a head (even, at most
+// the head size; 0: no rotation at all) in pairs, pair i by the angle pos * inv_freq[i]; the
+// channels behind them are passed through.
+struct Rotation {
+  const float* inv_freq;   // [rotary_dim / 2]
+  int rotary_dim;
+  int interleaved;         // pairs (2i, 2i+1); else (i, i + rotary_dim/2)
+};
+// The two channels of pair i of a head, i < d/2.  Pairs from rotary_dim/2 on are not rotated;
+// they are numbered so that the d/2 pairs cover every channel once.
+__host__ __device__ __forceinline__ void pair_channels(int i, int rotary_dim, int interleaved, int& a, int& b) {
+  if (interleaved || 2 * i >= rotary_dim) {
+    a = 2 * i;
+    b = 2 * i + 1;
+  } else {
+    a = i;
+    b = i + rotary_dim / 2;
+  }
+}
+
 // ---- error channel -------------------------------------------------------
 void set_error(const char* fmt, ...);
 

@@ -136,22 +136,24 @@ __global__ void add_partials_kernel(float* __restrict__ x, const float* __restri
 
 // ---- rotation and split ------------------------------------------------------
 // qkv[n, :] = [q (nq*d) | k (nkv*d) | v (nkv*d)] in float.  q and k are rotated
-// in pairs (i, i + d/2) by the angle pos * inv_freq[i]; v is copied.
+// in pairs by the angle pos * inv_freq[i] (which channels make pair i, and how many
+// of a head's channels are rotated: `Rotation`, `pair_channels`); v is copied.
+// The reference rotates all channels in pairs (i, i + d/2):
 // src/kernels/mod.rs:582-608, src/model/modules/attention.rs:68-78.
 constexpr int ROPE_MAX_HALF = 128;      // head sizes up to 256
 
 template <typename TO>
 __global__ void rope_split_kernel(const float* __restrict__ qkv, const int* __restrict__ row_pos,
-                                  const float* __restrict__ inv_freq, int nq, int nkv, int d,
+                                  Rotation rot, int nq, int nkv, int d,
                                   TO* __restrict__ q, TO* __restrict__ k, TO* __restrict__ v,
                                   TO* __restrict__ vt, int vt_cols, const int* __restrict__ row_seq,
                                   const int* __restrict__ tile_off, const int* __restrict__ n_cached) {
   __shared__ float cs[ROPE_MAX_HALF], sn[ROPE_MAX_HALF];
   const int n = blockIdx.x;
-  const int half = d / 2;
+  const int half = d / 2, rot_pairs = rot.rotary_dim / 2;
   const float pos = (float)row_pos[n];
-  for (int i = threadIdx.x; i < half; i += blockDim.x) {     // the row's angles, once
-    const float ang = inv_freq[i] * pos;
+  for (int i = threadIdx.x; i < rot_pairs; i += blockDim.x) {     // the row's angles, once
+    const float ang = rot.inv_freq[i] * pos;
     sincosf(ang, &sn[i], &cs[i]);          // one routine for both, the same in every kernel that rotates
   }
   __syncthreads();
@@ -159,13 +161,14 @@ __global__ void rope_split_kernel(const float* __restrict__ qkv, const int* __re
   const int n_rot = (nq + nkv) * half;
   for (int t = threadIdx.x; t < n_rot; t += blockDim.x) {
     const int h = t / half, i = t % half;
-    const float c = cs[i], s = sn[i];
-    const float a = src[h * d + i], b = src[h * d + i + half];
-    float ra, rb;
-    rotate_pair(a, b, c, s, ra, rb);
+    int ia, ib;
+    pair_channels(i, rot.rotary_dim, rot.interleaved, ia, ib);
+    const float a = src[h * d + ia], b = src[h * d + ib];
+    float ra = a, rb = b;
+    if (i < rot_pairs) rotate_pair(a, b, cs[i], sn[i], ra, rb);
     TO* dst = (h < nq) ? q + ((size_t)n * nq + h) * d : k + ((size_t)n * nkv + (h - nq)) * d;
-    dst[i] = from_f32<TO>(ra);
-    dst[i + half] = from_f32<TO>(rb);
+    dst[ia] = from_f32<TO>(ra);
+    dst[ib] = from_f32<TO>(rb);
   }
   const float* vs = src + (size_t)(nq + nkv) * d;
   if (v != nullptr) {
@@ -332,13 +335,13 @@ kv_commit_tiles_kernel(const T* __restrict__ k, const T* __restrict__ vt, int vt
 template <typename T>
 __global__ void rope_commit_kernel(const float* __restrict__ qkv, int n_parts, size_t part_stride,
                                    const int* __restrict__ row_pos,
-                                   const float* __restrict__ inv_freq, const int* __restrict__ table,
+                                   Rotation rot, const int* __restrict__ table,
                                    int table_stride, int ring_pages, int nq, int nkv, int d,
                                    T* __restrict__ q, T* __restrict__ pages) {
   // blockIdx.y of gridDim.y takes its share of the (q and k) heads and of the values
   __shared__ float cs[ROPE_MAX_HALF], sn[ROPE_MAX_HALF];
   const int n = blockIdx.x;
-  const int half = d / 2;
+  const int half = d / 2, rot_pairs = rot.rotary_dim / 2;
   const int p = row_pos[n];
   const float pos = (float)p;
   const float* src = qkv + (size_t)n * (nq + 2 * nkv) * d;
@@ -346,8 +349,8 @@ __global__ void rope_commit_kernel(const float* __restrict__ qkv, int n_parts, s
   const int r = p % PAGE;
   T* kd = pages + (size_t)page * 2 * nkv * PAGE * d;
   T* vd = kd + (size_t)nkv * PAGE * d;
-  for (int i = threadIdx.x; i < half; i += blockDim.x) {
-    const float ang = inv_freq[i] * pos;
+  for (int i = threadIdx.x; i < rot_pairs; i += blockDim.x) {
+    const float ang = rot.inv_freq[i] * pos;
     sincosf(ang, &sn[i], &cs[i]);          // one routine for both, the same in every kernel that rotates
   }
   __syncthreads();
@@ -355,18 +358,19 @@ __global__ void rope_commit_kernel(const float* __restrict__ qkv, int n_parts, s
   const int h_lo = (int)((long long)heads * blockIdx.y / gridDim.y), h_hi = (int)((long long)heads * (blockIdx.y + 1) / gridDim.y);
   for (int t = h_lo * half + threadIdx.x; t < h_hi * half; t += blockDim.x) {
     const int h = t / half, i = t % half;
-    const float c = cs[i], s = sn[i];
-    float a = src[h * d + i], b = src[h * d + i + half];
+    int ia, ib;
+    pair_channels(i, rot.rotary_dim, rot.interleaved, ia, ib);
+    float a = src[h * d + ia], b = src[h * d + ib];
 #pragma unroll 4
     for (int sp = 1; sp < n_parts; ++sp) {
-      a += src[sp * part_stride + h * d + i];
-      b += src[sp * part_stride + h * d + i + half];
+      a += src[sp * part_stride + h * d + ia];
+      b += src[sp * part_stride + h * d + ib];
     }
-    float ra, rb;
-    rotate_pair(a, b, c, s, ra, rb);
+    float ra = a, rb = b;
+    if (i < rot_pairs) rotate_pair(a, b, cs[i], sn[i], ra, rb);
     T* dst = (h < nq) ? q + ((size_t)n * nq + h) * d : kd + ((size_t)(h - nq) * PAGE + r) * d;
-    dst[i] = from_f32<T>(ra);
-    dst[i + half] = from_f32<T>(rb);
+    dst[ia] = from_f32<T>(ra);
+    dst[ib] = from_f32<T>(rb);
   }
   const float* vs = src + (size_t)(nq + nkv) * d;
   const int v_lo = (int)((long long)nkv * d * blockIdx.y / gridDim.y), v_hi = (int)((long long)nkv * d * (blockIdx.y + 1) / gridDim.y);
@@ -513,19 +517,24 @@ int tl_add_partials(float* x, const float* parts, int n_parts, int n, int H, hip
   return 0;
 }
 
-int tl_rope_split(const float* qkv, const int* row_pos, const float* inv_freq, int n, int nq,
-                  int nkv, int d, void* q, void* k, void* v, void* vt, int vt_cols, const int* row_seq,
-                  const int* tile_off, const int* n_cached, int out_dt, hipStream_t st) {
+// inv_freq [rotary_dim / 2], rotary_dim (even, 0..d; 0: no rotation), interleaved: see `Rotation`
+int tl_rope_split(const float* qkv, const int* row_pos, const float* inv_freq, int rotary_dim, int interleaved,
+                  int n, int nq, int nkv, int d, void* q, void* k, void* v, void* vt, int vt_cols,
+                  const int* row_seq, const int* tile_off, const int* n_cached, int out_dt, hipStream_t st) {
   TL_REQUIRE(n >= 0 && nq > 0 && nkv >= 0 && d > 0 && d % 2 == 0,
              "rope_split: bad sizes n=%d nq=%d nkv=%d d=%d (d must be even)", n, nq, nkv, d);
   TL_REQUIRE(d <= 2 * ROPE_MAX_HALF, "rope_split: head size %d is not served (at most %d)", d, 2 * ROPE_MAX_HALF);
+  TL_REQUIRE(rotary_dim >= 0 && rotary_dim <= d && rotary_dim % 2 == 0 && (rotary_dim == 0 || inv_freq != nullptr),
+             "rope_split: %d rotated channels of a head of %d (even, at most the head, with their frequencies)",
+             rotary_dim, d);
+  const Rotation rot{inv_freq, rotary_dim, interleaved != 0};
   if (n == 0) return 0;
   if (out_dt == DT_F32)
-    rope_split_kernel<float><<<n, 256, 0, st>>>(qkv, row_pos, inv_freq, nq, nkv, d, (float*)q,
+    rope_split_kernel<float><<<n, 256, 0, st>>>(qkv, row_pos, rot, nq, nkv, d, (float*)q,
                                                  (float*)k, (float*)v, (float*)vt, vt_cols, row_seq,
                                                  tile_off, n_cached);
   else if (out_dt == DT_BF16)
-    rope_split_kernel<bf16><<<n, 256, 0, st>>>(qkv, row_pos, inv_freq, nq, nkv, d, (bf16*)q,
+    rope_split_kernel<bf16><<<n, 256, 0, st>>>(qkv, row_pos, rot, nq, nkv, d, (bf16*)q,
                                                 (bf16*)k, (bf16*)v, (bf16*)vt, vt_cols, row_seq, tile_off,
                                                 n_cached);
   else
@@ -603,22 +612,26 @@ int tl_kv_commit_tiles(const void* k, const void* vt, int vt_cols, int dt, const
 }
 
 // n_parts >= 1: qkv is [n_parts][n][(nq + 2 nkv) d], summed on the way in
-int tl_rope_commit(const float* qkv, int n_parts, const int* row_pos, const float* inv_freq, const int* table,
-                   int table_stride, int ring_pages, int n, int nq, int nkv, int d, void* q, void* pages,
-                   int dt, hipStream_t st) {
+int tl_rope_commit(const float* qkv, int n_parts, const int* row_pos, const float* inv_freq, int rotary_dim,
+                   int interleaved, const int* table, int table_stride, int ring_pages, int n, int nq, int nkv,
+                   int d, void* q, void* pages, int dt, hipStream_t st) {
   TL_REQUIRE(n >= 0 && nq > 0 && nkv > 0 && d > 0 && d % 2 == 0 && ring_pages > 0 && table_stride > 0,
              "rope_commit: bad sizes n=%d nq=%d nkv=%d d=%d ring_pages=%d table_stride=%d", n, nq, nkv, d,
              ring_pages, table_stride);
   TL_REQUIRE(d <= 2 * ROPE_MAX_HALF, "rope_commit: head size %d is not served (at most %d)", d, 2 * ROPE_MAX_HALF);
   TL_REQUIRE(n_parts >= 1, "rope_commit: n_parts=%d", n_parts);
+  TL_REQUIRE(rotary_dim >= 0 && rotary_dim <= d && rotary_dim % 2 == 0 && (rotary_dim == 0 || inv_freq != nullptr),
+             "rope_commit: %d rotated channels of a head of %d (even, at most the head, with their frequencies)",
+             rotary_dim, d);
+  const Rotation rot{inv_freq, rotary_dim, interleaved != 0};
   if (n == 0) return 0;
   const size_t stride = (size_t)n * (nq + 2 * nkv) * d;
   const dim3 grid(n, n >= 128 ? 1 : (n >= 32 ? 4 : 8));       // few rows: cut the heads over more workgroups
   if (dt == DT_F32)
-    rope_commit_kernel<float><<<grid, 256, 0, st>>>(qkv, n_parts, stride, row_pos, inv_freq, table, table_stride,
+    rope_commit_kernel<float><<<grid, 256, 0, st>>>(qkv, n_parts, stride, row_pos, rot, table, table_stride,
                                                   ring_pages, nq, nkv, d, (float*)q, (float*)pages);
   else if (dt == DT_BF16)
-    rope_commit_kernel<bf16><<<grid, 256, 0, st>>>(qkv, n_parts, stride, row_pos, inv_freq, table, table_stride,
+    rope_commit_kernel<bf16><<<grid, 256, 0, st>>>(qkv, n_parts, stride, row_pos, rot, table, table_stride,
                                                  ring_pages, nq, nkv, d, (bf16*)q, (bf16*)pages);
   else
     TL_REQUIRE(false, "rope_commit: unknown dtype code %d", dt);

@@ -400,9 +400,10 @@ static int launch_rows(const bf16* A, const bf16* W, float* C, int M, int N, int
 // The skinny product (16 channels a workgroup, 8 waves over K, up to 16 rows) for the
 // fused projection of a step with one token a sequence, with what follows it done on
 // the sums while they are in LDS: rotation of q and k by the position, q to its buffer,
-// k and v into the sequence's page (v transposed).  To have both halves of a rotated
-// pair, a tile of a q or k head takes channels 8t..8t+7 and d/2+8t..d/2+8t+7; a tile of
-// a v head takes 16 in a row.  With kv_half the tiles of k and v heads are half as large
+// k and v into the sequence's page (v transposed).  To have both channels of a rotated
+// pair, a tile of a q or k head takes the first channels of pairs 8t..8t+7 and then their
+// second channels (`pair_channels`: with all of a head rotated in halves these are 8t..8t+7
+// and d/2+8t..d/2+8t+7); a tile of a v head takes 16 in a row.  With kv_half the tiles of k and v heads are half as large
 // (4 pairs, or 8 channels, in the first 8 rows of the MFMA tile; the other rows load
 // nothing): the launcher asks for that when it spreads the workgroups more evenly over
 // the compute units (7B: 384 tiles are one and a half a unit, 256 + 256 are two for all).
@@ -415,7 +416,7 @@ constexpr int QKV_WAVES = 8;
 template <bool TILED>
 __global__ void __launch_bounds__(QKV_WAVES * 64)
 gemm_qkv_rope_commit_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, int M, int K,
-                            const int* __restrict__ row_pos, const float* __restrict__ inv_freq,
+                            const int* __restrict__ row_pos, Rotation rot,
                             const int* __restrict__ table, int table_stride, int ring_pages, int nq,
                             int nkv, int d, bf16* __restrict__ q, bf16* __restrict__ pages, NormSplit ns,
                             int kv_half) {
@@ -424,7 +425,6 @@ gemm_qkv_rope_commit_kernel(const bf16* __restrict__ A, const bf16* __restrict__
   __shared__ float rs[16];
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
   const int li = lane % 16, kg = lane / 16;
-  const int half = d / 2;
   // which head, which tile of it, and how many pairs (or, for v, channels / 2) the tile holds
   int head, tt, np = 8;
   {
@@ -441,7 +441,12 @@ gemm_qkv_rope_commit_kernel(const bf16* __restrict__ A, const bf16* __restrict__
   }
   const bool rotated = head < nq + nkv;
   const bool loads = li < 2 * np;               // rows of the MFMA tile that hold a channel
-  const int ch = rotated ? (li < np ? np * tt + li : half + np * tt + li - np) : 2 * np * tt + li;
+  int ch = 2 * np * tt + li;
+  if (rotated) {
+    int ca, cb;
+    pair_channels(np * tt + (li < np ? li : li - np), rot.rotary_dim, rot.interleaved, ca, cb);
+    ch = li < np ? ca : cb;
+  }
   const bf16* wrow;
   if constexpr (TILED) {
     // the tile that holds this (half) tile's channels, and this lane's row in it
@@ -480,7 +485,8 @@ gemm_qkv_rope_commit_kernel(const bf16* __restrict__ A, const bf16* __restrict__
   if (s < s1) load_step(s, w0, a0);
   if (rotated && tid < 128) {                  // while the first loads are under way
     const int m = tid / 8, j = tid % 8;
-    if (m < M && j < np) sincosf(inv_freq[np * tt + j] * (float)row_pos[m], &sn[m][j], &cs[m][j]);
+    if (m < M && j < np && 2 * (np * tt + j) < rot.rotary_dim)
+      sincosf(rot.inv_freq[np * tt + j] * (float)row_pos[m], &sn[m][j], &cs[m][j]);
   }
   const bool scaled = ns.ssq_in != nullptr;
   RowFactors rf;
@@ -508,9 +514,11 @@ gemm_qkv_rope_commit_kernel(const bf16* __restrict__ A, const bf16* __restrict__
     if (tid < 128) {
       const int m = tid / 8, j = tid % 8;
       if (m < M && j < np) {
-        float ra, rb;
-        rotate_pair(total(j, m), total(j + np, m), cs[m][j], sn[m][j], ra, rb);
         const int i = np * tt + j;
+        float ra = total(j, m), rb = total(j + np, m);
+        if (2 * i < rot.rotary_dim) rotate_pair(ra, rb, cs[m][j], sn[m][j], ra, rb);
+        int ia, ib;
+        pair_channels(i, rot.rotary_dim, rot.interleaved, ia, ib);
         bf16* dst;
         if (head < nq) {
           dst = q + ((size_t)m * nq + head) * d;
@@ -519,8 +527,8 @@ gemm_qkv_rope_commit_kernel(const bf16* __restrict__ A, const bf16* __restrict__
           const int page = table[(size_t)m * table_stride + (p / PAGE) % ring_pages];
           dst = pages + (size_t)page * page_elems + ((size_t)(head - nq) * PAGE + p % PAGE) * d;
         }
-        dst[i] = (bf16)ra;
-        dst[i + half] = (bf16)rb;
+        dst[ia] = (bf16)ra;
+        dst[ib] = (bf16)rb;
       }
     }
   } else if (tid < 256) {
@@ -1046,7 +1054,8 @@ extern "C" int tl_gemm_mid_bf16(const void* A, const void* W, void* C, int M, in
 // Wt (or null): the tiled copy of W with the rows of `tl_qkv_tile_rows`, read instead of W
 // when K % 64 == 0.
 extern "C" int tl_gemm_qkv_rope_commit(const void* A, const void* W, const void* Wt, int M, int K, const int* row_pos,
-                                       const float* inv_freq, const int* table, int table_stride,
+                                       const float* inv_freq, int rotary_dim, int interleaved,
+                                       const int* table, int table_stride,
                                        int ring_pages, int nq, int nkv, int d, void* q, void* pages,
                                        const float* ssq_in, int n_part, float inv_h, float eps,
                                        int kv_half, hipStream_t st) {
@@ -1058,6 +1067,10 @@ extern "C" int tl_gemm_qkv_rope_commit(const void* A, const void* W, const void*
              "table_stride=%d", ring_pages, table_stride);
   TL_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "qkv_rope_commit: operands must be 16-byte aligned");
   TL_REQUIRE(ssq_in == nullptr || n_part > 0, "qkv_rope_commit: %d partial sums of squares", n_part);
+  TL_REQUIRE(rotary_dim >= 0 && rotary_dim <= d && rotary_dim % 2 == 0 && (rotary_dim == 0 || inv_freq != nullptr),
+             "qkv_rope_commit: %d rotated channels of a head of %d (even, at most the head, with their "
+             "frequencies)", rotary_dim, d);
+  const Rotation rot{inv_freq, rotary_dim, interleaved != 0};
   if (M == 0) return 0;
   const int full = (nq + 2 * nkv) * (d / 16), mixed = nq * (d / 16) + 2 * nkv * (d / 8);
   if (kv_half < 0) {
@@ -1078,11 +1091,11 @@ extern "C" int tl_gemm_qkv_rope_commit(const void* A, const void* W, const void*
   if (Wt != nullptr && K % 64 == 0) {
     TL_REQUIRE((uintptr_t)Wt % 16 == 0, "qkv_rope_commit: operands must be 16-byte aligned");
     gemm_qkv_rope_commit_kernel<true><<<grid, QKV_WAVES * 64, 0, st>>>(
-        (const bf16*)A, (const bf16*)Wt, M, K, row_pos, inv_freq, table, table_stride, ring_pages, nq, nkv, d,
+        (const bf16*)A, (const bf16*)Wt, M, K, row_pos, rot, table, table_stride, ring_pages, nq, nkv, d,
         (bf16*)q, (bf16*)pages, ns, kv_half);
   } else {
     gemm_qkv_rope_commit_kernel<false><<<grid, QKV_WAVES * 64, 0, st>>>(
-        (const bf16*)A, (const bf16*)W, M, K, row_pos, inv_freq, table, table_stride, ring_pages, nq, nkv, d,
+        (const bf16*)A, (const bf16*)W, M, K, row_pos, rot, table, table_stride, ring_pages, nq, nkv, d,
         (bf16*)q, (bf16*)pages, ns, kv_half);
   }
   TL_LAUNCH_CHECK("gemm_qkv_rope_commit");
@@ -1140,13 +1153,22 @@ extern "C" int tl_tile_weights(const void* W, const int* rows, int N, int K, voi
 }
 
 // The order of W's rows in the tiled copy that tl_gemm_qkv_rope_commit reads: tile t of a q or
-// k head holds channels 8t..8t+7 and d/2+8t..d/2+8t+7, v heads keep theirs.  rows: [(nq + 2 nkv) d], host.
-extern "C" int tl_qkv_tile_rows(int nq, int nkv, int d, int* rows) {
+// k head holds the first channels of pairs 8t..8t+7 and then their second channels (with all of a
+// head rotated in halves: 8t..8t+7 and d/2+8t..d/2+8t+7), v heads keep theirs.
+// rows: [(nq + 2 nkv) d], host.
+extern "C" int tl_qkv_tile_rows(int nq, int nkv, int d, int rotary_dim, int interleaved, int* rows) {
   TL_REQUIRE(nq > 0 && nkv > 0 && d >= 16 && d % 16 == 0, "qkv_tile_rows: bad heads nq=%d nkv=%d d=%d", nq, nkv, d);
+  TL_REQUIRE(rotary_dim >= 0 && rotary_dim <= d && rotary_dim % 2 == 0,
+             "qkv_tile_rows: %d rotated channels of a head of %d (even, at most the head)", rotary_dim, d);
   for (int head = 0; head < nq + 2 * nkv; ++head)
     for (int t = 0; t < d / 16; ++t)
       for (int r = 0; r < 16; ++r) {
-        const int ch = head < nq + nkv ? (r < 8 ? 8 * t + r : d / 2 + 8 * t + r - 8) : 16 * t + r;
+        int ch = 16 * t + r;
+        if (head < nq + nkv) {
+          int ca, cb;
+          pair_channels(8 * t + r % 8, rotary_dim, interleaved != 0, ca, cb);
+          ch = r < 8 ? ca : cb;
+        }
         rows[(head * (d / 16) + t) * 16 + r] = head * d + ch;
       }
   return 0;

@@ -84,10 +84,38 @@ def rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float, out: torch.Tensor) -> 
                             _stream()))
 
 
-def rope_split(qkv: torch.Tensor, row_pos: torch.Tensor, inv_freq: torch.Tensor, nq: int, nkv: int,
+class Rotation:
+    """How q and k are rotated by position: the first `rotary_dim` channels of a head in pairs,
+    pair i by the angle pos * inv_freq[i] (float32 [rotary_dim / 2] on the device); pairs are
+    (i, i + rotary_dim/2), or (2i, 2i+1) when `interleaved`; the channels behind them pass
+    through.  rotary_dim 0 (inv_freq None): nothing is rotated."""
+
+    def __init__(self, inv_freq: Optional[torch.Tensor], rotary_dim: int, interleaved: bool = False):
+        self.inv_freq, self.rotary_dim, self.interleaved = inv_freq, int(rotary_dim), bool(interleaved)
+
+
+NO_ROTATION = Rotation(None, 0)
+
+
+def _rotation(rot, d: int, what: str) -> Rotation:
+    """A `Rotation` checked against the head size `d`.  A bare tensor of d/2 frequencies stands
+    for the rotation of the whole head in halves; None for no rotation."""
+    if rot is None:
+        return NO_ROTATION
+    if isinstance(rot, torch.Tensor):
+        rot = Rotation(rot, d)
+    if rot.rotary_dim % 2 or not (0 <= rot.rotary_dim <= d):
+        raise KernelError(f"{what}: {rot.rotary_dim} rotated channels of a head of {d} (even, at most the head)")
+    if rot.rotary_dim:
+        _req(rot.inv_freq, what + ".inv_freq", torch.float32, (rot.rotary_dim // 2,))
+    return rot
+
+
+def rope_split(qkv: torch.Tensor, row_pos: torch.Tensor, rotation, nq: int, nkv: int,
                d: int, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, vt: Optional[torch.Tensor] = None,
                row_seq=None, tile_off=None, n_cached=None) -> None:
-    """Rotate q and k of the fused projection by their rows' positions and
+    """Rotate q and k of the fused projection by their rows' positions (`rotation`: a
+    `Rotation`, or the d/2 frequencies of a whole head rotated in halves) and
     write q [n,nq,d], k, v [n,nkv,d] (v may be None: the values are taken by
     `v_tiles` then).  With `vt` [nkv, d, cols] the values are
     also written transposed, row n into column tile_off[b] + pos - 64 *
@@ -95,7 +123,7 @@ def rope_split(qkv: torch.Tensor, row_pos: torch.Tensor, inv_freq: torch.Tensor,
     n = qkv.shape[0]
     _req(qkv, "rope.qkv", torch.float32, (n, (nq + 2 * nkv) * d))
     _req(row_pos, "rope.row_pos", torch.int32, (n,))
-    _req(inv_freq, "rope.inv_freq", torch.float32, (d // 2,))
+    rot = _rotation(rotation, d, "rope")
     _req(q, "rope.q", None, (n, nq, d))
     if nkv:
         _req(k, "rope.k", q.dtype, (n, nkv, d))
@@ -110,7 +138,8 @@ def rope_split(qkv: torch.Tensor, row_pos: torch.Tensor, inv_freq: torch.Tensor,
         _req(row_seq, "rope.row_seq", torch.int32, (n,))
         _req(tile_off, "rope.tile_off", torch.int32)
         _req(n_cached, "rope.n_cached", torch.int32, tuple(tile_off.shape))
-    _check(lib().tl_rope_split(_p(qkv), _p(row_pos), _p(inv_freq), n, nq, nkv, d, _p(q), _p(k), _p(v),
+    _check(lib().tl_rope_split(_p(qkv), _p(row_pos), _p(rot.inv_freq), rot.rotary_dim, int(rot.interleaved),
+                               n, nq, nkv, d, _p(q), _p(k), _p(v),
                                _p(vt), cols, _p(row_seq), _p(tile_off), _p(n_cached), _code(q.dtype),
                                _stream()))
 
@@ -294,12 +323,14 @@ def tile_weights(w: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.
     return out
 
 
-def qkv_tile_rows(nq: int, nkv: int, d: int, device) -> torch.Tensor:
+def qkv_tile_rows(nq: int, nkv: int, d: int, device, rotation=None) -> torch.Tensor:
     """The order of the rows of w = q|k|v in the tiled copy that `qkv_rope_commit` reads
-    (a tile of a q or k head holds both halves of 8 rotated pairs)."""
+    (a tile of a q or k head holds both channels of 8 pairs of `rotation`; None: the whole
+    head rotated in halves)."""
     n = (nq + 2 * nkv) * d
     buf = (ctypes.c_int * n)()
-    _check(lib().tl_qkv_tile_rows(int(nq), int(nkv), int(d), buf))
+    rotary_dim, interleaved = (d, False) if rotation is None else (rotation.rotary_dim, rotation.interleaved)
+    _check(lib().tl_qkv_tile_rows(int(nq), int(nkv), int(d), int(rotary_dim), int(interleaved), buf))
     return torch.tensor(list(buf), dtype=torch.int32, device=device)
 
 
@@ -503,16 +534,16 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
         gemm_plain(a, w, out, accumulate)
 
 
-def rope_commit(qkv: torch.Tensor, row_pos, inv_freq, table, ring_pages: int, nq: int, nkv: int, d: int,
+def rope_commit(qkv: torch.Tensor, row_pos, rotation, table, ring_pages: int, nq: int, nkv: int, d: int,
                 q: torch.Tensor, pages: torch.Tensor) -> None:
-    """Single-token steps: rotate q and k, write q [n,nq,d] and put k and v of
-    row n straight into sequence n's page for its position.  qkv may be
+    """Single-token steps: rotate q and k (`rotation`: see `rope_split`), write q [n,nq,d] and
+    put k and v of row n straight into sequence n's page for its position.  qkv may be
     [S, n, width]: partial products that are added up on the way in."""
     n_parts = qkv.shape[0] if qkv.dim() == 3 else 1
     n = qkv.shape[-2]
     _req(qkv, "rope.qkv", torch.float32, ((n_parts,) if qkv.dim() == 3 else ()) + (n, (nq + 2 * nkv) * d))
     _req(row_pos, "rope.row_pos", torch.int32, (n,))
-    _req(inv_freq, "rope.inv_freq", torch.float32, (d // 2,))
+    rot = _rotation(rotation, d, "rope")
     _req(q, "rope.q", pages.dtype, (n, nq, d))
     _req(table, "rope.table", torch.int32)
     _req(pages, "rope.pages")
@@ -520,7 +551,8 @@ def rope_commit(qkv: torch.Tensor, row_pos, inv_freq, table, ring_pages: int, nq
         raise KernelError(f"rope.pages: shape {tuple(pages.shape)}, kernel needs [*, 2, {nkv}, 64, {d}]")
     if table.dim() != 2 or table.shape[0] != n:
         raise KernelError("rope.table: needs one row per sequence")
-    _check(lib().tl_rope_commit(_p(qkv), n_parts, _p(row_pos), _p(inv_freq), _p(table), table.shape[1], ring_pages,
+    _check(lib().tl_rope_commit(_p(qkv), n_parts, _p(row_pos), _p(rot.inv_freq), rot.rotary_dim,
+                                int(rot.interleaved), _p(table), table.shape[1], ring_pages,
                                 n, nq, nkv, d, _p(q), _p(pages), _code(q.dtype), _stream()))
 
 
@@ -529,7 +561,7 @@ def qkv_rope_commit_ok(a: torch.Tensor, w: torch.Tensor, d: int, pages: torch.Te
     return bf16_gemm_ok(a, w) and a.shape[0] <= 16 and d % 16 == 0 and pages.dtype == torch.bfloat16
 
 
-def qkv_rope_commit(a: torch.Tensor, w: torch.Tensor, row_pos, inv_freq, table, ring_pages: int, nq: int,
+def qkv_rope_commit(a: torch.Tensor, w: torch.Tensor, row_pos, rotation, table, ring_pages: int, nq: int,
                     nkv: int, d: int, q: torch.Tensor, pages: torch.Tensor,
                     factor: Optional[RowFactor] = None, kv_half: Optional[bool] = None,
                     tiles: Optional[torch.Tensor] = None) -> None:
@@ -537,13 +569,14 @@ def qkv_rope_commit(a: torch.Tensor, w: torch.Tensor, row_pos, inv_freq, table, 
     the rotation of q and k, q into its buffer and k, v into the pages, in one kernel; the
     same bits as `gemm` and then `rope_commit`.  `factor`: see `gemm_bf16_norm`.  `kv_half`
     (tests): force or forbid the smaller tiles for k and v that the launcher may choose.
-    `tiles`: `tile_weights(w, qkv_tile_rows(nq, nkv, d))`, read instead of w."""
+    `tiles`: `tile_weights(w, qkv_tile_rows(nq, nkv, d, device, rotation))`, read instead of w.
+    `rotation`: see `rope_split`."""
     n, K = a.shape
     _req(a, "qkv_rope_commit.a", torch.bfloat16)
     _req(w, "qkv_rope_commit.w", torch.bfloat16, ((nq + 2 * nkv) * d, K))
     _req_tiles(tiles, (nq + 2 * nkv) * d, K)
     _req(row_pos, "qkv_rope_commit.row_pos", torch.int32, (n,))
-    _req(inv_freq, "qkv_rope_commit.inv_freq", torch.float32, (d // 2,))
+    rot = _rotation(rotation, d, "qkv_rope_commit")
     _req(q, "qkv_rope_commit.q", torch.bfloat16, (n, nq, d))
     _req(table, "qkv_rope_commit.table", torch.int32)
     _req(pages, "qkv_rope_commit.pages", torch.bfloat16)
@@ -557,7 +590,8 @@ def qkv_rope_commit(a: torch.Tensor, w: torch.Tensor, row_pos, inv_freq, table, 
         if factor.ssq.numel() < factor.n_part * 16 or factor.n_part < 1:
             raise KernelError(f"qkv_rope_commit.factor: {factor.ssq.numel()} floats for {factor.n_part} workgroups")
         ssq_in, n_part, inv_h, eps = factor.ssq, factor.n_part, 1.0 / factor.size, factor.eps
-    _check(lib().tl_gemm_qkv_rope_commit(_p(a), _p(w), _p(tiles), n, K, _p(row_pos), _p(inv_freq), _p(table),
+    _check(lib().tl_gemm_qkv_rope_commit(_p(a), _p(w), _p(tiles), n, K, _p(row_pos), _p(rot.inv_freq),
+                                         rot.rotary_dim, int(rot.interleaved), _p(table),
                                          table.shape[1], int(ring_pages), nq, nkv, d, _p(q), _p(pages),
                                          _p(ssq_in), n_part, ctypes.c_float(inv_h), ctypes.c_float(eps),
                                          -1 if kv_half is None else int(kv_half), _stream()))

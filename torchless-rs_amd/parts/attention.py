@@ -8,8 +8,12 @@ to the query at p iff j <= p and, with a window W, j > p - W
 (src/model/models/gpt_oss.rs:168-175; the reference's Mistral path reads the
 window from the file and never applies it).
 
-The three projections are bound under their own names and laid side by side
-at load so that one product serves them.  Rows of a step that bring more
+The three projections are bound under their own names (`names`: the leaf names
+are parameters, and a checkpoint that stores q|k|v as one tensor binds that one)
+and laid side by side at load so that one product serves them.  How q and k
+are rotated is the position part's answer (`Position.rotation`: frequencies, how
+many channels of a head, which pairing; or no rotation at all); the mixer hands
+it to the kernels and knows no formula of it.  Rows of a step that bring more
 than one token attend to the cache for older positions and to the step's own
 keys for the new ones, and the keys are committed afterwards; single-token
 steps commit first and read everything from the cache.
@@ -33,11 +37,20 @@ class AttentionMixer(Mixer):
     closes_stream = True          # its last write to the stream is `Linear.add_into`
     takes_row_factor = True       # its q|k|v product can do the division of the norm before it
 
+    # leaf names of the tensors under `prefix`; "qkv": one tensor [q | k | v] by rows instead of the three
+    NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight", "qkv": None}
+
     def __init__(self, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int,
                  position: PartSpec, window: Optional[int] = None, own_kv: bool = True,
-                 prefix: str = "self_attn."):
+                 prefix: str = "self_attn.", names: Optional[Dict[str, Optional[str]]] = None):
         if n_heads % n_kv_heads:
             raise ValueError(f"attention: {n_heads} heads are not a multiple of {n_kv_heads} KV heads")
+        unknown = set(names or {}) - set(self.NAMES)
+        if unknown:
+            raise ValueError(f"attention: no tensors called {sorted(unknown)}; there are {sorted(self.NAMES)}")
+        self.names = dict(self.NAMES, **(names or {}))
+        if self.names["qkv"] and not own_kv:
+            raise ValueError("attention: a mixer that reads another's keys and values binds q alone, not q|k|v")
         self.H, self.nq, self.nkv, self.d = int(hidden_size), int(n_heads), int(n_kv_heads), int(head_dim)
         self.window = int(window) if window else None
         self.own_kv = bool(own_kv)
@@ -51,28 +64,36 @@ class AttentionMixer(Mixer):
         return KVRequest(self.nkv, self.d, self.window) if self.own_kv else None
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
-        p = self.prefix
-        out = {p + "q_proj.weight": WeightSpec((self.nq * self.d, self.H))}
-        if self.own_kv:
-            out[p + "k_proj.weight"] = WeightSpec((self.nkv * self.d, self.H))
-            out[p + "v_proj.weight"] = WeightSpec((self.nkv * self.d, self.H))
-        out[p + "o_proj.weight"] = WeightSpec((self.H, self.nq * self.d))
+        p, nm = self.prefix, self.names
+        if nm["qkv"]:
+            out = {p + nm["qkv"]: WeightSpec(((self.nq + 2 * self.nkv) * self.d, self.H))}
+        else:
+            out = {p + nm["q"]: WeightSpec((self.nq * self.d, self.H))}
+            if self.own_kv:
+                out[p + nm["k"]] = WeightSpec((self.nkv * self.d, self.H))
+                out[p + nm["v"]] = WeightSpec((self.nkv * self.d, self.H))
+        out[p + nm["o"]] = WeightSpec((self.H, self.nq * self.d))
         return out
 
     def load(self, tensors, compute_dtype) -> None:
-        p = self.prefix
-        ws = [tensors[p + "q_proj.weight"]]
-        if self.own_kv:
-            ws += [tensors[p + "k_proj.weight"], tensors[p + "v_proj.weight"]]
-        if len({w.dtype for w in ws}) > 1:
-            ws = [w.to(torch.float32) for w in ws]
-        fused = torch.cat(ws, dim=0)
-        # single-token steps stream q|k|v and o from tiled copies; the fused q|k|v kernel has its own order of rows
+        p, nm = self.prefix, self.names
+        if nm["qkv"]:
+            fused = tensors[p + nm["qkv"]]
+        else:
+            ws = [tensors[p + nm["q"]]]
+            if self.own_kv:
+                ws += [tensors[p + nm["k"]], tensors[p + nm["v"]]]
+            if len({w.dtype for w in ws}) > 1:
+                ws = [w.to(torch.float32) for w in ws]
+            fused = torch.cat(ws, dim=0)
+        # single-token steps stream q|k|v and o from tiled copies; the fused q|k|v kernel has its own
+        # order of rows, which follows the pairs of the rotation
         rows = None
         if self.own_kv and self.d % 16 == 0 and fused.is_cuda and fused.dtype == torch.bfloat16:
-            rows = ops.qkv_tile_rows(self.nq, self.nkv, self.d, fused.device)
+            rows = ops.qkv_tile_rows(self.nq, self.nkv, self.d, fused.device,
+                                     self.position.rotation(fused.device) or ops.NO_ROTATION)
         self.qkv = Linear(fused, tiled=True, tile_rows=rows)
-        self.o = Linear(tensors[p + "o_proj.weight"], tiled=True)
+        self.o = Linear(tensors[p + nm["o"]], tiled=True)
 
     def forward(self, ctx, run, y: torch.Tensor, x: torch.Tensor) -> None:
         n, nq, nkv, d = y.shape[0], self.nq, self.nkv, self.d
@@ -80,7 +101,7 @@ class AttentionMixer(Mixer):
         group = run.kv_group
         pages = group.storage[run.kv_layer]
         table = ctx.tables[run.kv_group_index]
-        inv_freq = self.position.inv_freq(y.device)
+        rotation = self.position.rotation(y.device) or ops.NO_ROTATION
         q = ws.get("attn_q", (n, nq, d), ctx.dtype)
         out = ws.get("attn_out", (n, nq, d), ctx.dtype)
         fused = (self.own_kv and ctx.all_single and not run.kv_read_later
@@ -89,7 +110,7 @@ class AttentionMixer(Mixer):
         if self.own_kv and ctx.all_single and not run.kv_read_later:
             # one token a sequence: k and v go straight into the pages, then everything is read there
             if fused:
-                ops.qkv_rope_commit(y, self.qkv.weight, ctx.row_pos, inv_freq, table, group.ring_pages,
+                ops.qkv_rope_commit(y, self.qkv.weight, ctx.row_pos, rotation, table, group.ring_pages,
                                     nq, nkv, d, q, pages, factor=factor,     # product, rotation and commit in one
                                     tiles=self.qkv.own_tiles)
             else:
@@ -97,7 +118,7 @@ class AttentionMixer(Mixer):
                 if qkv is None:
                     qkv = ws.get("attn_qkv", (n, (nq + 2 * nkv) * d), torch.float32)
                     self.qkv(y, qkv)
-                ops.rope_commit(qkv, ctx.row_pos, inv_freq, table, group.ring_pages, nq, nkv, d, q, pages)
+                ops.rope_commit(qkv, ctx.row_pos, rotation, table, group.ring_pages, nq, nkv, d, q, pages)
             ops.attention(q, None, None, pages, table, group.ring_pages, ctx, ctx.len_after,
                           self.window, self.scale, out)
             self.o.add_into(out.view(n, nq * d), x, ctx, "attn_o_parts")
@@ -116,18 +137,18 @@ class AttentionMixer(Mixer):
                 # the matrix cores read values along the keys: only the transposed copy is made, by tiles
                 v = None
                 vt = ws.get("attn_vt" + tag, (nkv, d, ctx.host["aligned_cols"]), ctx.dtype)
-                ops.rope_split(qkv, ctx.row_pos, inv_freq, nq, nkv, d, q, k, None)
+                ops.rope_split(qkv, ctx.row_pos, rotation, nq, nkv, d, q, k, None)
                 ops.v_tiles(qkv, nq, nkv, d, vt, ctx.cu_seqlens, ctx.tile_off, ctx.len_before, ctx.len_after)
             else:
                 vt = None
                 v = ws.get("attn_v" + tag, (n, nkv, d), ctx.dtype)
-                ops.rope_split(qkv, ctx.row_pos, inv_freq, nq, nkv, d, q, k, v)
+                ops.rope_split(qkv, ctx.row_pos, rotation, nq, nkv, d, q, k, v)
             if run.kv_read_later:
                 ctx.host[f"kv_new_{run.index}"] = (k, v, vt)
         else:
             qf = ws.get("attn_qkv", (n, nq * d), torch.float32)
             self.qkv(y, qf)
-            ops.rope_split(qf, ctx.row_pos, inv_freq, nq, 0, d, q, None, None)
+            ops.rope_split(qf, ctx.row_pos, rotation, nq, 0, d, q, None, None)
             k, v, vt = ctx.host[f"kv_new_{run.kv_source}"]
         if ctx.all_single and not self.own_kv:
             ops.attention(q, None, None, pages, table, group.ring_pages, ctx, ctx.len_after,

@@ -121,14 +121,35 @@ class Part:
         pass
 
 
+@dataclass(frozen=True)
+class RmsForm:
+    """A norm of the form y = x * weight / sqrt(mean(x^2) + eps) over `size` channels."""
+    weight: torch.Tensor          # float32 [size]
+    size: int
+    eps: float
+
+
 class Norm(Part):
     def forward(self, ctx: "StepContext", x: torch.Tensor, out: torch.Tensor) -> None:
         """x: float32 [n, H] -> out [n, H] in the compute dtype."""
         raise NotImplementedError
 
+    def rms_form(self) -> Optional[RmsForm]:
+        """If the norm has the form of `RmsForm`, its terms: the products around it may then do
+        its two halves (the sums of squares where the stream is completed, the factor per row
+        on the results of the product that reads it).  None: the norm always runs by itself."""
+        return None
+
 
 class Position(Part):
-    pass
+    """A position encoding, as the attention mixer asks for it: how q and k are rotated."""
+
+    def rotation(self, device):
+        """An `ops.Rotation` (frequencies of the rotated pairs on `device`, how many of a head's
+        channels are rotated, and whether pairs are halves apart or interleaved), or None if
+        queries and keys are used as they are.  Keys enter the cache after the rotation, so
+        any encoding that transforms a key by its own position alone fits this."""
+        return None
 
 
 class Mixer(Part):

@@ -42,14 +42,14 @@ class PreNormBlock(Part):
     def entry_norm(self):
         """The norm that reads the stream first, if the part behind it can take a norm cut in
         two (the block before this one may then do the norm's first half)."""
-        ok = getattr(self.mixer_norm, "splits", False) and getattr(self.mixer, "takes_row_factor", False)
+        ok = self.mixer_norm.rms_form() is not None and getattr(self.mixer, "takes_row_factor", False)
         return self.mixer_norm if ok else None
 
     def forward(self, ctx, run, x: torch.Tensor, norm_after=None) -> None:
         """`norm_after`: the `entry_norm` of the block that runs next, if it has one."""
         y = ctx.workspace.get("block_y", tuple(x.shape), ctx.dtype)
         y1 = self._norm(self.mixer_norm, ctx, x, y)
-        if (getattr(self.ffn_norm, "splits", False) and getattr(self.ffn, "takes_row_factor", False)
+        if (self.ffn_norm.rms_form() is not None and getattr(self.ffn, "takes_row_factor", False)
                 and getattr(self.mixer, "closes_stream", False)):
             ctx.norm_ahead = self.ffn_norm
         self.mixer.forward(ctx, run, y1, x)

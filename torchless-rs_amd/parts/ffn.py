@@ -1,10 +1,11 @@
 """SwiGLU feed-forward: down( silu(gate y) * (up y) ), silu(g) = g / (1 + e^-g)
 (src/model/modules/mlp.rs:23-45, src/kernels/mod.rs:546-548 of the reference).
-gate and up are bound under their own names and laid side by side at load so
-that one product serves both."""
+gate and up are bound under their own names (`names`: the leaf names are
+parameters, and a checkpoint that stores gate|up as one tensor binds that one)
+and laid side by side at load so that one product serves both."""
 from __future__ import annotations
 
-from typing import Dict
+from typing import Dict, Optional
 
 import torch
 
@@ -19,22 +20,35 @@ class SwiGLU(FeedForward):
     closes_stream = True          # its last write to the stream is `Linear.add_into`
     takes_row_factor = True       # its gate|up product can do the division of the norm before it
 
-    def __init__(self, hidden_size: int, intermediate_size: int, prefix: str = "mlp."):
+    # leaf names of the tensors under `prefix`; "gate_up": one tensor [gate | up] by rows instead of the two
+    NAMES = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight", "gate_up": None}
+
+    def __init__(self, hidden_size: int, intermediate_size: int, prefix: str = "mlp.",
+                 names: Optional[Dict[str, Optional[str]]] = None):
         self.H = int(hidden_size)
         self.I = int(intermediate_size)
         self.prefix = prefix
+        unknown = set(names or {}) - set(self.NAMES)
+        if unknown:
+            raise ValueError(f"swiglu: no tensors called {sorted(unknown)}; there are {sorted(self.NAMES)}")
+        self.names = dict(self.NAMES, **(names or {}))
         self.gate_up = None
         self.down = None
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
-        p = self.prefix
-        return {p + "gate_proj.weight": WeightSpec((self.I, self.H)),
-                p + "up_proj.weight": WeightSpec((self.I, self.H)),
-                p + "down_proj.weight": WeightSpec((self.H, self.I))}
+        p, nm = self.prefix, self.names
+        if nm["gate_up"]:
+            return {p + nm["gate_up"]: WeightSpec((2 * self.I, self.H)), p + nm["down"]: WeightSpec((self.H, self.I))}
+        return {p + nm["gate"]: WeightSpec((self.I, self.H)),
+                p + nm["up"]: WeightSpec((self.I, self.H)),
+                p + nm["down"]: WeightSpec((self.H, self.I))}
 
     def load(self, tensors, compute_dtype) -> None:
-        p = self.prefix
-        g, u = tensors[p + "gate_proj.weight"], tensors[p + "up_proj.weight"]
+        p, nm = self.prefix, self.names
+        if nm["gate_up"]:
+            g, u = tensors[p + nm["gate_up"]][:self.I], tensors[p + nm["gate_up"]][self.I:]
+        else:
+            g, u = tensors[p + nm["gate"]], tensors[p + nm["up"]]
         if g.dtype != u.dtype:
             g, u = g.to(torch.float32), u.to(torch.float32)
         # bfloat16 on the matrix cores: gate and up rows interleaved so that the product's
@@ -42,7 +56,7 @@ class SwiGLU(FeedForward):
         self.paired = (compute_dtype == torch.bfloat16 and g.dtype == torch.bfloat16 and self.I % 32 == 0
                        and self.H % 8 == 0)
         self.gate_up = Linear(interleave_pairs(g, u) if self.paired else torch.cat([g, u], dim=0))
-        self.down = Linear(tensors[p + "down_proj.weight"], tiled=True)
+        self.down = Linear(tensors[p + nm["down"]], tiled=True)
 
     def forward(self, ctx, y: torch.Tensor, x: torch.Tensor) -> None:
         n = y.shape[0]

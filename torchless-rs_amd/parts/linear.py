@@ -80,14 +80,15 @@ class Linear:
         from .base import flush_pending
         flush_pending(ctx, x)
         norm = ctx.norm_ahead
-        if (norm is not None and ops.norm_split_ok(a, self.weight) and norm.size == self.out_features
-                and norm.weight is not None and norm.weight.dtype == torch.float32):
+        form = norm.rms_form() if norm is not None and ops.norm_split_ok(a, self.weight) else None
+        if (form is not None and form.size == self.out_features and form.weight is not None
+                and form.weight.dtype == torch.float32):
             # the next norm's first half rides on this product
             xt = ctx.workspace.get("prenormed_y", (a.shape[0], self.out_features), torch.bfloat16)
             ssq = ctx.workspace.get(name + "_ssq", (16, -(-self.out_features // 16)), torch.float32)
-            groups = ops.gemm_bf16_norm(a, self.weight, x, accumulate=True, norm_weight=norm.weight, xt=xt,
+            groups = ops.gemm_bf16_norm(a, self.weight, x, accumulate=True, norm_weight=form.weight, xt=xt,
                                         ssq_out=ssq, tiles=self.tiles)
-            ctx.prenormed = (norm, xt, ops.RowFactor(ssq, groups, norm.size, norm.eps))
+            ctx.prenormed = (norm, xt, ops.RowFactor(ssq, groups, form.size, form.eps))
             return
         parts = self.partial(a, ctx, name)
         if parts is None:

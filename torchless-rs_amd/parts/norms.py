@@ -8,13 +8,12 @@ import torch
 
 from ..kernels import ops
 from ..weights.binding import WeightSpec
-from .base import Norm, register_part
+from .base import Norm, RmsForm, register_part
 
 
 class RMSNorm(Norm):
     graph_safe = True
     takes_pending = True        # adds partial products left in ctx.pending while it reads the stream
-    splits = True               # a product before it may do its sums, a product after it its division
 
     def __init__(self, size: int, eps: float):
         self.size = int(size)
@@ -26,6 +25,9 @@ class RMSNorm(Norm):
 
     def load(self, tensors, compute_dtype) -> None:
         self.weight = tensors["weight"].to(torch.float32).contiguous()
+
+    def rms_form(self) -> RmsForm:
+        return RmsForm(self.weight, self.size, self.eps)
 
     def forward(self, ctx, x: torch.Tensor, out: torch.Tensor) -> None:
         """Partial products waiting in `ctx.pending` are added to x on the way."""
