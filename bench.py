@@ -50,6 +50,10 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64")
     ap.add_argument("--no-tiled-copies", action="store_true",
                     help="keep no second copies of q|k|v, o and down in the layout that single-token steps stream")
+    ap.add_argument("--workload", choices=["baseline"], default=None,
+                    help="also run the baseline's configurations as it words them (unequal prompt lengths drawn "
+                         "from a seed, 256/128/128 new tokens, temperature 0.7 for the NeMo shape) through the "
+                         "generation loop, and add their figures under 'workloads'")
     ap.add_argument("--only", choices=["prefill", "decode"], default=None,
                     help="measure one phase only and print its line to stderr (for profiling)")
     args = ap.parse_args()
@@ -60,6 +64,7 @@ def main() -> int:
     import torch
     from torchless_rs_amd import SamplingConfig, config_from_dict
     from torchless_rs_amd.engine import Engine, SeqInput, model_from_tensors
+    from torchless_rs_amd.engine.generate import BatchRun
     from torchless_rs_amd.models import model_spec_for
     from torchless_rs_amd.sampling.sampler import Sampler
     from torchless_rs_amd.weights import random_tensors
@@ -91,7 +96,7 @@ def main() -> int:
         """Prefill `batch` prompts of `context - steps - warmup` tokens, then time `steps` decode
         steps (model step + greedy sampling)."""
         held = min(context, W) if W else context
-        eng = engine or Engine(model, max_tokens=batch * (-(-held // 64) * 64 + 64), max_slots=batch)
+        eng = engine or Engine(model, max_tokens=batch * (-(-held // 64) * 64 + 64), max_slots=batch, freeze_gc=True)
         plen = max(1, context - steps - warmup - 1)
         slots = [eng.alloc() for _ in range(batch)]
         chunk = 2048
@@ -101,32 +106,67 @@ def main() -> int:
                 part = ids[c0:c0 + chunk]
                 last = c0 + chunk >= plen
                 lg = eng.step([SeqInput(s, part, [len(part) - 1] if last else [])])
+        # every sequence goes on with the same first token; from here the steps are the generation
+        # loop's own (`BatchRun.advance`: the next step is launched with the drawn tokens still on
+        # the device, then the host reads the tokens of the step before)
         first = sampler.sample(lg, [0], [0]) * batch
         lg = eng.step([SeqInput(s, [t], [0]) for s, t in zip(slots, first)])
-        drawn = sampler.draw(lg, list(range(batch)), [0] * batch)
-        entries = [SeqInput(s, [0], [0]) for s in slots]
-
-        def one():
-            # as the generation loop runs: the next step is launched with the drawn tokens still on
-            # the device, then the host reads the tokens of the step before
-            nonlocal drawn
-            lg = eng.step(entries, device_tokens=drawn.device)
-            ahead = sampler.draw(lg, list(range(batch)), [0] * batch)
-            drawn.tokens()
-            drawn = ahead
-
+        run = BatchRun(eng, sampler, accept=lambda i, t: False, max_tokens=1 << 30, run_ahead=True)
+        run.resume(list(range(batch)), lg, slots=slots)
         for _ in range(warmup):
-            one()
+            run.advance()
         torch.cuda.synchronize()
         t = time.perf_counter()
         for _ in range(steps):
-            one()
+            run.advance()
         torch.cuda.synchronize()
         dt = time.perf_counter() - t
         ctx_mid = plen + warmup + steps // 2
-        for s in slots:
-            eng.free(s)
+        run.release()
+        if engine is None:
+            eng.close()
         return dt / steps, ctx_mid
+
+    def run_workload(mdl, mcfg, n_layers, batch, lo, hi, new_tokens, temperature, seed):
+        """`batch` requests with prompt lengths uniform in [lo, hi] and `new_tokens` new tokens each,
+        through `generate_until_eos` as a user would call it: prompts in one step, then one token a
+        step.  The prefill ends and decoding begins when the host holds the first token."""
+        from torchless_rs_amd import generate_until_eos
+        g = torch.Generator().manual_seed(seed)
+        lens = torch.randint(lo, hi + 1, (batch,), generator=g).tolist()
+        prompts = [torch.randint(0, mcfg.vocab_size, (n,), generator=g).tolist() for n in lens]
+        win = mcfg.sliding_window
+        held = [min(n + new_tokens, win) if win else n + new_tokens for n in lens]
+        eng = Engine(mdl, max_tokens=sum(-(-h // 64) * 64 + 64 for h in held), max_slots=batch, freeze_gc=True)
+        scfg = SamplingConfig(temperature=temperature, seed=seed) if temperature > 0 else SamplingConfig.greedy()
+        stamps = []
+
+        def on_token(i, t):
+            if not stamps:
+                torch.cuda.synchronize()
+                stamps.append(time.perf_counter())
+
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        out = generate_until_eos(eng, prompts, scfg, max_tokens=new_tokens, on_token=on_token)
+        torch.cuda.synchronize()
+        t2 = time.perf_counter()
+        eng.close()
+        assert all(len(r.tokens) == new_tokens for r in out)
+        t_pre, t_dec = stamps[0] - t0, t2 - stamps[0]
+        per_l = ((mcfg.num_attention_heads + 2 * mcfg.num_key_value_heads) * mcfg.head_dim * mcfg.hidden_size
+                 + mcfg.hidden_size * mcfg.num_attention_heads * mcfg.head_dim
+                 + 3 * mcfg.intermediate_size * mcfg.hidden_size)
+        w_bytes = 2 * (n_layers * per_l + mcfg.vocab_size * mcfg.hidden_size)
+        kv_tok = 2 * mcfg.num_key_value_heads * mcfg.head_dim * 2 * n_layers
+        steps = new_tokens - 1                           # the first token comes out of the prompts' step
+        ctx = [n + new_tokens / 2 for n in lens]
+        step_bytes = w_bytes + sum((min(c, win) if win else c) for c in ctx) * kv_tok
+        gbs = step_bytes * steps / t_dec / 1e9
+        return {"batch": batch, "prompt_tokens": sum(lens), "new_tokens": new_tokens, "temperature": temperature,
+                "prefill_tok_s": round(sum(lens) / t_pre, 1), "prefill_ms": round(t_pre * 1e3, 1),
+                "decode_tok_s": round(batch * steps / t_dec, 1), "decode_ms_per_step": round(t_dec / steps * 1e3, 3),
+                "roofline_frac": round(gbs / HBM_PEAK_GBS, 4), "achieved_GBs": round(gbs, 1)}
 
     if args.only == "decode":
         sec, _ = run_decode(args.batch, args.context, args.steps, args.warmup)
@@ -136,7 +176,7 @@ def main() -> int:
 
     # prefill of one prompt
     T = args.prefill_tokens
-    eng = Engine(model, max_tokens=T + 64, max_slots=1)
+    eng = Engine(model, max_tokens=T + 64, max_slots=1, freeze_gc=True)
     ids = torch.randint(0, V, (T,), generator=gen).tolist()
     pre_ms = []
     for it in range(2):
@@ -147,7 +187,7 @@ def main() -> int:
         torch.cuda.synchronize()
         pre_ms.append((time.perf_counter() - t) * 1e3)
         eng.free(s)
-    del eng
+    eng.close()
     pre = min(pre_ms)
     attn_flops = sum(4 * nq * d * min(p + 1, W or (p + 1)) for p in range(T)) * L
     pre_flops = 2 * T * (L * per_layer) + 2 * V * H + attn_flops
@@ -170,6 +210,26 @@ def main() -> int:
             s_b, _ = run_decode(b, args.context, max(8, args.steps // 2), 2)
             points[f"decode_b{b}"] = round(b / s_b, 1)
             print(f"[bench] decode b{b}: {b / s_b:.1f} tok/s", file=sys.stderr, flush=True)
+
+    workloads = {}
+    if args.workload == "baseline":
+        if args.shape == "7b-v0.1":                     # the model that is loaded: prompts U[128, 2048], 256 new tokens
+            for b in (1, 8, 64):
+                workloads[f"7b-v0.1_b{b}"] = run_workload(model, cfg, L, b, 128, 2048, 256, 0.0, seed=5)
+                print(f"[bench] workload 7b-v0.1 b{b}: {workloads[f'7b-v0.1_b{b}']}", file=sys.stderr, flush=True)
+        del model
+        torch.cuda.empty_cache()
+        for key, b, lo, hi, new, temp, seed in (("7b-v0.3", 8, 1024, 16384, 128, 0.0, 6),
+                                                ("nemo-12b", 16, 256, 8192, 128, 0.7, 7)):
+            wcfg = config_from_dict(dict(SHAPES[key][1], architectures=["MistralForCausalLM"]))
+            wt = random_tensors(model_spec_for(wcfg).weight_specs(), seed=seed, std=0.02, dtype=torch.bfloat16, device=dev)
+            wm = model_from_tensors(wcfg, wt, "bfloat16", dev, tiled_copies=not args.no_tiled_copies)
+            del wt
+            workloads[f"{key}_b{b}"] = run_workload(wm, wcfg, wcfg.num_hidden_layers, b, lo, hi, new, temp, seed)
+            print(f"[bench] workload {key} b{b}: {workloads[f'{key}_b{b}']}", file=sys.stderr, flush=True)
+            del wm
+            torch.cuda.empty_cache()
+        model = None
 
     # what the simplest kernels get here: a plain read of 8 GiB, independent MFMAs on registers
     from torchless_rs_amd.kernels import ops as _ops
@@ -199,6 +259,8 @@ def main() -> int:
         "points": points,
         "ceilings": ceilings,
     }
+    if workloads:
+        out["workloads"] = workloads
     print(json.dumps(out), flush=True)
     return 0
 

@@ -96,53 +96,97 @@ def generate(engine, sampler, prompts: Sequence[Sequence[int]], max_tokens: int,
         return bool(r.finish_reason)
 
     for batch in plan_batches(need, engine.fits, max_batch):
-        slots: Dict[int, int] = {}
+        run = BatchRun(engine, sampler, accept, max_tokens, run_ahead)
         try:
-            _serve_batch(engine, sampler, prompts, batch, slots, results, accept, max_tokens, run_ahead)
+            run.start(batch, [prompts[i] for i in batch], [len(results[i].tokens) for i in batch])
+            while run.advance():
+                pass
         finally:
             # whatever ended the batch (a step that failed, the caller's `on_token`, an interrupt),
             # nothing of it stays held in the engine
-            for i in list(slots):
-                engine.free(slots.pop(i))
+            run.release()
     return results
 
 
-def _serve_batch(engine, sampler, prompts, batch, slots, results, accept, max_tokens, run_ahead) -> None:
-    """One batch from its prompts to its last token.  `slots` (request -> slot) is the caller's: what
-    is still in it when this returns or raises is freed there."""
-    for i in batch:
-        slots[i] = engine.alloc()
-    live = list(batch)
-    logits = engine.step([SeqInput(slots[i], list(prompts[i]), [len(prompts[i]) - 1]) for i in live])
-    if not run_ahead:
-        while True:
-            ids = sampler.sample(logits, live, [len(results[i].tokens) for i in live])
-            nxt, feed = [], {}
-            for i, t in zip(live, ids):
-                if accept(i, t):
-                    engine.free(slots.pop(i))
-                else:
+class BatchRun:
+    """One batch from its prompts to its last token, a step at a time: `start`, then `advance`
+    until it returns False.  `accept(request, token) -> finished` books a token for the caller;
+    `release` frees what is still held (call it in a `finally`).  `generate` is a loop around
+    this, and so is a measurement of decode steps: there is no second decode loop."""
+
+    def __init__(self, engine, sampler, accept: Callable[[int, int], bool], max_tokens: int, run_ahead: bool):
+        self.engine, self.sampler, self.accept = engine, sampler, accept
+        self.max_tokens, self.run_ahead = max_tokens, run_ahead
+        self.slots: Dict[int, int] = {}             # request -> slot, while it is alive
+        self.count: Dict[int, int] = {}             # request -> tokens booked so far
+        self.order: List[int] = []                  # run ahead: requests whose tokens `drawn` holds, row by row
+        self.drawn = None
+        self.logits = None                          # not running ahead: what the last step returned
+        self.live: List[int] = []
+
+    def start(self, requests: Sequence[int], prompts: Sequence[Sequence[int]], booked: Optional[Sequence[int]] = None) -> None:
+        """Take a slot for every request and run all prompts as one step."""
+        for i in requests:
+            self.slots[i] = self.engine.alloc()
+        logits = self.engine.step([SeqInput(self.slots[i], list(p), [len(p) - 1]) for i, p in zip(requests, prompts)])
+        self.resume(requests, logits, booked)
+
+    def resume(self, requests: Sequence[int], logits, booked: Optional[Sequence[int]] = None,
+               slots: Optional[Sequence[int]] = None) -> None:
+        """Go on from `logits`, one row for each request in order, that a caller's own steps
+        produced (its prompts fed in pieces, say); `slots`: the requests' slots, if the caller
+        took them."""
+        if slots is not None:
+            self.slots.update(zip(requests, slots))
+        self.count = {i: (booked[k] if booked is not None else 0) for k, i in enumerate(requests)}
+        self.live = list(requests)
+        if self.run_ahead:
+            self.order = list(requests)
+            self.drawn = self.sampler.draw(logits, self.order, [self.count[i] for i in self.order])
+        else:
+            self.logits = logits
+
+    def _book(self, i: int, t: int) -> None:
+        self.count[i] += 1
+        if self.accept(i, t):
+            self.engine.free(self.slots.pop(i))
+
+    def advance(self) -> bool:
+        """One more step of the batch; False when every request has finished."""
+        engine, slots = self.engine, self.slots
+        if not self.run_ahead:
+            if not self.live:
+                return False
+            ids = self.sampler.sample(self.logits, self.live, [self.count[i] for i in self.live])
+            feed = {}
+            for i, t in zip(self.live, ids):
+                self._book(i, t)
+                if i in slots:
                     feed[i] = [t]
-                    nxt.append(i)
-            live = nxt
-            if not live:
-                return
-            logits = engine.step([SeqInput(slots[i], feed[i], [0]) for i in live])
-    # run ahead: `order` are the requests whose tokens `drawn` holds (row by row); those of
-    # them that are not known to be finished go into the next step at once
-    order = live
-    drawn = sampler.draw(logits, order, [len(results[i].tokens) for i in order])
-    while order:
+            self.live = [i for i in self.live if i in slots]
+            if not self.live:
+                return False
+            self.logits = engine.step([SeqInput(slots[i], feed[i], [0]) for i in self.live])
+            return True
+        # run ahead: those of `order` that are not known to be finished go into the next step at once
+        order, drawn = self.order, self.drawn
+        if not order:
+            return False
         # a request that is alive and whose budget this token does not use up goes on, unless
         # the token is a stop id, which the host does not know yet
-        ahead = [i for i in order if i in slots and len(results[i].tokens) + 1 < max_tokens]
+        ahead = [i for i in order if i in slots and self.count[i] + 1 < self.max_tokens]
         nxt_drawn = None
         if ahead:
             rows = [order.index(i) for i in ahead]
             logits = engine.step([SeqInput(slots[i], [0], [0]) for i in ahead],
                                  device_tokens=drawn.device, token_rows=rows)
-            nxt_drawn = sampler.draw(logits, ahead, [len(results[i].tokens) + 1 for i in ahead])
+            nxt_drawn = self.sampler.draw(logits, ahead, [self.count[i] + 1 for i in ahead])
         for i, t in zip(order, drawn.tokens()):
-            if i in slots and accept(i, t):           # (a request dropped earlier: its row ran for nothing)
-                engine.free(slots.pop(i))
-        order, drawn = ahead, nxt_drawn
+            if i in slots:                            # (a request dropped earlier: its row ran for nothing)
+                self._book(i, t)
+        self.order, self.drawn = ahead, nxt_drawn
+        return bool(ahead)
+
+    def release(self) -> None:
+        for i in list(self.slots):
+            self.engine.free(self.slots.pop(i))
