@@ -114,6 +114,10 @@ def test_values_by_tiles_and_their_commit(ops, dt, window, nq, nkv, d):
     ops.v_tiles(qkv, nq, nkv, d, vt_new, cu, i32(off), i32(cached), i32(after))
     assert torch.equal(vt_old, vt_new)
     assert int((vt_new != 7.0).sum()) >= nkv * d * n - 8                       # (a value may be 7.0 by chance)
+    # rotation and transposition in one launch: the same bits
+    q3, k3, vt3 = torch.full_like(q, float("nan")), torch.full_like(k, float("nan")), torch.full_like(vt_new, 7.0)
+    ops.rope_v_tiles(qkv, row_pos, inv, nq, nkv, d, q3, k3, vt3, cu, i32(off), i32(cached), i32(after))
+    assert torch.equal(q3, q2) and torch.equal(k3, k2) and torch.equal(vt3, vt_new)
     # commit: pages of every sequence, rings for the window
     ring = -(-window // PAGE) if window else 1 << 24
     need = [min(-(-a // PAGE), ring) for a in after]

@@ -143,13 +143,11 @@ __global__ void add_partials_kernel(float* __restrict__ x, const float* __restri
 constexpr int ROPE_MAX_HALF = 128;      // head sizes up to 256
 
 template <typename TO>
-__global__ void rope_split_kernel(const float* __restrict__ qkv, const int* __restrict__ row_pos,
-                                  Rotation rot, int nq, int nkv, int d,
-                                  TO* __restrict__ q, TO* __restrict__ k, TO* __restrict__ v,
-                                  TO* __restrict__ vt, int vt_cols, const int* __restrict__ row_seq,
-                                  const int* __restrict__ tile_off, const int* __restrict__ n_cached) {
-  __shared__ float cs[ROPE_MAX_HALF], sn[ROPE_MAX_HALF];
-  const int n = blockIdx.x;
+__device__ __forceinline__ void rope_split_row(int n, float* cs, float* sn, const float* __restrict__ qkv,
+                                               const int* __restrict__ row_pos, Rotation rot, int nq, int nkv, int d,
+                                               TO* __restrict__ q, TO* __restrict__ k, TO* __restrict__ v,
+                                               TO* __restrict__ vt, int vt_cols, const int* __restrict__ row_seq,
+                                               const int* __restrict__ tile_off, const int* __restrict__ n_cached) {
   const int half = d / 2, rot_pairs = rot.rotary_dim / 2;
   const float pos = (float)row_pos[n];
   for (int i = threadIdx.x; i < rot_pairs; i += blockDim.x) {     // the row's angles, once
@@ -180,6 +178,17 @@ __global__ void rope_split_kernel(const float* __restrict__ qkv, const int* __re
     const int col = tile_off[b] + row_pos[n] - (n_cached[b] / PAGE) * PAGE;
     for (int t = threadIdx.x; t < nkv * d; t += blockDim.x) vt[(size_t)t * vt_cols + col] = from_f32<TO>(vs[t]);
   }
+}
+
+template <typename TO>
+__global__ void rope_split_kernel(const float* __restrict__ qkv, const int* __restrict__ row_pos,
+                                  Rotation rot, int nq, int nkv, int d,
+                                  TO* __restrict__ q, TO* __restrict__ k, TO* __restrict__ v,
+                                  TO* __restrict__ vt, int vt_cols, const int* __restrict__ row_seq,
+                                  const int* __restrict__ tile_off, const int* __restrict__ n_cached) {
+  __shared__ float cs[ROPE_MAX_HALF], sn[ROPE_MAX_HALF];
+  rope_split_row<TO>(blockIdx.x, cs, sn, qkv, row_pos, rot, nq, nkv, d, q, k, v, vt, vt_cols, row_seq, tile_off,
+                     n_cached);
 }
 
 // ---- commit keys and values of this step to the pages -----------------------
@@ -235,16 +244,16 @@ __device__ __forceinline__ ColumnTile column_tile(int col0, int B, const int* ti
 // the transposed values of a step, written in whole lines (a row-by-row kernel writes them
 // two bytes at a time, a line apart).  grid: (columns / 64, kv heads, d / 64 rounded up).
 template <typename TO>
-__global__ void __launch_bounds__(256)
-v_tiles_kernel(const float* __restrict__ qkv, int width, int v_off, int d, TO* __restrict__ vt,
-               int vt_cols, int B, const int* __restrict__ cu_seqlens, const int* __restrict__ tile_off,
-               const int* __restrict__ n_cached, const int* __restrict__ len_after) {
-  __shared__ TO tile[64][PAGE + 2];
-  const int col0 = blockIdx.x * PAGE, kvh = blockIdx.y;
+__device__ __forceinline__ void v_tile(int col_block, int kvh, int d_block, TO (*tile)[PAGE + 2],
+                                       const float* __restrict__ qkv, int width, int v_off, int d,
+                                       TO* __restrict__ vt, int vt_cols, int B, const int* __restrict__ cu_seqlens,
+                                       const int* __restrict__ tile_off, const int* __restrict__ n_cached,
+                                       const int* __restrict__ len_after) {
+  const int col0 = col_block * PAGE;
   const ColumnTile t = column_tile(col0, B, tile_off, n_cached, len_after);
   if (t.lo >= t.hi) return;
   const int row0 = cu_seqlens[t.b] - n_cached[t.b];       // row of position p is row0 + p
-  const int c0 = blockIdx.z * 64, dc = min(64, d - c0);    // this block's 64 of the d values
+  const int c0 = d_block * 64, dc = min(64, d - c0);       // this block's 64 of the d values
   // all loads first (16 a thread), then the stores: one trip to memory
   float tmp[16];
 #pragma unroll
@@ -266,6 +275,40 @@ v_tiles_kernel(const float* __restrict__ qkv, int width, int v_off, int d, TO* _
     const int i = idx / PAGE, r = idx % PAGE, p = t.p0 + r;
     if (i < dc && p >= t.lo && p < t.hi) vt[((size_t)kvh * d + c0 + i) * vt_cols + col0 + r] = tile[i][r];
   }
+}
+
+template <typename TO>
+__global__ void __launch_bounds__(256)
+v_tiles_kernel(const float* __restrict__ qkv, int width, int v_off, int d, TO* __restrict__ vt,
+               int vt_cols, int B, const int* __restrict__ cu_seqlens, const int* __restrict__ tile_off,
+               const int* __restrict__ n_cached, const int* __restrict__ len_after) {
+  __shared__ TO tile[64][PAGE + 2];
+  v_tile<TO>(blockIdx.x, blockIdx.y, blockIdx.z, tile, qkv, width, v_off, d, vt, vt_cols, B, cu_seqlens, tile_off,
+             n_cached, len_after);
+}
+
+// Both of the above in one launch, for a step with several rows a sequence: the first n workgroups
+// rotate a row each (q and k; the values are the tiles' business), the others transpose a tile of
+// values each.  The two read the same buffer and write different ones.
+template <typename TO>
+__global__ void __launch_bounds__(256)
+rope_v_tiles_kernel(const float* __restrict__ qkv, const int* __restrict__ row_pos, Rotation rot, int n, int nq,
+                    int nkv, int d, TO* __restrict__ q, TO* __restrict__ k, TO* __restrict__ vt, int vt_cols, int B,
+                    const int* __restrict__ cu_seqlens, const int* __restrict__ tile_off,
+                    const int* __restrict__ n_cached, const int* __restrict__ len_after) {
+  __shared__ __attribute__((aligned(16))) unsigned char sh[sizeof(TO) * 64 * (PAGE + 2) > 2 * sizeof(float) * ROPE_MAX_HALF
+                                                            ? sizeof(TO) * 64 * (PAGE + 2)
+                                                            : 2 * sizeof(float) * ROPE_MAX_HALF];
+  if ((int)blockIdx.x < n) {
+    float* cs = reinterpret_cast<float*>(sh);
+    rope_split_row<TO>(blockIdx.x, cs, cs + ROPE_MAX_HALF, qkv, row_pos, rot, nq, nkv, d, q, k, (TO*)nullptr,
+                       (TO*)nullptr, 0, nullptr, nullptr, nullptr);
+    return;
+  }
+  const int item = blockIdx.x - n, d_blocks = (d + 63) / 64;
+  const int d_block = item % d_blocks, kvh = (item / d_blocks) % nkv, col_block = item / (d_blocks * nkv);
+  v_tile<TO>(col_block, kvh, d_block, reinterpret_cast<TO(*)[PAGE + 2]>(sh), qkv, (nq + 2 * nkv) * d, (nq + nkv) * d, d,
+             vt, vt_cols, B, cu_seqlens, tile_off, n_cached, len_after);
 }
 
 // Commit of a step whose values lie transposed by tiles: the first blocks put the keys of 8 rows
@@ -608,6 +651,36 @@ int tl_kv_commit_tiles(const void* k, const void* vt, int vt_cols, int dt, const
   else
     TL_REQUIRE(false, "kv_commit_tiles: unknown dtype code %d", dt);
   TL_LAUNCH_CHECK("kv_commit_tiles");
+  return 0;
+}
+
+// tl_rope_split (q and k only) and tl_v_tiles in one launch: see rope_v_tiles_kernel
+int tl_rope_v_tiles(const float* qkv, const int* row_pos, const float* inv_freq, int rotary_dim, int interleaved,
+                    int n, int nq, int nkv, int d, void* q, void* k, void* vt, int vt_cols, int B,
+                    const int* cu_seqlens, const int* tile_off, const int* n_cached, const int* len_after, int dt,
+                    hipStream_t st) {
+  TL_REQUIRE(n >= 0 && nq > 0 && nkv > 0 && d > 0 && d % 2 == 0 && d <= 2 * ROPE_MAX_HALF && B > 0,
+             "rope_v_tiles: bad sizes n=%d nq=%d nkv=%d d=%d B=%d (d even, at most %d)", n, nq, nkv, d, B,
+             2 * ROPE_MAX_HALF);
+  TL_REQUIRE(vt_cols > 0 && vt_cols % PAGE == 0, "rope_v_tiles: %d columns are no multiple of %d", vt_cols, PAGE);
+  TL_REQUIRE(rotary_dim >= 0 && rotary_dim <= d && rotary_dim % 2 == 0 && (rotary_dim == 0 || inv_freq != nullptr),
+             "rope_v_tiles: %d rotated channels of a head of %d (even, at most the head, with their frequencies)",
+             rotary_dim, d);
+  if (n == 0) return 0;
+  const Rotation rot{inv_freq, rotary_dim, interleaved != 0};
+  const long long blocks = (long long)n + (long long)(vt_cols / PAGE) * nkv * ((d + 63) / 64);
+  TL_REQUIRE(blocks < 2147483647LL, "rope_v_tiles: %lld workgroups are too many", blocks);
+  if (dt == DT_F32)
+    rope_v_tiles_kernel<float><<<(unsigned)blocks, 256, 0, st>>>(qkv, row_pos, rot, n, nq, nkv, d, (float*)q, (float*)k,
+                                                                  (float*)vt, vt_cols, B, cu_seqlens, tile_off, n_cached,
+                                                                  len_after);
+  else if (dt == DT_BF16)
+    rope_v_tiles_kernel<bf16><<<(unsigned)blocks, 256, 0, st>>>(qkv, row_pos, rot, n, nq, nkv, d, (bf16*)q, (bf16*)k,
+                                                                 (bf16*)vt, vt_cols, B, cu_seqlens, tile_off, n_cached,
+                                                                 len_after);
+  else
+    TL_REQUIRE(false, "rope_v_tiles: unknown dtype code %d", dt);
+  TL_LAUNCH_CHECK("rope_v_tiles");
   return 0;
 }
 

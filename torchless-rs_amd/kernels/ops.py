@@ -188,6 +188,27 @@ def v_tiles(qkv: torch.Tensor, nq: int, nkv: int, d: int, vt: torch.Tensor, cu_s
                             _p(tile_off), _p(n_cached), _p(len_after), _stream()))
 
 
+def rope_v_tiles(qkv: torch.Tensor, row_pos, rotation, nq: int, nkv: int, d: int, q: torch.Tensor, k: torch.Tensor,
+                 vt: torch.Tensor, cu_seqlens, tile_off, n_cached, len_after) -> None:
+    """`rope_split` (q and k) and `v_tiles` in one launch: the same bits as the two."""
+    n = qkv.shape[0]
+    _req(qkv, "rope_v_tiles.qkv", torch.float32, (n, (nq + 2 * nkv) * d))
+    _req(row_pos, "rope_v_tiles.row_pos", torch.int32, (n,))
+    rot = _rotation(rotation, d, "rope_v_tiles")
+    _req(q, "rope_v_tiles.q", None, (n, nq, d))
+    _req(k, "rope_v_tiles.k", q.dtype, (n, nkv, d))
+    _req(vt, "rope_v_tiles.vt", q.dtype)
+    if vt.dim() != 3 or tuple(vt.shape[:2]) != (nkv, d) or vt.shape[2] % 64:
+        raise KernelError(f"rope_v_tiles.vt: shape {tuple(vt.shape)}, kernel needs [{nkv}, {d}, a multiple of 64]")
+    B = tile_off.shape[0]
+    _tiles_args(B, cu_seqlens, tile_off, n_cached, len_after, "rope_v_tiles")
+    if cu_seqlens is None:
+        raise KernelError("rope_v_tiles.cu_seqlens: needed")
+    _check(lib().tl_rope_v_tiles(_p(qkv), _p(row_pos), _p(rot.inv_freq), rot.rotary_dim, int(rot.interleaved), n, nq,
+                                 nkv, d, _p(q), _p(k), _p(vt), vt.shape[2], B, _p(cu_seqlens), _p(tile_off),
+                                 _p(n_cached), _p(len_after), _code(q.dtype), _stream()))
+
+
 def kv_commit_tiles(k: torch.Tensor, vt: torch.Tensor, row_seq, row_pos, tile_off, n_cached, len_after,
                     table: torch.Tensor, ring_pages: int, pages: torch.Tensor) -> None:
     """`kv_commit` for a step whose values lie transposed by tiles (`v_tiles`): keys row by

@@ -137,8 +137,8 @@ class AttentionMixer(Mixer):
                 # the matrix cores read values along the keys: only the transposed copy is made, by tiles
                 v = None
                 vt = ws.get("attn_vt" + tag, (nkv, d, ctx.host["aligned_cols"]), ctx.dtype)
-                ops.rope_split(qkv, ctx.row_pos, rotation, nq, nkv, d, q, k, None)
-                ops.v_tiles(qkv, nq, nkv, d, vt, ctx.cu_seqlens, ctx.tile_off, ctx.len_before, ctx.len_after)
+                ops.rope_v_tiles(qkv, ctx.row_pos, rotation, nq, nkv, d, q, k, vt, ctx.cu_seqlens, ctx.tile_off,
+                                 ctx.len_before, ctx.len_after)       # rotation and transposition in one launch
             else:
                 vt = None
                 v = ws.get("attn_v" + tag, (n, nkv, d), ctx.dtype)
