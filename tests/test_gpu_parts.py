@@ -598,3 +598,93 @@ def test_part_parameters_that_cannot_be_are_refused():
         make_part("position", PartSpec("rotary", {"head_dim": 16, "theta": 10.0, "rotary_dim": 18}))
     with pytest.raises(ValueError, match="rotated channels"):
         make_part("position", PartSpec("rotary", {"head_dim": 16, "theta": 10.0, "rotary_dim": 7}))
+
+
+def test_a_toy_mixer_whose_values_are_wider_than_its_keys():
+    """The cache does not assume that keys and values have one size: a mixer asks for keys of 8
+    and values of 24 channels (`KVRequest(..., v_head_dim=24)`), gets a group with storage of that
+    shape, and writes and reads it through the group's views.  One head, no rotation, all keys
+    visible; library operations are fine for a toy."""
+    from torchless_rs_amd.cache import KVRequest, PAGE
+    from torchless_rs_amd.engine import Engine, SeqInput
+    from torchless_rs_amd.engine.model import Model
+    from torchless_rs_amd.parts import LayerSpec, Mixer, PartSpec, register_part, unregister_part
+    from torchless_rs_amd.weights import TensorDict, WeightSpec, random_tensors
+    H, V, I, dk, dv = 32, 40, 48, 8, 24
+
+    class WideValues(Mixer):
+        def __init__(self, hidden_size, key_dim, value_dim):
+            self.H, self.dk, self.dv = hidden_size, key_dim, value_dim
+
+        def weight_specs(self):
+            return {"wq.weight": WeightSpec((self.dk, self.H)), "wk.weight": WeightSpec((self.dk, self.H)),
+                    "wv.weight": WeightSpec((self.dv, self.H)), "wo.weight": WeightSpec((self.H, self.dv))}
+
+        def kv_request(self):
+            return KVRequest(1, self.dk, None, v_head_dim=self.dv)
+
+        def load(self, tensors, compute_dtype):
+            self.w = {k: v.float() for k, v in tensors.items()}
+
+        def forward(self, ctx, run, y, x):
+            keys, values = run.kv_group.keys(run.kv_layer), run.kv_group.values_t(run.kv_layer)
+            table = ctx.tables[run.kv_group_index].tolist()
+            cu, pos = ctx.host["cu"], ctx.row_pos.tolist()
+            y = y.float()
+            q, k, v = y @ self.w["wq.weight"].t(), y @ self.w["wk.weight"].t(), y @ self.w["wv.weight"].t()
+            for b in range(ctx.n_seqs):
+                for r in range(int(cu[b]), int(cu[b + 1])):
+                    p = pos[r]
+                    keys[table[b][p // PAGE], 0, p % PAGE] = k[r]
+                    values[table[b][p // PAGE], 0, :, p % PAGE] = v[r]
+                    ks = torch.stack([keys[table[b][j // PAGE], 0, j % PAGE] for j in range(p + 1)])
+                    vs = torch.stack([values[table[b][j // PAGE], 0, :, j % PAGE] for j in range(p + 1)])
+                    a = torch.softmax(ks @ q[r] / math.sqrt(self.dk), 0)
+                    x[r] += (a @ vs) @ self.w["wo.weight"].t()
+
+    register_part("mixer", "wide_values", WideValues)
+    try:
+        norm = PartSpec("rmsnorm", {"size": H, "eps": 1e-5})
+        layers = [LayerSpec(prefix=f"model.layers.{i}.", mixer=PartSpec("wide_values", {"hidden_size": H, "key_dim": dk, "value_dim": dv}),
+                            ffn=PartSpec("swiglu", {"hidden_size": H, "intermediate_size": I}), mixer_norm=norm, ffn_norm=norm)
+                  for i in range(2)]
+        spec = _toy_model(layers, H, V)
+        w = random_tensors(spec.weight_specs(), seed=14, std=0.3, dtype=torch.float32)
+        model = Model(spec, None, torch.float32, DEV)
+        model.load_weights(TensorDict(w))
+        eng = Engine(model, max_tokens=64 * 6, max_slots=3)
+        (group,) = eng.cache.groups
+        assert group.keys(1).shape[1:] == (1, PAGE, dk) and group.values_t(1).shape[1:] == (1, dv, PAGE)
+        assert group.storage.shape[-1] == PAGE * (dk + dv)
+        group.storage.fill_(float("nan"))
+
+        def plain_forward(ids):
+            wd = {k_: v_.double() for k_, v_ in w.items()}
+            T = len(ids)
+            x = wd["model.embed_tokens.weight"][ids]
+            for i in range(2):
+                p = f"model.layers.{i}."
+                y = plain.rmsnorm(x, wd[p + "input_layernorm.weight"], 1e-5)
+                q, k, v = (plain.linear(y, wd[p + n + ".weight"]) for n in ("wq", "wk", "wv"))
+                s = (q @ k.t()) / math.sqrt(dk)
+                s = s.masked_fill(~plain.visible(torch.arange(T), None), float("-inf"))
+                x = x + plain.linear(plain.softmax(s) @ v, wd[p + "wo.weight"])
+                x = x + plain.swiglu(plain.rmsnorm(x, wd[p + "post_attention_layernorm.weight"], 1e-5), wd, p)
+            return plain.linear(plain.rmsnorm(x, wd["model.norm.weight"], 1e-5), wd["lm_head.weight"])
+
+        g = torch.Generator().manual_seed(15)
+        a, b = (torch.randint(0, V, (n,), generator=g).tolist() for n in (70, 9))      # the first crosses a page
+        wa, wb = plain_forward(a), plain_forward(b)
+        sa, sb = eng.alloc(), eng.alloc()
+        lg = eng.step([SeqInput(sa, a[:60], list(range(60))), SeqInput(sb, b[:4], list(range(4)))]).clone()
+        got_a, got_b = [lg[:60]], [lg[60:]]
+        for t in range(5):
+            lg = eng.step([SeqInput(sa, [a[60 + t]], [0]), SeqInput(sb, [b[4 + t]], [0])]).clone()
+            got_a.append(lg[:1]); got_b.append(lg[1:])
+        eng.free(sb)
+        got_a.append(eng.step([SeqInput(sa, a[65:], list(range(5)))]).clone())
+        eng.free(sa)
+        assert rel_err(torch.cat(got_a), wa) < 1e-5 and rel_err(torch.cat(got_b), wb) < 1e-5
+        eng.close()
+    finally:
+        unregister_part("mixer", "wide_values")

@@ -42,10 +42,16 @@ NO_RING = 1 << 24          # "ring" of a group that keeps every position: never 
 
 @dataclass(frozen=True)
 class KVRequest:
-    """Keys and values per position.  `window` None: all positions are kept."""
+    """Keys and values per position.  `window` None: all positions are kept.  `v_head_dim`
+    None: values are as wide as keys (`head_dim`)."""
     n_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    v_head_dim: Optional[int] = None
+
+    @property
+    def value_dim(self) -> int:
+        return self.head_dim if self.v_head_dim is None else self.v_head_dim
 
 
 @dataclass(frozen=True)
@@ -76,7 +82,10 @@ class _Books:
     def close(self) -> None:
         h, self.h = getattr(self, "h", None), None
         if h:
-            native.lib().tl_books_delete(h)
+            try:
+                native.lib().tl_books_delete(h)
+            except (TypeError, AttributeError):         # the interpreter is shutting down: the library is gone with it
+                pass
 
     __del__ = close
 
@@ -190,10 +199,27 @@ class KVGroup:
         self.pool = self.pages_of_slot = None        # views of the books, tied by the cache
         self.storage = None
         if allocate:
-            # [layer, page, K|V, kv_head, row, head_dim]
-            self.storage = torch.empty(
-                (len(self.runs), n_pages, 2, request.n_kv_heads, PAGE, request.head_dim),
-                dtype=dtype, device=device)
+            # A page holds the keys of its 64 positions, [kv_head, row, head_dim], and behind them the
+            # values transposed, [kv_head, value_dim, row].  With values as wide as keys that is
+            # [layer, page, K|V, kv_head, 64, head_dim], the shape the attention kernels take.
+            nkv, dk, dv = request.n_kv_heads, request.head_dim, request.value_dim
+            if dk == dv:
+                self.storage = torch.empty((len(self.runs), n_pages, 2, nkv, PAGE, dk), dtype=dtype, device=device)
+            else:
+                self.storage = torch.empty((len(self.runs), n_pages, nkv * PAGE * (dk + dv)), dtype=dtype,
+                                           device=device)
+
+    def keys(self, layer: int) -> torch.Tensor:
+        """A view of one layer's keys: [page, kv_head, row, head_dim]."""
+        r = self.request
+        flat = self.storage[layer].reshape(self.n_pages, -1)
+        return flat[:, :r.n_kv_heads * PAGE * r.head_dim].view(self.n_pages, r.n_kv_heads, PAGE, r.head_dim)
+
+    def values_t(self, layer: int) -> torch.Tensor:
+        """A view of one layer's values, transposed as they are kept: [page, kv_head, value_dim, row]."""
+        r = self.request
+        flat = self.storage[layer].reshape(self.n_pages, -1)
+        return flat[:, r.n_kv_heads * PAGE * r.head_dim:].view(self.n_pages, r.n_kv_heads, r.value_dim, PAGE)
 
     def pages_needed(self, length: int) -> int:
         return min(pages_for(length), self.ring_pages)
