@@ -619,10 +619,10 @@ def test_qkv_rope_commit_equals_product_then_rope_commit(ops, nq, nkv, d, K, len
     pages1 = c["pages"].clone()
     ops.rope_commit(qkv, c["row_pos"], inv, c["table"], c["ring"], nq, nkv, d, q1, pages1)
     assert ops.qkv_rope_commit_ok(y, w, d, c["pages"])
-    for kv_half in (None, False, True):                      # the launcher's choice, whole tiles, half tiles for k and v
+    for units in (0, 1, 2, 3, 4):                            # the launcher's choice, then 8 to 32 weight rows a workgroup
         q2 = torch.full_like(q1, float("nan"))
         pages2 = c["pages"].clone()
-        ops.qkv_rope_commit(y, w, c["row_pos"], inv, c["table"], c["ring"], nq, nkv, d, q2, pages2, kv_half=kv_half)
+        ops.qkv_rope_commit(y, w, c["row_pos"], inv, c["table"], c["ring"], nq, nkv, d, q2, pages2, units=units)
         assert torch.equal(q1, q2)
         assert torch.equal(torch.nan_to_num(pages1.float(), nan=-7.0), torch.nan_to_num(pages2.float(), nan=-7.0))
     # and against the plain rotation of the plain product
@@ -631,6 +631,8 @@ def test_qkv_rope_commit_equals_product_then_rope_commit(ops, nq, nkv, d, K, len
     want_q = plain.rope(full[:, :nq], pos, 10000.0)
     assert rel_err(q2, want_q) < KTOL["bfloat16"]
     assert not ops.qkv_rope_commit_ok(torch.zeros(17, K, dtype=torch.bfloat16, device=DEV), w, d, pages2)
+    with pytest.raises(ops.KernelError, match="units a workgroup"):
+        ops.qkv_rope_commit(y, w, c["row_pos"], inv, c["table"], c["ring"], nq, nkv, d, q2, pages2, units=5)
     with pytest.raises(ops.KernelError, match="steps of 16"):
         ops.qkv_rope_commit(y, w[: (nq + 2 * nkv) * 8].contiguous(), c["row_pos"], inv[: 4].contiguous(), c["table"],
                             c["ring"], nq, nkv, 8, torch.empty(n, nq, 8, dtype=torch.bfloat16, device=DEV),
@@ -658,8 +660,9 @@ def test_gemm_norm_halves(ops, M, N, K, N2):
     plain_x = x0.clone().to(DEV)
     ops.gemm_bf16(a.to(DEV), w.to(DEV), plain_x, accumulate=True)
     assert torch.equal(plain_x, x)                                    # the stream itself is unchanged by the extra
-    assert groups == -(-N // 16)
-    assert rel_err(ssq[:M].sum(1), (x.double().cpu() ** 2).sum(1)) < 1e-5
+    assert 0 < groups <= -(-N // 16)                                  # workgroups own 16 channels or more
+    written = ssq.flatten()[: 16 * groups].view(16, groups)          # [row][workgroup], as many columns as workgroups
+    assert rel_err(written[:M].sum(1), (x.double().cpu() ** 2).sum(1)) < 1e-5
     assert rel_err(xt, x.double().cpu() * g.double()) < KTOL["bfloat16"]
     factor = ops.RowFactor(ssq, groups, N, eps)
     normed = plain.rmsnorm(x.double().cpu(), g.double(), eps)
@@ -670,7 +673,7 @@ def test_gemm_norm_halves(ops, M, N, K, N2):
     # exactly: the unscaled product times the factor of the row
     raw = torch.empty(M, N2, device=DEV)
     ops.gemm_bf16(xt, w2.to(DEV), raw)
-    r = torch.rsqrt(ssq[:M].double().sum(1) / N + eps).float()
+    r = torch.rsqrt(written[:M].double().sum(1) / N + eps).float()
     assert rel_err(out, raw.double().cpu() * r.double().cpu()[:, None]) < 1e-6
     if N2 % 64 == 0:
         from torchless_rs_amd.parts.linear import interleave_pairs
@@ -759,8 +762,8 @@ def test_products_from_the_tiled_copy_give_the_same_bits(ops, M, N, K):
         xt = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
         ssq = torch.full((16, N // 16), float("nan"), device=DEV)
         groups = ops.gemm_bf16_norm(a, w, x, accumulate=True, norm_weight=g, xt=xt, ssq_out=ssq, tiles=t)
-        res.append((x, xt, ssq[:M].clone(), groups))
-    assert res[0][3] == res[1][3] == N // 16
+        res.append((x, xt, ssq.flatten()[: 16 * groups].view(16, groups)[:M].clone(), groups))
+    assert 0 < res[0][3] == res[1][3] <= N // 16
     for u, v in zip(res[0][:3], res[1][:3]):
         assert torch.equal(u, v)
     ssq_in = (torch.rand(16, 3, generator=torch.Generator().manual_seed(67)) * K).to(DEV)
@@ -792,13 +795,13 @@ def test_qkv_rope_commit_from_the_tiled_copy(ops, nq, nkv, d, K, lens):
     tiles = ops.tile_weights(w, rows)
     ssq_in = (torch.rand(16, 4, generator=torch.Generator().manual_seed(22)) * K).to(DEV)
     for factor in (None, ops.RowFactor(ssq_in, 4, K, 1e-6)):
-        for kv_half in (None, False, True):
+        for units in (0, 1, 2, 3, 4):
             out = []
             for t in (None, tiles):
                 q = torch.full((n, nq, d), float("nan"), dtype=torch.bfloat16, device=DEV)
                 pages = c["pages"].clone()
                 ops.qkv_rope_commit(y, w, c["row_pos"], inv, c["table"], c["ring"], nq, nkv, d, q, pages,
-                                    factor=factor, kv_half=kv_half, tiles=t)
+                                    factor=factor, units=units, tiles=t)
                 out.append((q, torch.nan_to_num(pages.float(), nan=-7.0)))
             assert torch.equal(out[0][0], out[1][0])
             assert torch.equal(out[0][1], out[1][1])
@@ -1068,11 +1071,11 @@ def test_qkv_rope_commit_takes_any_rotation(ops, share, interleaved, nq, nkv, d,
         assert rows[:16].tolist() == list(range(0, 16, 2)) + list(range(1, 16, 2))
     tiles = ops.tile_weights(w, rows) if K % 64 == 0 else None
     for t in (None, tiles):
-        for kv_half in (False, True):
+        for units in (1, 2, 3, 4):
             q2, pages2 = torch.full_like(q1, float("nan")), c["pages"].clone()
             ops.qkv_rope_commit(y, w, c["row_pos"], rot, c["table"], c["ring"], nq, nkv, d, q2, pages2,
-                                kv_half=kv_half, tiles=t)
-            assert torch.equal(q1, q2), (t is not None, kv_half)
+                                units=units, tiles=t)
+            assert torch.equal(q1, q2), (t is not None, units)
             assert torch.equal(torch.nan_to_num(pages1.float(), nan=-7.0), torch.nan_to_num(pages2.float(), nan=-7.0))
     full = (y.double().cpu() @ w.double().cpu().t()).view(n, nq + 2 * nkv, d)
     assert rel_err(q1, plain.rope_variant(full[:, :nq], c["row_pos"].cpu().long(), 10000.0, r, interleaved)) < KTOL["bfloat16"]

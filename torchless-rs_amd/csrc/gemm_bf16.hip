@@ -118,12 +118,17 @@ tile_weights_kernel(const bf16* __restrict__ W, const int* __restrict__ rows, in
 template <int NT, int MT, int SK_WAVES, bool FULLK, bool TILED = false>      // FULLK: K % 64 == 0, no load needs a guard (and a branch)
 __global__ void __launch_bounds__(SK_WAVES * 64)
 gemm_skinny_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float* __restrict__ C, int M,
-                   int N, int K, int epilogue, NormSplit ns) {
+                   int N, int K, int epilogue, NormSplit ns, int rows_per_wg) {
+  // rows_per_wg: the channels a workgroup owns, at most 16 NT (0: all 16 NT).  A compute unit streams
+  // at a rate of its own, so a product is fastest when every unit has the same share of W: the
+  // launcher picks N / units where that is no multiple of 16, and the lanes of an MFMA tile that
+  // have no channel read another's again and their sums are dropped.
   __shared__ float red[SK_WAVES][NT * MT * 256];
   __shared__ float rs[16];
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const int li = lane % 16, kg = lane / 16;
-  const int n0 = blockIdx.x * (16 * NT);
+  const int R = rows_per_wg > 0 ? rows_per_wg : 16 * NT;
+  const int n0 = blockIdx.x * R;
   const int steps = (K + 63) / 64;
   const int per = (steps + SK_WAVES - 1) / SK_WAVES;
   const int s0 = wave * per;
@@ -132,9 +137,10 @@ gemm_skinny_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float
   const bf16* wrow[NT];
   const bf16* arow[MT];
 #pragma unroll
-  for (int t = 0; t < NT; ++t)
-    wrow[t] = TILED ? W + (size_t)(n0 / 16 + t) * 16 * K + kg * 128 + li * 8
-                    : W + (size_t)min(n0 + t * 16 + li, N - 1) * K;
+  for (int t = 0; t < NT; ++t) {
+    const int gr = min(n0 + min(t * 16 + li, R - 1), N - 1);          // this lane's channel (clamped: never a branch)
+    wrow[t] = TILED ? W + (size_t)(gr / 16) * 16 * K + kg * 128 + (gr % 16) * 8 : W + (size_t)gr * K;
+  }
 #pragma unroll
   for (int u = 0; u < MT; ++u) arow[u] = A + (size_t)min(u * 16 + li, M - 1) * K;
 
@@ -182,7 +188,7 @@ gemm_skinny_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float
   float c_old = 0.f, w_norm = 0.f;
   if (one_each && epilogue == EPI_ACCUMULATE) {
     const int nl = threadIdx.x % NB, m = threadIdx.x / NB;
-    if ((int)threadIdx.x < NB * 16 * MT && n0 + nl < N && m < M) {
+    if ((int)threadIdx.x < NB * 16 * MT && nl < R && n0 + nl < N && m < M) {
       c_old = C[(size_t)m * N + n0 + nl];
       if (writer) w_norm = ns.norm_w[n0 + nl];
     }
@@ -240,7 +246,7 @@ gemm_skinny_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float
     const float v = total(nl, m);
     const int n = n0 + nl;
     float xn = 0.f;
-    if (n < N && m < M) {
+    if (nl < R && n < N && m < M) {
       float* c = C + (size_t)m * N + n;
       xn = (epilogue == EPI_ACCUMULATE) ? (one_each ? c_old : *c) + v : v;
       *c = xn;
@@ -259,21 +265,53 @@ static bool tiles_fit(int N, int K) { return N % 16 == 0 && K % 64 == 0; }
 
 template <int NT, int MT, int SK_WAVES = 8>
 static int launch_skinny(const bf16* A, const bf16* W, float* C, int M, int N, int K, int epilogue,
-                         hipStream_t st, NormSplit ns = NormSplit{}, const bf16* Wt = nullptr) {
-  const int grid = (N + 16 * NT - 1) / (16 * NT);
-  if constexpr (NT == 1 && MT == 1 && SK_WAVES == 8) {
+                         hipStream_t st, NormSplit ns = NormSplit{}, const bf16* Wt = nullptr, int rows_per_wg = 0) {
+  const int R = rows_per_wg > 0 ? rows_per_wg : 16 * NT;
+  const int grid = (N + R - 1) / R;
+  if constexpr (MT == 1 && SK_WAVES == 8 && NT <= 2) {
     if (Wt != nullptr && tiles_fit(N, K)) {
-      gemm_skinny_kernel<NT, MT, SK_WAVES, true, true><<<grid, SK_WAVES * 64, 0, st>>>(A, Wt, C, M, N, K, epilogue, ns);
+      gemm_skinny_kernel<NT, MT, SK_WAVES, true, true><<<grid, SK_WAVES * 64, 0, st>>>(A, Wt, C, M, N, K, epilogue, ns, R);
       TL_LAUNCH_CHECK("gemm_skinny");
       return 0;
     }
   }
   if (K % 64 == 0)
-    gemm_skinny_kernel<NT, MT, SK_WAVES, true><<<grid, SK_WAVES * 64, 0, st>>>(A, W, C, M, N, K, epilogue, ns);
+    gemm_skinny_kernel<NT, MT, SK_WAVES, true><<<grid, SK_WAVES * 64, 0, st>>>(A, W, C, M, N, K, epilogue, ns, R);
   else
-    gemm_skinny_kernel<NT, MT, SK_WAVES, false><<<grid, SK_WAVES * 64, 0, st>>>(A, W, C, M, N, K, epilogue, ns);
+    gemm_skinny_kernel<NT, MT, SK_WAVES, false><<<grid, SK_WAVES * 64, 0, st>>>(A, W, C, M, N, K, epilogue, ns, R);
   TL_LAUNCH_CHECK("gemm_skinny");
   return 0;
+}
+
+static int compute_units() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    cus = n;
+  }
+  return cus;
+}
+
+// The channels a workgroup of the kernel for at most 16 rows owns (16 to 32).  One tile of 16 each
+// while the device has a unit for every tile; beyond that the tiles would go round the units
+// unevenly (320 tiles on 256 units take as long as 512), so the channels are dealt in equal shares
+// to a whole number of rounds of workgroups.
+static int balanced_share(int N) {
+  const int cus = compute_units();
+  if ((N + 15) / 16 <= cus) return 16;
+  const long long rounds = ((long long)N + 32LL * cus - 1) / (32LL * cus);
+  const long long wgs = rounds * cus;
+  const int share = (int)((N + wgs - 1) / wgs);
+  return share < 16 ? 16 : share;
+}
+
+// the product for at most 16 rows and not many channels, in balanced shares
+static int launch_shares(const bf16* A, const bf16* W, const bf16* Wt, float* C, int M, int N, int K, int epilogue,
+                         hipStream_t st, NormSplit ns, int share) {
+  if (share <= 16) return launch_skinny<1, 1, 8>(A, W, C, M, N, K, epilogue, st, ns, Wt, share);
+  return launch_skinny<2, 1, 8>(A, W, C, M, N, K, epilogue, st, ns, Wt, share);
 }
 
 // ------------------------------------------------------- rows, 1 KB at a time ----
@@ -397,96 +435,103 @@ static int launch_rows(const bf16* A, const bf16* W, float* C, int M, int N, int
 }
 
 // ------------------------------------------------- q|k|v of single tokens ----
-// The skinny product (16 channels a workgroup, 8 waves over K, up to 16 rows) for the
-// fused projection of a step with one token a sequence, with what follows it done on
-// the sums while they are in LDS: rotation of q and k by the position, q to its buffer,
-// k and v into the sequence's page (v transposed).  To have both channels of a rotated
-// pair, a tile of a q or k head takes the first channels of pairs 8t..8t+7 and then their
-// second channels (`pair_channels`: with all of a head rotated in halves these are 8t..8t+7
-// and d/2+8t..d/2+8t+7); a tile of a v head takes 16 in a row.  With kv_half the tiles of k and v heads are half as large
-// (4 pairs, or 8 channels, in the first 8 rows of the MFMA tile; the other rows load
-// nothing): the launcher asks for that when it spreads the workgroups more evenly over
-// the compute units (7B: 384 tiles are one and a half a unit, 256 + 256 are two for all).
+// The skinny product (8 waves over K, up to 16 rows) for the fused projection of a step with
+// one token a sequence, with what follows it done on the sums while they are in LDS: rotation
+// of q and k by the position, q to its buffer, k and v into the sequence's page (v transposed).
+// The projection's channels are dealt in units of 8 weight rows, d / 8 a head: unit h of a q or
+// k head holds the first channels of its pairs 4h..4h+3 and then their second channels
+// (`pair_channels`: with all of a head rotated in halves these are 4h..4h+3 and d/2+4h..d/2+4h+3),
+// so that both channels of a rotated pair meet in one workgroup; a unit of a v head holds 8
+// channels in a row.  A workgroup owns `units` consecutive units (at most 2 NT, two to an MFMA
+// tile of 16 rows; rows of a tile without a unit load nothing).  The launcher deals the
+// units in equal shares to the compute units, because each of them streams at a rate of its own
+// (7B: 768 units are 3 for each of 256).
 // The sums and the rotation are those of the unfused kernels, bit for bit
 // (a' = a c - b s; b' = a s + b c; src/kernels/mod.rs:603-605 of the reference).
-// TILED: W is the tiled copy whose tile (head, t) holds the 16 channels named above in that
-// order (`tl_qkv_tile_rows`), so a half tile is rows np*sub.. and 8 + np*sub.. of its tile.
+// TILED: W is the tiled copy whose tile (head, t) holds units 2t and 2t+1 of the head, first
+// channels in its rows 0..7, second channels in 8..15 (`tl_qkv_tile_rows`).
 constexpr int QKV_WAVES = 8;
 
-template <bool TILED>
+template <bool TILED, int NT>
 __global__ void __launch_bounds__(QKV_WAVES * 64)
 gemm_qkv_rope_commit_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, int M, int K,
                             const int* __restrict__ row_pos, Rotation rot,
                             const int* __restrict__ table, int table_stride, int ring_pages, int nq,
                             int nkv, int d, bf16* __restrict__ q, bf16* __restrict__ pages, NormSplit ns,
-                            int kv_half) {
-  __shared__ float red[QKV_WAVES][256];
-  __shared__ float cs[16][8], sn[16][8];
+                            int units) {
+  __shared__ float red[QKV_WAVES][NT * 256];
+  __shared__ float cs[2 * NT][16][4], sn[2 * NT][16][4];
   __shared__ float rs[16];
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
   const int li = lane % 16, kg = lane / 16;
-  // which head, which tile of it, and how many pairs (or, for v, channels / 2) the tile holds
-  int head, tt, np = 8;
-  {
-    const int full = d / 16, q_tiles = nq * full;
-    if (!kv_half || (int)blockIdx.x < q_tiles) {
-      head = blockIdx.x / full;
-      tt = blockIdx.x % full;
+  const int per_head = d / 8, n_units = (nq + 2 * nkv) * per_head;
+  const int g0 = blockIdx.x * units;
+  const int mine = min(units, n_units - g0);           // units of this workgroup
+  const bf16* wrow[NT];
+  bool loads[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const int u = 2 * t + li / 8, j = li % 8;          // this lane's row of tile t: row j of unit u
+    loads[t] = u < mine;
+    const int g = g0 + (loads[t] ? u : 0);
+    const int head = g / per_head, h = g % per_head;
+    const bool rotated = head < nq + nkv;
+    if constexpr (TILED) {
+      const int sub = h % 2;
+      const int r = rotated ? (j < 4 ? 4 * sub + j : 8 + 4 * sub + j - 4) : 8 * sub + j;
+      wrow[t] = W + (size_t)(head * (d / 16) + h / 2) * 16 * K + kg * 128 + r * 8;
     } else {
-      const int r = blockIdx.x - q_tiles;
-      head = nq + r / (2 * full);
-      tt = r % (2 * full);
-      np = 4;
+      int ch = 8 * h + j;
+      if (rotated) {
+        int ca, cb;
+        pair_channels(4 * h + (j < 4 ? j : j - 4), rot.rotary_dim, rot.interleaved, ca, cb);
+        ch = j < 4 ? ca : cb;
+      }
+      wrow[t] = W + ((size_t)head * d + ch) * K;
     }
-  }
-  const bool rotated = head < nq + nkv;
-  const bool loads = li < 2 * np;               // rows of the MFMA tile that hold a channel
-  int ch = 2 * np * tt + li;
-  if (rotated) {
-    int ca, cb;
-    pair_channels(np * tt + (li < np ? li : li - np), rot.rotary_dim, rot.interleaved, ca, cb);
-    ch = li < np ? ca : cb;
-  }
-  const bf16* wrow;
-  if constexpr (TILED) {
-    // the tile that holds this (half) tile's channels, and this lane's row in it
-    const int sub = np == 8 ? 0 : tt % 2;
-    const int tile = head * (d / 16) + (np == 8 ? tt : tt / 2);
-    const int r = rotated ? (li < np ? np * sub + li : 8 + np * sub + li - np) : 2 * np * sub + li;
-    wrow = W + (size_t)tile * 16 * K + kg * 128 + (loads ? r : 0) * 8;
-  } else {
-    wrow = W + ((size_t)head * d + (loads ? ch : 0)) * K;
   }
   const bf16* arow = A + (size_t)min(li, M - 1) * K;
   const int steps = (K + 63) / 64;
   const int per = (steps + QKV_WAVES - 1) / QKV_WAVES;
   const int s0 = wave * per, s1 = min(steps, s0 + per);
 
-  f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
-  auto load_step = [&](int s, bf16x8 (&wv)[2], bf16x8 (&av)[2]) {
+  f32x4 acc[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  auto load_step = [&](int s, bf16x8 (&wv)[NT][2], bf16x8 (&av)[2]) {
     const int k = s * 64 + kg * 16;
     const bool ok0 = k + 8 <= K, ok1 = k + 16 <= K;
-    if constexpr (TILED) {
-      wv[0] = loads ? load8(wrow + (size_t)s * TILE_STEP) : zero8();
-      wv[1] = loads ? load8(wrow + (size_t)s * TILE_STEP + TILE_STEP / 2) : zero8();
-    } else {
-      wv[0] = (ok0 && loads) ? load8(wrow + k) : zero8();
-      wv[1] = (ok1 && loads) ? load8(wrow + k + 8) : zero8();
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      if constexpr (TILED) {
+        wv[t][0] = loads[t] ? load8(wrow[t] + (size_t)s * TILE_STEP) : zero8();
+        wv[t][1] = loads[t] ? load8(wrow[t] + (size_t)s * TILE_STEP + TILE_STEP / 2) : zero8();
+      } else {
+        wv[t][0] = (ok0 && loads[t]) ? load8(wrow[t] + k) : zero8();
+        wv[t][1] = (ok1 && loads[t]) ? load8(wrow[t] + k + 8) : zero8();
+      }
     }
     av[0] = ok0 ? load8(arow + k) : zero8();
     av[1] = ok1 ? load8(arow + k + 8) : zero8();
   };
-  auto mma_step = [&](bf16x8 (&wv)[2], bf16x8 (&av)[2]) {
-    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[0], av[0], acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[1], av[1], acc, 0, 0, 0);
+  auto mma_step = [&](bf16x8 (&wv)[NT][2], bf16x8 (&av)[2]) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[t][0], av[0], acc[t], 0, 0, 0);
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[t][1], av[1], acc[t], 0, 0, 0);
+    }
   };
-  bf16x8 w0[2], a0[2], w1[2], a1[2];
+  bf16x8 w0[NT][2], a0[2], w1[NT][2], a1[2];
   int s = s0;
   if (s < s1) load_step(s, w0, a0);
-  if (rotated && tid < 128) {                  // while the first loads are under way
-    const int m = tid / 8, j = tid % 8;
-    if (m < M && j < np && 2 * (np * tt + j) < rot.rotary_dim)
-      sincosf(rot.inv_freq[np * tt + j] * (float)row_pos[m], &sn[m][j], &cs[m][j]);
+  // the threads of the epilogue: 128 a unit; of a rotated unit 64 work, one a row and pair
+  const int eu = tid / 128, et = tid % 128;
+  const int eg = g0 + min(eu, mine - 1);
+  const int ehead = eg / per_head, eh = eg % per_head;
+  const bool e_on = eu < mine, e_rot = ehead < nq + nkv;
+  if (e_on && e_rot && et < 64) {              // while the first loads are under way
+    const int m = et / 4, j = et % 4, i = 4 * eh + j;
+    if (m < M && 2 * i < rot.rotary_dim) sincosf(rot.inv_freq[i] * (float)row_pos[m], &sn[eu][m][j], &cs[eu][m][j]);
   }
   const bool scaled = ns.ssq_in != nullptr;
   RowFactors rf;
@@ -500,44 +545,46 @@ gemm_qkv_rope_commit_kernel(const bf16* __restrict__ A, const bf16* __restrict__
   if (s < s1) mma_step(w0, a0);
   if (scaled) rf.finish(ns, rs);
 #pragma unroll
-  for (int r = 0; r < 4; ++r) red[wave][r * 64 + lane] = acc[r];     // D[n = 4 kg + r][m = li]
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) red[wave][(t * 4 + r) * 64 + lane] = acc[t][r];     // D[n = 4 kg + r][m = li] of tile t
   __syncthreads();
-  auto total = [&](int nl, int m) {
-    const int idx = (nl % 4) * 64 + (nl / 4) * 16 + m;
+  auto total = [&](int row, int m) {               // row: 8 u + j, row j of the workgroup's unit u
+    const int nl = row % 16;
+    const int idx = ((row / 16) * 4 + nl % 4) * 64 + (nl / 4) * 16 + m;
     float v = 0.f;
 #pragma unroll
     for (int w = 0; w < QKV_WAVES; ++w) v += red[w][idx];
     return scaled ? v * rs[m] : v;
   };
+  if (!e_on) return;
   const size_t page_elems = 2 * (size_t)nkv * PAGE * d;
-  if (rotated) {
-    if (tid < 128) {
-      const int m = tid / 8, j = tid % 8;
-      if (m < M && j < np) {
-        const int i = np * tt + j;
-        float ra = total(j, m), rb = total(j + np, m);
-        if (2 * i < rot.rotary_dim) rotate_pair(ra, rb, cs[m][j], sn[m][j], ra, rb);
-        int ia, ib;
-        pair_channels(i, rot.rotary_dim, rot.interleaved, ia, ib);
-        bf16* dst;
-        if (head < nq) {
-          dst = q + ((size_t)m * nq + head) * d;
-        } else {
-          const int p = row_pos[m];
-          const int page = table[(size_t)m * table_stride + (p / PAGE) % ring_pages];
-          dst = pages + (size_t)page * page_elems + ((size_t)(head - nq) * PAGE + p % PAGE) * d;
-        }
-        dst[ia] = (bf16)ra;
-        dst[ib] = (bf16)rb;
+  if (e_rot) {
+    const int m = et / 4, j = et % 4;
+    if (et < 64 && m < M) {
+      const int i = 4 * eh + j;
+      float ra = total(8 * eu + j, m), rb = total(8 * eu + 4 + j, m);
+      if (2 * i < rot.rotary_dim) rotate_pair(ra, rb, cs[eu][m][j], sn[eu][m][j], ra, rb);
+      int ia, ib;
+      pair_channels(i, rot.rotary_dim, rot.interleaved, ia, ib);
+      bf16* dst;
+      if (ehead < nq) {
+        dst = q + ((size_t)m * nq + ehead) * d;
+      } else {
+        const int p = row_pos[m];
+        const int page = table[(size_t)m * table_stride + (p / PAGE) % ring_pages];
+        dst = pages + (size_t)page * page_elems + ((size_t)(ehead - nq) * PAGE + p % PAGE) * d;
       }
+      dst[ia] = (bf16)ra;
+      dst[ib] = (bf16)rb;
     }
-  } else if (tid < 256) {
-    const int m = tid / 16, nl = tid % 16;
-    if (m < M && nl < 2 * np) {
+  } else {
+    const int m = et / 8, nl = et % 8;
+    if (m < M) {
       const int p = row_pos[m];
       const int page = table[(size_t)m * table_stride + (p / PAGE) % ring_pages];
       bf16* vd = pages + (size_t)page * page_elems + (size_t)nkv * PAGE * d;
-      vd[((size_t)(head - nq - nkv) * d + 2 * np * tt + nl) * PAGE + p % PAGE] = (bf16)total(nl, m);
+      vd[((size_t)(ehead - nq - nkv) * d + 8 * eh + nl) * PAGE + p % PAGE] = (bf16)total(8 * eu + nl, m);
     }
   }
 }
@@ -963,7 +1010,7 @@ extern "C" int tl_gemm_bf16(const void* A, const void* W, const void* Wt, void* 
   if (M <= 16) {
     if (wide && rows_fit(M, N, K)) return launch_rows(a, w, c, M, N, K, epilogue, st);
     if (wide && (M > 4 || epilogue == EPI_SILU_PAIR)) return launch_skinny<4, 1, 4>(a, w, c, M, N, K, epilogue, st);
-    return launch_skinny<1, 1, 8>(a, w, c, M, N, K, epilogue, st, NormSplit{}, (const bf16*)Wt);
+    return launch_shares(a, w, (const bf16*)Wt, c, M, N, K, epilogue, st, NormSplit{}, balanced_share(N));
   }
   if (M <= 32) {
     if (wide) return launch_skinny<4, 2, 4>(a, w, c, M, N, K, epilogue, st);
@@ -1001,6 +1048,12 @@ extern "C" int tl_gemm_bf16_variant(const void* A, const void* W, void* C, int M
     TL_REQUIRE(rows_fit(M, N, K), "gemm_rows: M=%d N=%d K=%d (at most 16 rows, N a multiple of 64, K of %d)", M, N,
                K, ROWS_CHUNK);
     return launch_rows(a, w, c, M, N, K, epilogue, st);
+  }
+  if (variant >= 1000 && variant <= 1032) {            // 1000 + channels a workgroup, at most 16 rows
+    TL_REQUIRE(M <= 16 && epilogue != EPI_SILU_PAIR, "gemm_skinny: variant %d takes at most 16 rows and no pairs", variant);
+    const int R = variant - 1000;
+    if (R <= 16) return launch_skinny<1, 1, 8>(a, w, c, M, N, K, epilogue, st, NormSplit{}, nullptr, R);
+    return launch_skinny<2, 1, 8>(a, w, c, M, N, K, epilogue, st, NormSplit{}, nullptr, R);
   }
   const int mt = (variant / 10) % 10;
   TL_REQUIRE(M <= 16 * mt, "gemm_skinny: variant %d takes at most %d rows, not %d", variant, 16 * mt, M);
@@ -1050,7 +1103,8 @@ extern "C" int tl_gemm_mid_bf16(const void* A, const void* W, void* C, int M, in
 // q|k|v of a step with one token a sequence (row m is sequence m, at position row_pos[m]):
 // W is [(nq + 2 nkv) d, K]; q receives [M, nq, d], the pages k and v of the new position.
 // With ssq_in, row m's sums are multiplied by rsqrt(sum_j ssq_in[m][j] * inv_h + eps) first.
-// kv_half: 1 halves the tiles of k and v heads, 0 does not, -1 lets the launcher choose.
+// units: the units of 8 weight rows (see the kernel) a workgroup owns, 1 to 4; 0 lets the
+// launcher deal them in equal shares to the device's compute units.
 // Wt (or null): the tiled copy of W with the rows of `tl_qkv_tile_rows`, read instead of W
 // when K % 64 == 0.
 extern "C" int tl_gemm_qkv_rope_commit(const void* A, const void* W, const void* Wt, int M, int K, const int* row_pos,
@@ -1058,7 +1112,7 @@ extern "C" int tl_gemm_qkv_rope_commit(const void* A, const void* W, const void*
                                        const int* table, int table_stride,
                                        int ring_pages, int nq, int nkv, int d, void* q, void* pages,
                                        const float* ssq_in, int n_part, float inv_h, float eps,
-                                       int kv_half, hipStream_t st) {
+                                       int units, hipStream_t st) {
   TL_REQUIRE(M >= 0 && M <= 16 && K > 0 && K % 8 == 0, "qkv_rope_commit: bad sizes M=%d K=%d (at most 16 rows, "
              "K a multiple of 8)", M, K);
   TL_REQUIRE(nq > 0 && nkv > 0 && d >= 16 && d % 16 == 0, "qkv_rope_commit: bad heads nq=%d nkv=%d d=%d (head "
@@ -1070,34 +1124,32 @@ extern "C" int tl_gemm_qkv_rope_commit(const void* A, const void* W, const void*
   TL_REQUIRE(rotary_dim >= 0 && rotary_dim <= d && rotary_dim % 2 == 0 && (rotary_dim == 0 || inv_freq != nullptr),
              "qkv_rope_commit: %d rotated channels of a head of %d (even, at most the head, with their "
              "frequencies)", rotary_dim, d);
+  TL_REQUIRE(units >= 0 && units <= 4, "qkv_rope_commit: %d units a workgroup (1 to 4, or 0 for the launcher's choice)", units);
   const Rotation rot{inv_freq, rotary_dim, interleaved != 0};
   if (M == 0) return 0;
-  const int full = (nq + 2 * nkv) * (d / 16), mixed = nq * (d / 16) + 2 * nkv * (d / 8);
-  if (kv_half < 0) {
-    // in units of half a tile, on as many compute units as the device has: which way ends sooner?
-    static int cus = 0;
-    if (cus == 0) {
-      int dev = 0, n = 0;
-      if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-        n = 256;
-      cus = n;
-    }
-    const int t_full = 2 * ((full + cus - 1) / cus), t_mixed = (2 * nq * (d / 16) + 2 * nkv * (d / 8) + cus - 1) / cus;
-    kv_half = t_mixed < t_full;
+  const long long n_units = (long long)(nq + 2 * nkv) * (d / 8);
+  if (units == 0) {
+    // a whole number of rounds of workgroups over the compute units, of at most 4 units each
+    const int cus = compute_units();
+    const long long wgs = ((n_units + 4LL * cus - 1) / (4LL * cus)) * cus;
+    units = (int)((n_units + wgs - 1) / wgs);
   }
-  const int grid = kv_half ? mixed : full;
+  const int grid = (int)((n_units + units - 1) / units);
   NormSplit ns{};
   ns.ssq_in = ssq_in; ns.n_part = n_part; ns.inv_h = inv_h; ns.eps = eps;
-  if (Wt != nullptr && K % 64 == 0) {
-    TL_REQUIRE((uintptr_t)Wt % 16 == 0, "qkv_rope_commit: operands must be 16-byte aligned");
-    gemm_qkv_rope_commit_kernel<true><<<grid, QKV_WAVES * 64, 0, st>>>(
-        (const bf16*)A, (const bf16*)Wt, M, K, row_pos, rot, table, table_stride, ring_pages, nq, nkv, d,
-        (bf16*)q, (bf16*)pages, ns, kv_half);
+  const bool tiled = Wt != nullptr && K % 64 == 0;
+  TL_REQUIRE(!tiled || (uintptr_t)Wt % 16 == 0, "qkv_rope_commit: operands must be 16-byte aligned");
+  const bf16* w = tiled ? (const bf16*)Wt : (const bf16*)W;
+#define TL_QKV(TILED, NT)                                                                               \
+  gemm_qkv_rope_commit_kernel<TILED, NT><<<grid, QKV_WAVES * 64, 0, st>>>(                              \
+      (const bf16*)A, w, M, K, row_pos, rot, table, table_stride, ring_pages, nq, nkv, d, (bf16*)q, \
+      (bf16*)pages, ns, units)
+  if (units <= 2) {
+    if (tiled) TL_QKV(true, 1); else TL_QKV(false, 1);
   } else {
-    gemm_qkv_rope_commit_kernel<false><<<grid, QKV_WAVES * 64, 0, st>>>(
-        (const bf16*)A, (const bf16*)W, M, K, row_pos, rot, table, table_stride, ring_pages, nq, nkv, d,
-        (bf16*)q, (bf16*)pages, ns, kv_half);
+    if (tiled) TL_QKV(true, 2); else TL_QKV(false, 2);
   }
+#undef TL_QKV
   TL_LAUNCH_CHECK("gemm_qkv_rope_commit");
   return 0;
 }
@@ -1126,7 +1178,8 @@ extern "C" int tl_gemm_bf16_norm(const void* A, const void* W, const void* Wt, v
   const bool wide = N >= 16384 || epilogue == EPI_SILU_PAIR;
   const bool rows = wide && !writer && rows_fit(M, N, K);        // many channels, K in chunks of 512: whole rows, 1 KB a load
   const bool four = wide && (M > 4 || epilogue == EPI_SILU_PAIR);
-  const int groups = four ? (N + 63) / 64 : (N + 15) / 16;
+  const int share = four ? 64 : balanced_share(N);
+  const int groups = (N + share - 1) / share;
   if (n_groups) *n_groups = groups;
   TL_REQUIRE(!writer || ssq_capacity >= groups * 16, "gemm_bf16_norm: ssq_out holds %d floats, %d are needed",
              ssq_capacity, groups * 16);
@@ -1137,7 +1190,7 @@ extern "C" int tl_gemm_bf16_norm(const void* A, const void* W, const void* Wt, v
   if (rows) return launch_rows((const bf16*)A, (const bf16*)W, (float*)C, M, N, K, epilogue, st, ns);
   if (four) return launch_skinny<4, 1, 4>((const bf16*)A, (const bf16*)W, (float*)C, M, N, K, epilogue, st, ns);
   TL_REQUIRE((uintptr_t)Wt % 16 == 0, "gemm_bf16_norm: operands must be 16-byte aligned");
-  return launch_skinny<1, 1, 8>((const bf16*)A, (const bf16*)W, (float*)C, M, N, K, epilogue, st, ns, (const bf16*)Wt);
+  return launch_shares((const bf16*)A, (const bf16*)W, (const bf16*)Wt, (float*)C, M, N, K, epilogue, st, ns, share);
 }
 
 // Wt [N/16][K/64][2][4][16][8] = the tiled copy of W [N, K] (N % 16 == 0, K % 64 == 0) with its

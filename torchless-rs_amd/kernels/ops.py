@@ -584,12 +584,12 @@ def qkv_rope_commit_ok(a: torch.Tensor, w: torch.Tensor, d: int, pages: torch.Te
 
 def qkv_rope_commit(a: torch.Tensor, w: torch.Tensor, row_pos, rotation, table, ring_pages: int, nq: int,
                     nkv: int, d: int, q: torch.Tensor, pages: torch.Tensor,
-                    factor: Optional[RowFactor] = None, kv_half: Optional[bool] = None,
+                    factor: Optional[RowFactor] = None, units: int = 0,
                     tiles: Optional[torch.Tensor] = None) -> None:
     """For a step with one token a sequence (at most 16): the product a @ w^T with w = q|k|v,
     the rotation of q and k, q into its buffer and k, v into the pages, in one kernel; the
-    same bits as `gemm` and then `rope_commit`.  `factor`: see `gemm_bf16_norm`.  `kv_half`
-    (tests): force or forbid the smaller tiles for k and v that the launcher may choose.
+    same bits as `gemm` and then `rope_commit`.  `factor`: see `gemm_bf16_norm`.  `units`
+    (tests): how many units of 8 weight rows a workgroup owns, 1 to 4; 0 leaves it to the launcher.
     `tiles`: `tile_weights(w, qkv_tile_rows(nq, nkv, d, device, rotation))`, read instead of w.
     `rotation`: see `rope_split`."""
     n, K = a.shape
@@ -615,7 +615,7 @@ def qkv_rope_commit(a: torch.Tensor, w: torch.Tensor, row_pos, rotation, table, 
                                          rot.rotary_dim, int(rot.interleaved), _p(table),
                                          table.shape[1], int(ring_pages), nq, nkv, d, _p(q), _p(pages),
                                          _p(ssq_in), n_part, ctypes.c_float(inv_h), ctypes.c_float(eps),
-                                         -1 if kv_half is None else int(kv_half), _stream()))
+                                         int(units), _stream()))
 
 
 def aligned_columns(n_cached, n_new):
