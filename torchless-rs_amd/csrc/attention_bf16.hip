@@ -559,7 +559,10 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
 
 // Merge the splits of one (sequence, head): common maximum, weighted sums, in the order of the
 // splits.  (A second kernel and not the last workgroup of the first: what other XCDs wrote is
-// only sure to be seen across a kernel boundary without flushing L2 from inside the kernel.)
+// only sure to be seen across a kernel boundary or after a device-wide fence, and that fence
+// writes back and invalidates the XCD's L2.  Measured with the last workgroup merging behind a
+// counter: one fence a workgroup makes a step of 32 layers at batch 8 4.7 ms instead of 4.0, one
+// a thread 6.3.)
 // One wave per (row, head).  Splits are taken 8 at a time with all their loads (maxima, sums and
 // this lane's elements) issued together, so that a usual split count costs one trip to memory;
 // chunks merge by the running-maximum rule.
