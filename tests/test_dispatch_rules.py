@@ -14,6 +14,7 @@ def test_mid_splits_are_powers_of_two_that_fit():
     assert ops.mid_splits(64, 4096, 4096) == 8 and ops.mid_splits(64, 6144, 4096) == 8
     assert ops.mid_splits(128, 4096, 14336) == 8 and ops.mid_splits(64, 28672, 4096) == 1
     assert ops.mid_splits(20, 72, 48) == 1                  # one step of K: nothing to cut
+    assert ops.mid_splits(64, 5120, 14336) == 16 and ops.mid_splits(64, 5120, 14336, units=320) == 8   # whole rounds of workgroups
 
 
 def test_decode_splits_follow_batch_and_length():

@@ -68,7 +68,7 @@ class Linear:
         them up, where that pays (17..MID_ROWS rows and K worth cutting); else None."""
         if not self.mid(a):
             return None
-        S = ops.mid_splits(a.shape[0], self.out_features, self.in_features)
+        S = ops.mid_splits(a.shape[0], self.out_features, self.in_features, ops.compute_units(a.device))
         if S == 1:
             return None
         parts = ctx.workspace.get(name, (S, a.shape[0], self.out_features), torch.float32)
