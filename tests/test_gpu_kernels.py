@@ -402,6 +402,26 @@ def test_gemm_bf16_kernels(ops, variant, M, N, K):
     assert rel_err(acc, want + base.double()) < 3e-6
 
 
+@pytest.mark.parametrize("share", [5, 16, 17, 20, 31, 32])
+@pytest.mark.parametrize("M,N,K", [(1, 50, 72), (7, 130, 264), (16, 200, 1000), (3, 384, 96)])
+def test_gemm_bf16_in_shares_of_any_size(ops, share, M, N, K):
+    """The kernel for at most 16 rows with `share` channels a workgroup (the launcher's way of giving
+    every compute unit as much to read as the others): the bits of 16 channels a workgroup."""
+    a = rnd(M, K, seed=21, dtype=torch.bfloat16).to(DEV)
+    w = rnd(N, K, seed=22, dtype=torch.bfloat16).to(DEV)
+    want = torch.full((M, N), float("nan"), device=DEV)
+    ops.gemm_bf16(a, w, want, variant=112)
+    out = torch.full((M, N), float("nan"), device=DEV)
+    ops.gemm_bf16(a, w, out, variant=1000 + share)
+    assert torch.equal(out, want)
+    base = rnd(M, N, seed=23).to(DEV)
+    acc, acc_want = base.clone(), base.clone()
+    ops.gemm_bf16(a, w, acc, accumulate=True, variant=1000 + share)
+    ops.gemm_bf16(a, w, acc_want, accumulate=True, variant=112)
+    assert torch.equal(acc, acc_want)
+    assert rel_err(out, a.double().cpu() @ w.double().cpu().t()) < 3e-6
+
+
 def test_gemm_bf16_row_does_not_depend_on_the_batch(ops):
     a = rnd(64, 512, seed=24, dtype=torch.bfloat16).to(DEV)
     w = rnd(96, 512, seed=25, dtype=torch.bfloat16).to(DEV)
@@ -642,7 +662,7 @@ def test_qkv_rope_commit_equals_product_then_rope_commit(ops, nq, nkv, d, K, len
 # ---- an RMSNorm cut in two around products of at most 16 rows ----------------------------
 
 @pytest.mark.parametrize("M", [1, 5, 16])
-@pytest.mark.parametrize("N,K,N2", [(200, 72, 50), (64, 264, 16384), (1000, 96, 130), (4616, 72, 48)])   # the last: more than 256 workgroups wrote
+@pytest.mark.parametrize("N,K,N2", [(200, 72, 50), (64, 264, 16384), (1000, 96, 130), (4616, 72, 48), (8296, 40, 48)])   # the last two: more tiles of 16 channels than compute units, in one round of workgroups and in two
 def test_gemm_norm_halves(ops, M, N, K, N2):
     """The product that completes the stream writes x * w and its workgroups' sums of x^2;
     the product that reads them applies rsqrt(mean + eps): together the plain norm between."""
@@ -741,7 +761,7 @@ def test_tile_weights(ops, N, K):
 
 
 @pytest.mark.parametrize("M", [1, 7, 16])
-@pytest.mark.parametrize("N,K", [(16, 64), (48, 192), (4112, 320), (96, 4096)])
+@pytest.mark.parametrize("N,K", [(16, 64), (48, 192), (4112, 320), (96, 4096), (8208, 128)])
 def test_products_from_the_tiled_copy_give_the_same_bits(ops, M, N, K):
     """The same values meet in the same MFMAs in the same order, wherever they were read from."""
     a = rnd(M, K, seed=63, dtype=torch.bfloat16).to(DEV)

@@ -1028,7 +1028,8 @@ extern "C" int tl_gemm_bf16(const void* A, const void* W, const void* Wt, void* 
   return 0;
 }
 
-// For tests and tuning: force one kernel whatever M is.  variant 0: tiled; 1: big; 2: rows; else NT*100 + MT*10 + waves/4.
+// For tests and tuning: force one kernel whatever M is.  variant 0: tiled; 1: big; 2: rows; 1000 + R: the kernel for at
+// most 16 rows with R channels a workgroup (1 to 32); else NT*100 + MT*10 + waves/4.
 extern "C" int tl_gemm_bf16_variant(const void* A, const void* W, void* C, int M, int N, int K,
                                     int epilogue, int variant, hipStream_t st) {
   TL_REQUIRE(M > 0 && N > 0 && K > 0 && K % 8 == 0, "gemm_bf16: bad sizes M=%d N=%d K=%d", M, N, K);
@@ -1049,7 +1050,7 @@ extern "C" int tl_gemm_bf16_variant(const void* A, const void* W, void* C, int M
                K, ROWS_CHUNK);
     return launch_rows(a, w, c, M, N, K, epilogue, st);
   }
-  if (variant >= 1000 && variant <= 1032) {            // 1000 + channels a workgroup, at most 16 rows
+  if (variant > 1000 && variant <= 1032) {
     TL_REQUIRE(M <= 16 && epilogue != EPI_SILU_PAIR, "gemm_skinny: variant %d takes at most 16 rows and no pairs", variant);
     const int R = variant - 1000;
     if (R <= 16) return launch_skinny<1, 1, 8>(a, w, c, M, N, K, epilogue, st, NormSplit{}, nullptr, R);

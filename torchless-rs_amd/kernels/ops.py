@@ -370,7 +370,7 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: b
     rows come in groups of 64 (32 gate rows and the 32 up rows that belong to
     them) and out is bfloat16 [M, N/2] = silu(gate) * up.  `variant` (tests
     and tuning) forces one kernel.  `tiles`: `tile_weights(w)`, read instead of
-    w by the kernel for at most 16 rows and 16 channels a workgroup."""
+    w by the kernel for at most 16 rows and 16 to 32 channels a workgroup."""
     M, K = a.shape
     N = w.shape[0]
     _req(a, "gemm.a", torch.bfloat16)
