@@ -46,6 +46,14 @@ def test_a_failed_run_is_an_error_line_and_exit_1(tmp_path, capsys):
     assert err.startswith("Error: ") and "Traceback" not in err
 
 
+def test_default_number_of_new_tokens_follows_the_context():
+    """src/main.rs:140-153: a quarter of the context, clamped to 1024 (2048 from 4096 on) .. 32768."""
+    from torchless_rs_amd.api import default_max_tokens
+    assert default_max_tokens(2048) == 1024 and default_max_tokens(4095) == 1024
+    assert default_max_tokens(4096) == 2048 and default_max_tokens(32768) == 8192
+    assert default_max_tokens(1 << 20) == 32768
+
+
 def test_ids_and_sampling_names():
     assert parse_ids("1, 5 17") == [1, 5, 17]
     assert SamplingConfig().temperature == 1.0                            # sampler/mod.rs:46-54

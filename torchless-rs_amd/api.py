@@ -31,17 +31,30 @@ def generate_until_eos(engine: Engine, prompts: Sequence[Sequence[int]], config:
                      max_batch, on_token)
 
 
-def generate(model_dir: str, prompts: Sequence[Sequence[int]], max_tokens: int = 16,
+def default_max_tokens(max_seq_len: int) -> int:
+    """The tokens to generate when the caller names no number: a quarter of the context, at
+    least 1024 (2048 from a context of 4096 on) and at most 32768 (`resolve_max_tokens`,
+    src/main.rs:140-153 of the reference)."""
+    low = 2048 if max_seq_len >= 4096 else 1024
+    return min(max(max_seq_len // 4, low), 32768)
+
+
+def generate(model_dir: str, prompts: Sequence[Sequence[int]], max_tokens: Optional[int] = None,
              temperature: float = 0.7, top_k: Optional[int] = None, top_p: Optional[float] = None,
              seed: int = 0, stop_ids: Optional[Sequence[int]] = None, dtype: str = "bfloat16",
              max_seq_len: Optional[int] = None, device: str = "cuda:0",
              freeze_gc: bool = False) -> List[GenerationResult]:
     """Load the model folder and generate for every prompt.  `stop_ids` None
-    means config.json's eos_token_id, if it has one.  The engine made for the call is closed
+    means config.json's eos_token_id, if it has one; `max_tokens` None means `default_max_tokens`
+    of the context, cut to the room behind the longest prompt.  The engine made for the call is closed
     when it ends, its cache given back.  `freeze_gc`: see `Engine`."""
     model = load_model(model_dir, dtype, device)
     if stop_ids is None:
         stop_ids = list(getattr(model.config, "eos_token_ids", []) or [])
+    if max_tokens is None:
+        # the reference's default, and no more than the context has room for behind the longest prompt
+        context = max_seq_len or getattr(model.config, "max_position_embeddings", None) or 4096
+        max_tokens = max(1, min(default_max_tokens(context), context - max(len(p) for p in prompts)))
     longest = max(len(p) for p in prompts) + max_tokens
     # the longest sequence allowed: the model's max_position_embeddings unless the caller sets
     # another limit, which may exceed it with a warning (src/main.rs:111-137 of the reference)

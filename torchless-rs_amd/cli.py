@@ -22,9 +22,10 @@ from typing import List, Optional
 USAGE = """Usage: {prog} [OPTIONS] <model_path> [prompt]
 
 Options:
-  --max-tokens <N>      Maximum tokens to generate per prompt (default: 16)
+  --max-tokens <N>      Maximum tokens to generate per prompt (default: a quarter of
+                        --max-seq-len, from 1024 to 32768, within the context's room)
   --max-seq-len <N>     Maximum sequence length / context window
-                        (default: the prompt plus --max-tokens)
+                        (default: the model's max_position_embeddings)
   --temperature <T>     Sampling temperature (default: 0.7)
                         0.0 = greedy/deterministic, 0.7 = balanced, 1.0+ = creative
   --top-k <K>           Top-k sampling: only consider the top K tokens
@@ -129,7 +130,7 @@ def main(argv: Optional[List[str]] = None, prog: str = "torchless") -> int:
         return 1
     stop = opts["--stop-ids"]
     stop_ids = None if stop is None else ([] if stop.strip().lower() == "none" else parse_ids(stop))
-    max_tokens = 16 if opts["--max-tokens"] is None else opts["--max-tokens"]
+    max_tokens = opts["--max-tokens"]            # None: the default follows the context (api.default_max_tokens)
 
     from .api import generate
     t0 = time.time()
