@@ -367,8 +367,10 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
   const int p = row_pos[b];
   const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
   const int pg_lo = lo / PAGE, pg_hi = p / PAGE, n_pg = pg_hi - pg_lo + 1;
-  const int per = (n_pg + n_splits - 1) / n_splits;
-  const int my_lo = pg_lo + split * per, my_hi = min(pg_hi + 1, my_lo + per);   // [my_lo, my_hi)
+  // [my_lo, my_hi): the pages in shares that differ by one at most (65 pages in 8 splits are 8 or 9 each,
+  // not seven times 9 and once 2: the compute units then end together)
+  const int my_lo = pg_lo + (int)((long long)split * n_pg / n_splits);
+  const int my_hi = pg_lo + (int)((long long)(split + 1) * n_pg / n_splits);
   const size_t head_elems = (size_t)PAGE * d, page_elems = 2 * (size_t)nkv * head_elems;
 
   bf16x8 qreg[KB];
