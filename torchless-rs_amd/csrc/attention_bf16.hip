@@ -362,7 +362,6 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
   const int split = blockIdx.y;
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64, li = lane % 16, kg = lane / 16;
   const int hl = hg * 16 + li;                        // head within the KV group (column of S^T)
-  const bool h_ok = hl < g;
   const int h = kvh * g + min(hl, g - 1);
   const int p = row_pos[b];
   const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
