@@ -20,8 +20,14 @@ def test_mid_splits_are_powers_of_two_that_fit():
 def test_decode_splits_follow_batch_and_length():
     assert ops.decode_groups(8, 32, 8) == 64 and ops.decode_groups(1, 34, 2) == 4      # 17 heads a group: two tiles
     assert ops.decode_splits(64, 32, 8, 32) == 1            # enough workgroups without a cut
-    assert ops.decode_splits(8, 32, 8, 65) == 8             # 64 groups: eight parts reach 512 workgroups
+    assert ops.decode_splits(32, 32, 8, 65) == 1            # one workgroup a compute unit already
+    assert ops.decode_splits(8, 32, 8, 65) == 4             # 64 groups: four parts are one workgroup a unit
+    assert ops.decode_splits(16, 32, 8, 65) == 2
+    assert ops.decode_splits(3, 32, 8, 65) == 10            # 24 groups: 11 parts would start a second round
+    assert ops.decode_splits(20, 32, 8, 65) == 3            # 160 groups: two rounds of thirds beat one of wholes
     assert ops.decode_splits(1, 32, 8, 64) == 16            # at least four pages a part
+    assert ops.decode_splits(1, 32, 8, 513) == 31           # a long context: one round of workgroups, 17 pages each
+    assert ops.decode_splits(8, 32, 8, 65, units=128) == 2  # by the device's compute units
     assert ops.decode_splits(1, 32, 8, 1) == 1
     for B in (1, 3, 8, 64):
         for pages in (1, 4, 5, 64, 1100):

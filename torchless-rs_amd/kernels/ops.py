@@ -9,6 +9,7 @@ library nothing here runs.
 from __future__ import annotations
 
 import ctypes
+import functools
 from typing import Optional
 
 import torch
@@ -710,16 +711,26 @@ def decode_groups(B: int, nq: int, nkv: int) -> int:
     return B * nkv * (-(-(nq // nkv) // 16))
 
 
-SPLIT_TARGET = 512          # workgroups a decode step's attention aims at
 SPLIT_PAGES = 4             # fewest pages a part of the keys has
+SPLIT_COST = 0.15           # what a part more costs in the merge, in pages of a workgroup's way
 
 
-def decode_splits(B: int, nq: int, nkv: int, max_pages: int) -> int:
-    """Into how many parts the keys of a decode step are cut so that the chip
-    has some two workgroups a compute unit to run, each with at least
-    four pages (measured: more parts cost more in the merge than they gain)."""
-    groups = decode_groups(B, nq, nkv)
-    return max(1, min(-(-max_pages // SPLIT_PAGES), -(-SPLIT_TARGET // groups), 4096))
+@functools.lru_cache(maxsize=4096)
+def _decode_splits(groups: int, max_pages: int, units: int) -> int:
+    most = max(1, min(-(-max_pages // SPLIT_PAGES), -(-4 * units // groups), 4096))
+    # rounds of workgroups over the compute units x pages a workgroup goes through, and the merge
+    cost = lambda s: -(-groups * s // units) * -(-max_pages // s) + SPLIT_COST * s
+    return min(range(1, most + 1), key=lambda s: (cost(s), s))
+
+
+def decode_splits(B: int, nq: int, nkv: int, max_pages: int, units: int = 256) -> int:
+    """Into how many parts the keys of a decode step are cut.  A compute unit streams at a rate of
+    its own, so the step's attention takes as long as the unit with the most to read: rounds of
+    workgroups over the `units` compute units times the pages a workgroup has, plus the merge's
+    share for every part.  Eight sequences with eight KV heads each are 4 parts (256 workgroups,
+    one a unit: 3.91 ms a step against 3.96 with 8 parts and 4.08 with 6); parts have at least
+    four pages."""
+    return _decode_splits(decode_groups(B, nq, nkv), int(max_pages), int(units))
 
 
 def uses_transposed_values(dtype: torch.dtype, d: int, all_single: bool) -> bool:
@@ -739,7 +750,7 @@ def attention(q, k_new, v_new, pages, table, ring_pages: int, ctx, n_cached, win
     fast = q.dtype == torch.bfloat16 and d % 16 == 0 and 16 <= d <= 256
     if fast and k_new is None and ctx.all_single:
         nkv = pages.shape[2]
-        splits = decode_splits(n, nq, nkv, table.shape[1])      # by the table's width: fixed while a graph lives
+        splits = decode_splits(n, nq, nkv, table.shape[1], compute_units(q.device))      # by the table's width: fixed while a graph lives
         part = ctx.workspace.get("attn_part", (n * nq * splits * (d + 2),), torch.float32)
         attn_decode_bf16(q, pages, table, ring_pages, ctx.row_pos, window, scale, splits, part, out)
     elif fast and k_new is not None and vt_new is not None:
