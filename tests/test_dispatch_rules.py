@@ -28,6 +28,7 @@ def test_decode_splits_follow_batch_and_length():
     assert ops.decode_splits(1, 32, 8, 64) == 16            # at least four pages a part
     assert ops.decode_splits(1, 32, 8, 513) == 31           # a long context: one round of workgroups, 17 pages each
     assert ops.decode_splits(8, 32, 8, 65, units=128) == 2  # by the device's compute units
+    assert ops.decode_splits(8, 32, 8, 65, head_dim=64) == 8 and ops.decode_splits(32, 16, 4, 64, head_dim=32) == 8   # small heads: more workgroups a unit
     assert ops.decode_splits(1, 32, 8, 1) == 1
     for B in (1, 3, 8, 64):
         for pages in (1, 4, 5, 64, 1100):

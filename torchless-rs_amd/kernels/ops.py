@@ -723,14 +723,16 @@ def _decode_splits(groups: int, max_pages: int, units: int) -> int:
     return min(range(1, most + 1), key=lambda s: (cost(s), s))
 
 
-def decode_splits(B: int, nq: int, nkv: int, max_pages: int, units: int = 256) -> int:
+def decode_splits(B: int, nq: int, nkv: int, max_pages: int, units: int = 256, head_dim: int = 128) -> int:
     """Into how many parts the keys of a decode step are cut.  A compute unit streams at a rate of
     its own, so the step's attention takes as long as the unit with the most to read: rounds of
     workgroups over the `units` compute units times the pages a workgroup has, plus the merge's
     share for every part.  Eight sequences with eight KV heads each are 4 parts (256 workgroups,
     one a unit: 3.91 ms a step against 3.96 with 8 parts and 4.08 with 6); parts have at least
-    four pages."""
-    return _decode_splits(decode_groups(B, nq, nkv), int(max_pages), int(units))
+    four pages.  With heads of 64 or less a workgroup has too few bytes under way to keep a unit
+    busy alone, and a round is two workgroups a unit (four with heads of 32: 32 sequences of 4 KV
+    heads of 32 take 19.2 us in 4 parts, 27.2 in 2)."""
+    return _decode_splits(decode_groups(B, nq, nkv), int(max_pages), int(units) * max(1, 128 // max(1, int(head_dim))))
 
 
 def uses_transposed_values(dtype: torch.dtype, d: int, all_single: bool) -> bool:
@@ -750,7 +752,7 @@ def attention(q, k_new, v_new, pages, table, ring_pages: int, ctx, n_cached, win
     fast = q.dtype == torch.bfloat16 and d % 16 == 0 and 16 <= d <= 256
     if fast and k_new is None and ctx.all_single:
         nkv = pages.shape[2]
-        splits = decode_splits(n, nq, nkv, table.shape[1], compute_units(q.device))      # by the table's width: fixed while a graph lives
+        splits = decode_splits(n, nq, nkv, table.shape[1], compute_units(q.device), d)   # by the table's width: fixed while a graph lives
         part = ctx.workspace.get("attn_part", (n * nq * splits * (d + 2),), torch.float32)
         attn_decode_bf16(q, pages, table, ring_pages, ctx.row_pos, window, scale, splits, part, out)
     elif fast and k_new is not None and vt_new is not None:
