@@ -2,14 +2,17 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 8192] [--layers L]
                     [--shape 7b-v0.1|7b-v0.3|nemo-12b] [--only decode|prefill] [--prefill-tokens T]
-                    [--no-points] [--no-tiled-copies]
+                    [--no-points] [--no-kernels] [--no-workloads] [--no-tiled-copies]
 
 One JSON line: decoded tokens a second of the default run (batch 8 at the
 context length of the configuration), the prefill of one 2,048-token prompt,
-the decode step's share of the HBM roofline, decoding at batch 1 and 64, and
-what a plain read and a chain of MFMAs reach on the machine ("ceilings").
-Weights are random (seeded), token ids synthetic.  The context is built by a
-real prefill of synthetic prompts.
+the decode step's share of the HBM roofline, decoding at batch 1 and 64
+("points"), the step's kernels one by one with their own shares of the HBM
+roofline ("kernels"), the baseline's configurations as it words them, run
+through the generation loop ("workloads"), and what a plain read and a chain
+of MFMAs reach on the machine ("ceilings").  Weights are random (seeded),
+token ids synthetic.  The context is built by a real prefill of synthetic
+prompts.
 """
 from __future__ import annotations
 
@@ -48,12 +51,14 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None, help="fewer layers than the shape has")
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 and 64")
+    ap.add_argument("--no-kernels", action="store_true", help="skip the timing of the step's kernels one by one")
+    ap.add_argument("--no-workloads", action="store_true", help="skip the baseline's configurations as it words them")
     ap.add_argument("--no-tiled-copies", action="store_true",
                     help="keep no second copies of q|k|v, o and down in the layout that single-token steps stream")
-    ap.add_argument("--workload", choices=["baseline"], default=None,
-                    help="also run the baseline's configurations as it words them (unequal prompt lengths drawn "
-                         "from a seed, 256/128/128 new tokens, temperature 0.7 for the NeMo shape) through the "
-                         "generation loop, and add their figures under 'workloads'")
+    ap.add_argument("--workload", choices=["baseline"], default="baseline",
+                    help="the baseline's configurations as it words them (unequal prompt lengths drawn from a seed, "
+                         "256/128/128 new tokens, temperature 0.7 for the NeMo shape) run through the generation "
+                         "loop, under 'workloads' (the default; --no-workloads skips them)")
     ap.add_argument("--only", choices=["prefill", "decode"], default=None,
                     help="measure one phase only and print its line to stderr (for profiling)")
     args = ap.parse_args()
@@ -65,6 +70,7 @@ def main() -> int:
     from torchless_rs_amd import SamplingConfig, config_from_dict
     from torchless_rs_amd.engine import Engine, SeqInput, model_from_tensors
     from torchless_rs_amd.engine.generate import BatchRun
+    from torchless_rs_amd.kernels.page import PAGE, round_up
     from torchless_rs_amd.models import model_spec_for
     from torchless_rs_amd.sampling.sampler import Sampler
     from torchless_rs_amd.weights import random_tensors
@@ -92,11 +98,12 @@ def main() -> int:
     sampler = Sampler(SamplingConfig.greedy(), dev)
     gen = torch.Generator().manual_seed(11)
 
-    def run_decode(batch: int, context: int, steps: int, warmup: int, engine=None):
+    def run_decode(batch: int, context: int, steps: int, warmup: int, engine=None, then=None):
         """Prefill `batch` prompts of `context - steps - warmup` tokens, then time `steps` decode
-        steps (model step + greedy sampling)."""
+        steps (model step + greedy sampling).  `then(engine, slots)`: called after the timed steps
+        while the sequences are still held."""
         held = min(context, W) if W else context
-        eng = engine or Engine(model, max_tokens=batch * (-(-held // 64) * 64 + 64), max_slots=batch, freeze_gc=True)
+        eng = engine or Engine(model, max_tokens=batch * (round_up(held) + PAGE), max_slots=batch, freeze_gc=True)
         plen = max(1, context - steps - warmup - 1)
         slots = [eng.alloc() for _ in range(batch)]
         chunk = 2048
@@ -122,10 +129,95 @@ def main() -> int:
         torch.cuda.synchronize()
         dt = time.perf_counter() - t
         ctx_mid = plen + warmup + steps // 2
+        extra = then(eng, [run.slots[i] for i in range(batch)]) if then is not None else None
         run.release()
         if engine is None:
             eng.close()
-        return dt / steps, ctx_mid
+        return (dt / steps, ctx_mid) if then is None else (dt / steps, ctx_mid, extra)
+
+    def kernels_one_by_one(eng, slots):
+        """The kernels of one decode step, each kind by itself: one more step is run with every call
+        into the kernels' Python face noted (function and arguments, layer after layer), then the calls
+        of each kind are captured as a graph of their own (every layer's launch of that kernel, each on
+        its own weights and cache, so that nothing is warm that the step would not find warm) and the
+        graph is timed with events.  Bytes are what the kernel has to read once: its weight, or the
+        keys and values of the live sequences."""
+        from torchless_rs_amd.kernels import ops as K
+        names = ("embed", "rmsnorm", "add_rmsnorm", "qkv_rope_commit", "rope_commit", "attention", "gemm_bf16_norm",
+                 "gemm_bf16", "gemm_mid_bf16", "gemm", "gemm_library", "add_partials", "gather_rows", "silu_mul_pairs")
+        real = {n: getattr(K, n) for n in names}
+        tape = []
+        depth = [0]
+
+        def noted(name):
+            def call(*a, **k):
+                if depth[0] == 0:               # (a face that calls another face counts once)
+                    tape.append((name, a, k))
+                depth[0] += 1
+                try:
+                    return real[name](*a, **k)
+                finally:
+                    depth[0] -= 1
+            return call
+
+        use_graphs, eng.use_graphs = eng.use_graphs, False
+        for n in names:
+            setattr(K, n, noted(n))
+        try:
+            ctx, want_rows, n_want = eng.build_context([SeqInput(s, [0], [0]) for s in slots])
+            eng.model.forward(ctx, eng.runs, want_rows, n_want)
+        finally:
+            for n, f in real.items():
+                setattr(K, n, f)
+            eng.use_graphs = use_graphs
+        torch.cuda.synchronize()
+        held_rows = sum(min(int(n), W) if W else int(n) for n in ctx.host["len_after"])
+
+        def kind_and_bytes(name, a, k):
+            if name == "attention":
+                return "attention", held_rows * 2 * nkv * d * 2
+            w = next((t for t in a[:3] if isinstance(t, torch.Tensor) and t.dim() == 2 and t.dtype == torch.bfloat16
+                      and t.shape[0] > 64), None)
+            if name in ("qkv_rope_commit", "gemm_bf16_norm", "gemm_bf16", "gemm_mid_bf16", "gemm", "gemm_library") and w is not None:
+                label = {(nq + 2 * nkv) * d: "qkv", 2 * I: "gate_up", V: "head"}.get(w.shape[0])
+                if label is None:
+                    label = "o" if w.shape[1] == nq * d else "down"
+                if name == "qkv_rope_commit":
+                    label = "qkv_rope_commit"
+                return label, w.numel() * 2
+            return name, 0
+
+        kinds = {}
+        for name, a, k in tape:
+            kind, nbytes = kind_and_bytes(name, a, k)
+            kinds.setdefault(kind, {"calls": [], "bytes": 0})
+            kinds[kind]["calls"].append((real[name], a, k))
+            kinds[kind]["bytes"] += nbytes
+        out, total = {}, 0.0
+        side = torch.cuda.Stream()
+        for kind, rec in kinds.items():
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                for f, a, k in rec["calls"]:
+                    f(*a, **k)
+            torch.cuda.synchronize()
+            best = float("inf")
+            for _ in range(5):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                graph.replay()
+                e1.record()
+                e1.synchronize()
+                best = min(best, e0.elapsed_time(e1) * 1e3)
+            n = len(rec["calls"])
+            out[f"{kind}_us"] = round(best / n, 2)
+            out[f"{kind}_calls"] = n
+            if rec["bytes"]:
+                out[f"{kind}_frac"] = round(rec["bytes"] / (best * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)
+            total += best
+            del graph
+        out["sum_us"] = round(total, 1)
+        return out
 
     def run_workload(mdl, mcfg, n_layers, batch, lo, hi, new_tokens, temperature, seed):
         """`batch` requests with prompt lengths uniform in [lo, hi] and `new_tokens` new tokens each,
@@ -137,7 +229,7 @@ def main() -> int:
         prompts = [torch.randint(0, mcfg.vocab_size, (n,), generator=g).tolist() for n in lens]
         win = mcfg.sliding_window
         held = [min(n + new_tokens, win) if win else n + new_tokens for n in lens]
-        eng = Engine(mdl, max_tokens=sum(-(-h // 64) * 64 + 64 for h in held), max_slots=batch, freeze_gc=True)
+        eng = Engine(mdl, max_tokens=sum(round_up(h) + PAGE for h in held), max_slots=batch, freeze_gc=True)
         scfg = SamplingConfig(temperature=temperature, seed=seed) if temperature > 0 else SamplingConfig.greedy()
         stamps = []
 
@@ -176,7 +268,7 @@ def main() -> int:
 
     # prefill of one prompt
     T = args.prefill_tokens
-    eng = Engine(model, max_tokens=T + 64, max_slots=1, freeze_gc=True)
+    eng = Engine(model, max_tokens=T + PAGE, max_slots=1, freeze_gc=True)
     ids = torch.randint(0, V, (T,), generator=gen).tolist()
     pre_ms = []
     for it in range(2):
@@ -197,7 +289,12 @@ def main() -> int:
     if args.only == "prefill":
         return 0
 
-    sec, ctx_mid = run_decode(args.batch, args.context, args.steps, args.warmup)
+    if args.no_kernels:
+        (sec, ctx_mid), kernels = run_decode(args.batch, args.context, args.steps, args.warmup), {}
+    else:
+        sec, ctx_mid, kernels = run_decode(args.batch, args.context, args.steps, args.warmup, then=kernels_one_by_one)
+        kernels["step_us"] = round(sec * 1e6, 1)
+        print(f"[bench] kernels of the step one by one {kernels}", file=sys.stderr, flush=True)
     held = min(ctx_mid, W) if W else ctx_mid
     step_bytes = weight_bytes + args.batch * held * kv_per_token
     achieved = step_bytes / sec / 1e9
@@ -207,12 +304,12 @@ def main() -> int:
     points = {}
     if not args.no_points:
         for b in (1, 64):
-            s_b, _ = run_decode(b, args.context, max(8, args.steps // 2), 2)
+            s_b, _ = run_decode(b, args.context, max(32, args.steps), 4)
             points[f"decode_b{b}"] = round(b / s_b, 1)
             print(f"[bench] decode b{b}: {b / s_b:.1f} tok/s", file=sys.stderr, flush=True)
 
     workloads = {}
-    if args.workload == "baseline":
+    if args.workload == "baseline" and not args.no_workloads:
         if args.shape == "7b-v0.1":                     # the model that is loaded: prompts U[128, 2048], 256 new tokens
             for b in (1, 8, 64):
                 workloads[f"7b-v0.1_b{b}"] = run_workload(model, cfg, L, b, 128, 2048, 256, 0.0, seed=5)
@@ -259,8 +356,13 @@ def main() -> int:
         "points": points,
         "ceilings": ceilings,
     }
+    if kernels:
+        out["kernels"] = kernels
     if workloads:
-        out["workloads"] = workloads
+        # flat: decoded and prefilled tokens a second and the decode steps' share of the HBM roofline
+        out["workloads"] = {f"{k}_{f}": v[f] for k, v in workloads.items()
+                            for f in ("decode_tok_s", "prefill_tok_s", "roofline_frac")}
+        out["workload_details"] = workloads
     print(json.dumps(out), flush=True)
     return 0
 

@@ -89,7 +89,7 @@ def softmax(s: torch.Tensor) -> torch.Tensor:
     return e / e.sum(dim=-1, keepdim=True)
 
 
-def attention_core(q, k, v, positions, window) -> torch.Tensor:
+def attention_core(q, k, v, positions, window, scale=None) -> torch.Tensor:
     """q[T,nq,d], k,v[T,nkv,d] (already rotated) -> ctx[T,nq,d].
     Query head h reads KV head h // (nq/nkv); score = (k.q) * 1/sqrt(d),
     scale applied after the dot; softmax over the visible keys; weighted sum
@@ -98,7 +98,8 @@ def attention_core(q, k, v, positions, window) -> torch.Tensor:
     T, nq, d = q.shape
     nkv = k.shape[1]
     g = nq // nkv
-    scale = 1.0 / math.sqrt(d)
+    if scale is None:           # (another factor: only for parts that tests build with one)
+        scale = 1.0 / math.sqrt(d)
     mask = visible(positions, window)
     out = torch.empty_like(q)
     for h in range(nq):
@@ -283,7 +284,8 @@ def to_bf16(t: torch.Tensor) -> torch.Tensor:
     return t.to(torch.float32).to(torch.bfloat16).to(t.dtype)
 
 
-def forward_rounded(weights: dict, cfg: dict, ids, step_rows, library_rows=64) -> torch.Tensor:
+def forward_rounded(weights: dict, cfg: dict, ids, step_rows, library_rows=64, matrix_core_heads=None,
+                    ffn_norm_in_halves=True) -> torch.Tensor:
     """`forward` in float64 with a rounding to bfloat16 at every place where the engine's
     bfloat16 path stores one, and nowhere else: the output of a norm, q and k after the rotation,
     v, the probabilities as they enter the product with the values (their sum is taken
@@ -299,6 +301,11 @@ def forward_rounded(weights: dict, cfg: dict, ids, step_rows, library_rows=64) -
     (The kernels round a probability against the running maximum of the keys seen so far and
     scale float32 sums afterwards; here it is rounded against the row's maximum: another
     realisation of the same rounding.)
+    `matrix_core_heads` (default: the head size is a multiple of 16): with other head sizes the
+    engine's attention runs in its plain kernels, which keep the probabilities in float32, and
+    its q|k|v product cannot take a norm in halves, so the norm before it is stored whole.
+    `ffn_norm_in_halves`: false where the output projection or gate|up cannot do the halves
+    (heads x head size no multiple of 8, an inner size no multiple of 32).
     The formulas are those of the functions above; only the roundings are added."""
     f64 = torch.float64
     take = lambda name: weights[name].to(f64)            # a layer at a time, where the tensors lie
@@ -315,6 +322,9 @@ def forward_rounded(weights: dict, cfg: dict, ids, step_rows, library_rows=64) -
     nkv = cfg.get("num_key_value_heads") or nq
     d = cfg.get("head_dim") or cfg["hidden_size"] // nq
     theta = cfg.get("rope_theta", 10000.0)
+    if matrix_core_heads is None:
+        matrix_core_heads = d % 16 == 0
+    round_p = to_bf16 if matrix_core_heads else (lambda t: t)
 
     def normed(x, weight, may_split):
         """(input of the products, factor on their results)"""
@@ -328,7 +338,7 @@ def forward_rounded(weights: dict, cfg: dict, ids, step_rows, library_rows=64) -
     for i in range(cfg["num_hidden_layers"]):
         p = f"model.layers.{i}."
         w = {p + n: take(p + n) for n in LAYER_TENSORS}
-        y, r = normed(x, w[p + "input_layernorm.weight"], i > 0)
+        y, r = normed(x, w[p + "input_layernorm.weight"], i > 0 and matrix_core_heads)
         q = (linear(y, w[p + "self_attn.q_proj.weight"]) * r).view(T, nq, d)
         k = (linear(y, w[p + "self_attn.k_proj.weight"]) * r).view(T, nkv, d)
         v = (linear(y, w[p + "self_attn.v_proj.weight"]) * r).view(T, nkv, d)
@@ -340,9 +350,9 @@ def forward_rounded(weights: dict, cfg: dict, ids, step_rows, library_rows=64) -
             s = (q[:, h, :] @ k[:, kvh, :].t()) * (1.0 / math.sqrt(d))
             s = s.masked_fill(~mask, float("-inf"))
             e = torch.exp(s - s.max(dim=-1, keepdim=True).values)
-            ctx[:, h, :] = (to_bf16(e) @ v[:, kvh, :]) / e.sum(dim=-1, keepdim=True)
+            ctx[:, h, :] = (round_p(e) @ v[:, kvh, :]) / e.sum(dim=-1, keepdim=True)
         x = x + linear(to_bf16(ctx).reshape(T, nq * d), w[p + "self_attn.o_proj.weight"])
-        y, r = normed(x, w[p + "post_attention_layernorm.weight"], True)
+        y, r = normed(x, w[p + "post_attention_layernorm.weight"], ffn_norm_in_halves)
         g = linear(y, w[p + "mlp.gate_proj.weight"]) * r
         u = linear(y, w[p + "mlp.up_proj.weight"]) * r
         g, u = torch.where(pre_round, to_bf16(g), g), torch.where(pre_round, to_bf16(u), u)

@@ -46,3 +46,25 @@ def test_a_shared_folder_under_tmp_is_not_trusted(tmp_path):
     os.chmod(mine, 0o777)
     assert not build._own_private_dir(str(mine))
     assert not build._own_private_dir(str(tmp_path / "absent"))
+
+
+def test_a_current_library_in_the_private_folder_goes_before_a_stale_one_in_the_package(tmp_path, monkeypatch):
+    """A package folder that cannot be written keeps its stale library for good; the current one that an
+    earlier process built into the private folder must be found, not built again by every process."""
+    pkg, private = tmp_path / "pkg", tmp_path / "private"
+    pkg.mkdir()
+    private.mkdir(mode=0o700)
+    monkeypatch.setattr(build, "build_dirs", lambda: [str(pkg), str(private)])
+    stale, fresh = str(pkg / "lib.so"), str(private / "lib.so")
+    open(stale, "w").close()
+    build._write_stamp(stale, "old")
+    assert build.built_library("lib.so", "new") == stale          # nothing current anywhere: the first found
+    open(fresh, "w").close()
+    build._write_stamp(fresh, "new")
+    assert build.built_library("lib.so", "new") == fresh
+    assert build.built_library("lib.so") == stale                  # without a digest: the order of preference
+    assert build.built_library("lib.so", "old") == stale
+    os.chmod(private, 0o777)                                        # a folder others can write to is never looked into
+    assert build.built_library("lib.so", "new") == stale
+    os.remove(stale)
+    assert build.built_library("lib.so", "new") is None

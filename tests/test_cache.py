@@ -188,3 +188,28 @@ def test_a_closed_cache_gives_its_storage_back_and_refuses_use():
     with pytest.raises(CacheMisuse, match="closed"):
         c.alloc_slot()
     c.close()                                               # twice is harmless
+
+
+def test_every_view_of_a_closed_cache_refuses_use():
+    """The views kept on a cache (slots, lengths, a group's pool and its pages by slot) reach the host
+    library through the same checked handle as the cache: after `close` each raises, none hands the
+    library a null handle."""
+    c = make(two_groups=True)
+    s = c.alloc_slot()
+    c.prepare([(s, 70)])
+    c.commit([(s, 70)])
+    slots, length, group = c.slots, c.length, c.groups[0]
+    c.close()
+    touches = [
+        lambda: slots.n_free, lambda: slots.n_held, lambda: slots.holds(s),
+        lambda: length[s], lambda: len(length), lambda: s in length, lambda: list(length), lambda: length.values(),
+        lambda: group.pool.n_free, lambda: group.pool.n_held, lambda: group.pool.holds(0),
+        lambda: group.pages_of_slot[s], lambda: s in group.pages_of_slot, lambda: len(group.pages_of_slot),
+        lambda: list(group.pages_of_slot),
+        lambda: c.held_slots(), lambda: c.fits([10]), lambda: c.prepare([(s, 1)]), lambda: c.commit([(s, 1)]),
+        lambda: c.free_slot(s), lambda: c.check(), lambda: c.tokens_held(),
+    ]
+    for i, touch in enumerate(touches):
+        with pytest.raises(CacheMisuse, match="closed"):
+            touch()
+            pytest.fail(f"touch {i} went through")

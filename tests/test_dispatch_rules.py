@@ -6,33 +6,33 @@ def test_mid_splits_are_powers_of_two_that_fit():
     for M in (17, 64, 128):
         for N in (72, 4096, 6144, 28672, 32000):
             for K in (48, 256, 1000, 4096, 14336):
-                S = ops.mid_splits(M, N, K)
+                S = ops.mid_splits(M, N, K, 256)
                 steps = -(-K // 256)
                 assert S >= 1 and S & (S - 1) == 0, (M, N, K, S)
                 assert S <= max(1, steps) and S <= 16, (M, N, K, S)
     # the 7B sizes: narrow outputs are cut in 8, the wide one is not cut
-    assert ops.mid_splits(64, 4096, 4096) == 8 and ops.mid_splits(64, 6144, 4096) == 8
-    assert ops.mid_splits(128, 4096, 14336) == 8 and ops.mid_splits(64, 28672, 4096) == 1
-    assert ops.mid_splits(20, 72, 48) == 1                  # one step of K: nothing to cut
-    assert ops.mid_splits(64, 5120, 14336) == 16 and ops.mid_splits(64, 5120, 14336, units=320) == 8   # whole rounds of workgroups
+    assert ops.mid_splits(64, 4096, 4096, 256) == 8 and ops.mid_splits(64, 6144, 4096, 256) == 8
+    assert ops.mid_splits(128, 4096, 14336, 256) == 8 and ops.mid_splits(64, 28672, 4096, 256) == 1
+    assert ops.mid_splits(20, 72, 48, 256) == 1                  # one step of K: nothing to cut
+    assert ops.mid_splits(64, 5120, 14336, 256) == 16 and ops.mid_splits(64, 5120, 14336, units=320) == 8   # whole rounds of workgroups
 
 
 def test_decode_splits_follow_batch_and_length():
     assert ops.decode_groups(8, 32, 8) == 64 and ops.decode_groups(1, 34, 2) == 4      # 17 heads a group: two tiles
-    assert ops.decode_splits(64, 32, 8, 32) == 1            # enough workgroups without a cut
-    assert ops.decode_splits(32, 32, 8, 65) == 1            # one workgroup a compute unit already
-    assert ops.decode_splits(8, 32, 8, 65) == 4             # 64 groups: four parts are one workgroup a unit
-    assert ops.decode_splits(16, 32, 8, 65) == 2
-    assert ops.decode_splits(3, 32, 8, 65) == 10            # 24 groups: 11 parts would start a second round
-    assert ops.decode_splits(20, 32, 8, 65) == 3            # 160 groups: two rounds of thirds beat one of wholes
-    assert ops.decode_splits(1, 32, 8, 64) == 16            # at least four pages a part
-    assert ops.decode_splits(1, 32, 8, 513) == 31           # a long context: one round of workgroups, 17 pages each
-    assert ops.decode_splits(8, 32, 8, 65, units=128) == 2  # by the device's compute units
-    assert ops.decode_splits(8, 32, 8, 65, head_dim=64) == 8 and ops.decode_splits(32, 16, 4, 64, head_dim=32) == 8   # small heads: more workgroups a unit
-    assert ops.decode_splits(1, 32, 8, 1) == 1
+    assert ops.decode_splits(64, 32, 8, 32, 256, 128) == 1            # enough workgroups without a cut
+    assert ops.decode_splits(32, 32, 8, 65, 256, 128) == 1            # one workgroup a compute unit already
+    assert ops.decode_splits(8, 32, 8, 65, 256, 128) == 4             # 64 groups: four parts are one workgroup a unit
+    assert ops.decode_splits(16, 32, 8, 65, 256, 128) == 2
+    assert ops.decode_splits(3, 32, 8, 65, 256, 128) == 10            # 24 groups: 11 parts would start a second round
+    assert ops.decode_splits(20, 32, 8, 65, 256, 128) == 3            # 160 groups: two rounds of thirds beat one of wholes
+    assert ops.decode_splits(1, 32, 8, 64, 256, 128) == 16            # at least four pages a part
+    assert ops.decode_splits(1, 32, 8, 513, 256, 128) == 31           # a long context: one round of workgroups, 17 pages each
+    assert ops.decode_splits(8, 32, 8, 65, 128, 128) == 2  # by the device's compute units
+    assert ops.decode_splits(8, 32, 8, 65, 256, 64) == 8 and ops.decode_splits(32, 16, 4, 64, 256, 32) == 8   # small heads: more workgroups a unit
+    assert ops.decode_splits(1, 32, 8, 1, 256, 128) == 1
     for B in (1, 3, 8, 64):
         for pages in (1, 4, 5, 64, 1100):
-            S = ops.decode_splits(B, 32, 8, pages)
+            S = ops.decode_splits(B, 32, 8, pages, 256, 128)
             assert 1 <= S <= max(1, -(-pages // ops.SPLIT_PAGES))
 
 

@@ -14,7 +14,8 @@ import torch
 
 import plain_mistral as plain
 from test_gpu_kernels import philox_uniform
-from util import CONFIGS, TOL, make_model_dir, prompts, read_model_dir, rel_err, within_the_format
+from util import (CONFIGS, TOL, held_to_the_format, make_model_dir, prompts, read_model_dir, rel_err,
+                  within_the_format)
 
 pytestmark = pytest.mark.gpu
 REPO = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -58,11 +59,14 @@ def engine_for(zoo, name, dtype, poison=True):
 def test_each_request_alone_and_whole(zoo, name, dtype):
     from torchless_rs_amd.engine import SeqInput
     eng, z = engine_for(zoo, name, dtype), zoo[name]
+    gots = []
     for p, want in zip(z["prompts"], z["want"]):
         s = eng.alloc()
         got = eng.step([SeqInput(s, p, list(range(len(p))))]).clone()
         eng.free(s)
         assert rel_err(got, want) < TOL[dtype], (name, dtype, len(p))
+        gots.append(got)
+    held_to_the_format(dtype, gots, z["want"], z["w"], z["cfg"], z["prompts"], [[len(p)] * len(p) for p in z["prompts"]])
     eng.cache.check()
 
 
@@ -71,6 +75,7 @@ def test_each_request_alone_and_whole(zoo, name, dtype):
 def test_last_32_one_by_one(zoo, name, dtype):
     from torchless_rs_amd.engine import SeqInput
     eng, z = engine_for(zoo, name, dtype), zoo[name]
+    gots, rows = [], []
     for p, want in zip(z["prompts"], z["want"]):
         k = min(32, len(p) - 1)
         s = eng.alloc()
@@ -82,6 +87,9 @@ def test_last_32_one_by_one(zoo, name, dtype):
             outs.append(eng.step([SeqInput(s, [t], [0])]).clone())
         eng.free(s)
         assert rel_err(torch.cat(outs), want) < TOL[dtype], (name, dtype, len(p))
+        gots.append(torch.cat(outs))
+        rows.append([len(p) - k] * (len(p) - k) + [1] * k)
+    held_to_the_format(dtype, gots, z["want"], z["w"], z["cfg"], z["prompts"], rows)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -118,6 +126,9 @@ def test_unequal_batches_one_after_another(zoo, name, dtype):
             live = [i for i in live if fed[i] < len(ps[i])]
         for i, want in enumerate(wants):
             assert rel_err(torch.cat(got[i]), want) < TOL[dtype], (name, dtype, heads, i)
+        tails = [len(p) - h for p, h in zip(ps, heads)]
+        rows = [[sum(heads)] * h + [sum(1 for t2 in tails if t < t2) for t in range(tl)] for h, tl in zip(heads, tails)]
+        held_to_the_format(dtype, [torch.cat(g) for g in got], wants, z["w"], z["cfg"], ps, rows, heads)
         eng.cache.check()
     assert used[0] == used[1] == used[2]
 
@@ -388,6 +399,7 @@ def test_random_schedules(zoo, name, dtype, seed):
     seqs = prompts(V, lengths, seed=90 + seed)
     want = [plain.forward(z["w"], z["cfg"], p) for p in seqs]
     waiting, live, fed, got = list(range(len(seqs))), {}, {}, {i: [] for i in range(len(seqs))}
+    rows = {i: [] for i in range(len(seqs))}
     step = 0
     while waiting or live:
         while waiting and len(live) < 4:
@@ -402,15 +414,18 @@ def test_random_schedules(zoo, name, dtype, seed):
             batch.append(SeqInput(live[i], seqs[i][fed[i]:fed[i] + n], list(range(n))))
             fed[i] += n
         lg = eng.step(batch).clone()
-        r = 0
+        r, n_rows = 0, sum(len(e.tokens) for e in batch)
         for i, e in zip(chosen, batch):
             got[i].append(lg[r:r + len(e.tokens)])
+            rows[i] += [n_rows] * len(e.tokens)
             r += len(e.tokens)
             if fed[i] == len(seqs[i]):
                 eng.free(live.pop(i))
         eng.cache.check()
     for i in range(len(seqs)):
         assert rel_err(torch.cat(got[i]), want[i]) < TOL[dtype], i
+    held_to_the_format(dtype, [torch.cat(got[i]) for i in range(len(seqs))], want, z["w"], z["cfg"], seqs,
+                       [rows[i] for i in range(len(seqs))])
     assert not eng.cache.length
 
 

@@ -82,12 +82,12 @@ def test_7b_shape_at_full_depth():
     heads = [n - t for n, t in zip(LENS, TAILS)]
     rows_whole = [[n] * n for n in LENS]
     rows_batch = [[sum(heads)] * h + [sum(1 for t2 in TAILS if t < t2) for t in range(tl)] for h, tl in zip(heads, TAILS)]
-    for name, rows, want in (("whole", rows_whole, exact[:2]), ("batch", rows_batch, exact[:2])):
-        rounded = [plain.forward_rounded(tensors, SHAPE, p, r) for p, r in zip(ids, rows)]
+    rows_again = rows_batch[::-1]                  # the second batch: lengths and tails in the other order
+    for name, rows, want, reqs in (("whole", rows_whole, exact[:2], ids), ("batch", rows_batch, exact[:2], ids),
+                                   ("again", rows_again, exact[2:], others)):
+        rounded = [plain.forward_rounded(tensors, SHAPE, p, r) for p, r in zip(reqs, rows)]
         ok, numbers = within_the_format(b[name], rounded, want)
         print(f"   bfloat16 {name}: " + ", ".join(f"{k} {v:.2e}" for k, v in numbers.items()))
         assert ok, (name, numbers)
-    again = max(rel_err(g, x) for g, x in zip(b["again"], exact[2:]))
-    first = max(rel_err(g, x) for g, x in zip(b["batch"], exact[:2]))
-    print(f"   bfloat16 second batch in the same slots {again:.2e}, first {first:.2e}")
-    assert again < 2 * first + 1e-3
+    # (the second batch, in the slots and pages that the first gave back, is held to the plain rounded
+    # implementation of its own requests like the others: a stale row worth the format's cost would show)

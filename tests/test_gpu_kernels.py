@@ -386,8 +386,7 @@ def test_draws_do_not_depend_on_batch_mates_and_follow_the_probabilities(ops):
 # ---- bfloat16 products on the matrix cores -----------------------------------------
 
 @pytest.mark.parametrize("variant,M", [(112, 1), (112, 7), (111, 16), (212, 3), (411, 5), (222, 17), (222, 32),
-                                       (421, 20), (242, 33), (441, 64), (142, 50), (0, 1), (0, 70), (0, 128),
-                                       (0, 300), (1, 3), (1, 129), (1, 300), (1, 600)])
+                                       (421, 20), (242, 33), (441, 64), (142, 50)])
 @pytest.mark.parametrize("N,K", [(50, 72), (16, 64), (130, 264), (200, 1000), (384, 96)])
 def test_gemm_bf16_kernels(ops, variant, M, N, K):
     a = rnd(M, K, seed=21, dtype=torch.bfloat16)
@@ -432,10 +431,10 @@ def test_gemm_bf16_row_does_not_depend_on_the_batch(ops):
         outs[M] = o
     for M in outs:
         assert torch.equal(outs[M][0], outs[64][0])
-    big = torch.empty(64, 96, device=DEV)
-    ops.gemm_bf16(a, w, big, variant=0)
-    assert rel_err(big, outs[64]) < 1e-6                    # the tiled kernel agrees up to rounding
     assert rel_err(outs[64], a.double().cpu() @ w.double().cpu().t()) < 3e-6
+    more = torch.empty(65, 96, device=DEV)
+    with pytest.raises(ops.KernelError, match="at most 64"):      # more rows are not this entry point's
+        ops.gemm_bf16(torch.cat([a, a[:1]]).contiguous(), w, more)
 
 
 def test_gemm_dispatch_falls_back_when_k_is_odd(ops):
@@ -543,7 +542,7 @@ def test_attention_bf16_far_key_and_edge(ops):
         assert torch.isfinite(out2).all()
 
 
-@pytest.mark.parametrize("variant,M", [(411, 1), (411, 9), (421, 30), (441, 64), (0, 5), (0, 200), (1, 7), (1, 520)])
+@pytest.mark.parametrize("variant,M", [(411, 1), (411, 9), (421, 30), (441, 64)])
 @pytest.mark.parametrize("I,K", [(64, 72), (160, 64), (96, 200)])
 def test_gemm_bf16_paired_silu_epilogue(ops, variant, M, I, K):
     """gate and up rows interleaved in groups of 32: the product writes silu(gate) * up."""
@@ -578,8 +577,8 @@ def test_gemm_library_products(ops, M, N, K):
     ops.gemm(a.to(DEV), w.to(DEV), acc, accumulate=True)
     assert rel_err(acc, want + base.double()) < 3e-6
     ours = torch.empty(M, N, device=DEV)
-    ops.gemm_bf16(a.to(DEV), w.to(DEV), ours)
-    assert rel_err(ours, out) < 1e-6                         # our kernel agrees up to rounding
+    ops.gemm_plain(a.to(DEV), w.to(DEV), ours)
+    assert rel_err(ours, out) < 1e-6                         # the plain kernel agrees up to rounding
     o16 = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
     ops.gemm_library(a.to(DEV), w.to(DEV), o16)
     assert rel_err(o16, want) < KTOL["bfloat16"]
@@ -949,9 +948,15 @@ def test_rope_commit_adds_partial_products(ops):
 
 
 def test_ceilings_are_measured(ops):
-    """The plain read and the MFMA chain that bench.py quotes run and give sane figures."""
-    c = ops.measure_ceilings(DEV, gib=0.25)
-    assert 100.0 < c["hbm_read_GBs"] < 20000.0 and 50.0 < c["mfma_bf16_TFLOPs"] < 5000.0
+    """The plain read (in every shape), the copy and the MFMA chain that bench.py quotes: on an MI355X the
+    best read reaches at least 5 of the published 8 TB/s and the chain 1.8 of 2.5 PFLOP/s, and neither
+    exceeds the published peak; a figure outside means that the measurement is broken, not the machine."""
+    c = ops.measure_ceilings(DEV, gib=2.0)
+    assert 5000.0 <= c["hbm_read_GBs"] <= 8000.0, c
+    assert c["hbm_read_shape"] in ops.READ_SHAPES.values() and len(c["hbm_read_by_shape_GBs"]) == len(ops.READ_SHAPES)
+    assert all(1000.0 < v <= 8000.0 for v in c["hbm_read_by_shape_GBs"].values()), c
+    assert 3000.0 <= c["hbm_copy_GBs"] <= 8000.0, c
+    assert 1800.0 <= c["mfma_bf16_TFLOPs"] <= 2500.0, c
 
 
 @pytest.mark.parametrize("window", [None, 4096])

@@ -688,3 +688,169 @@ def test_a_toy_mixer_whose_values_are_wider_than_its_keys():
         eng.close()
     finally:
         unregister_part("mixer", "wide_values")
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("d", [32, 40])         # on the matrix cores, and on the plain kernels (no multiple of 16)
+def test_attention_part_with_a_scale_of_its_own(dt, d):
+    """The factor on the scores is a parameter of the mixer (default 1/sqrt(head size)) that reaches all
+    three attention kernels: whole rows (prefill), single tokens (decode), and the plain kernel.  The
+    factor here is six times the default one, so that taking the default shows far above the tolerance."""
+    from torchless_rs_amd.cache import Cache
+    from torchless_rs_amd.engine import SeqInput
+    from torchless_rs_amd.parts import PartSpec, RunBinding, make_part
+    from torchless_rs_amd.parts.base import flush_pending
+    H, nq, nkv, n, scale = 48, 4, 2, 70, 6.0 / math.sqrt(d)
+    mixer = make_part("mixer", PartSpec("attention", {
+        "hidden_size": H, "n_heads": nq, "n_kv_heads": nkv, "head_dim": d, "window": None, "scale": scale,
+        "position": PartSpec("rotary", {"head_dim": d, "theta": 300.0})}))
+    assert make_part("mixer", PartSpec("attention", {"hidden_size": H, "n_heads": nq, "n_kv_heads": nkv, "head_dim": d,
+                                                     "position": PartSpec("none", {})})).scale == 1 / math.sqrt(d)
+    w = {"self_attn.q_proj.weight": rnd(nq * d, H, seed=1, scale=0.3, dtype=DT[dt]),
+         "self_attn.k_proj.weight": rnd(nkv * d, H, seed=2, scale=0.3, dtype=DT[dt]),
+         "self_attn.v_proj.weight": rnd(nkv * d, H, seed=3, scale=0.3, dtype=DT[dt]),
+         "self_attn.o_proj.weight": rnd(H, nq * d, seed=4, scale=0.3, dtype=DT[dt])}
+    mixer.load({k: v.to(DEV) for k, v in w.items()}, DT[dt])
+    y = rnd(n, H, seed=9, dtype=DT[dt])
+    wd = {k: v.double() for k, v in w.items()}
+    pos = torch.arange(n)
+    q = plain.rope(plain.linear(y.double(), wd["self_attn.q_proj.weight"]).view(n, nq, d), pos, 300.0)
+    k = plain.rope(plain.linear(y.double(), wd["self_attn.k_proj.weight"]).view(n, nkv, d), pos, 300.0)
+    v = plain.linear(y.double(), wd["self_attn.v_proj.weight"]).view(n, nkv, d)
+    want = plain.linear(plain.attention_core(q, k, v, pos, None, scale=scale).reshape(n, nq * d), wd["self_attn.o_proj.weight"])
+    default = plain.linear(plain.attention_core(q, k, v, pos, None).reshape(n, nq * d), wd["self_attn.o_proj.weight"])
+    assert rel_err(default, want) > 0.1
+    cache = Cache({0: mixer.kv_request()}, {}, 64 * 3, DT[dt], DEV, 1)
+    cache.groups[0].storage.fill_(float("nan"))
+    run = RunBinding(index=0, kv_group=cache.groups[0], kv_group_index=0, kv_layer=0, kv_source=0)
+    s = cache.alloc_slot()
+    got = []
+    for rows in [40] + [1] * 30:
+        o = sum(g.shape[0] for g in got)
+        ctx = context(cache, [SeqInput(s, [0] * rows, [])], DT[dt])
+        x = torch.zeros(rows, H, device=DEV)
+        mixer.forward(ctx, run, y[o:o + rows].to(DEV), x)
+        flush_pending(ctx, x)
+        cache.commit([(s, rows)])
+        got.append(x.clone())
+    assert rel_err(torch.cat(got), want) < PTOL[dt]
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_a_block_of_another_arrangement_gets_the_split_norms_from_the_helpers(dt):
+    """A layer with three norms and two feed-forwards, x += mixer(n1 x); x += ffn(n2 x); x += ffn_b(n3 x),
+    defined here as a block part around the framework's parts with the three helpers of parts/base
+    (`read_through_norm`, `expect_norm`, `part_done`).  In bfloat16 single-token steps its norms then run
+    cut in two around the products like those of the framework's own block: no norm kernel inside or
+    between layers (counted), and the logits are those of the plain composition."""
+    from torchless_rs_amd.engine import Engine, SeqInput
+    from torchless_rs_amd.engine.model import Model
+    from torchless_rs_amd.kernels import ops
+    from torchless_rs_amd.parts import LayerSpec, Part, PartSpec, make_part, register_part, unregister_part
+    from torchless_rs_amd.parts.base import expect_norm, part_done, read_through_norm, splittable_entry
+    from torchless_rs_amd.weights import TensorDict, random_tensors
+    H, V, I, Ib, nq, nkv, d, L, eps = 128, 80, 192, 96, 4, 2, 32, 2, 1e-5
+
+    class ThreeNorms(Part):
+        def __init__(self, layer, ffn_b, norm_b):
+            self.mixer, self.ffn = make_part("mixer", layer.mixer), make_part("ffn", layer.ffn)
+            self.n1, self.n2 = make_part("norm", layer.mixer_norm), make_part("norm", layer.ffn_norm)
+            self.ffn_b, self.n3 = make_part("ffn", ffn_b), make_part("norm", norm_b)
+            self.parts = (self.mixer, self.ffn, self.ffn_b, self.n1, self.n2, self.n3)
+            self.graph_safe = all(p.graph_safe for p in self.parts)
+
+        def may_capture(self, n_rows):
+            return all(p.may_capture(n_rows) for p in self.parts)
+
+        def weight_specs(self):
+            out = {}
+            for name, norm in (("ln_a.", self.n1), ("ln_b.", self.n2), ("ln_c.", self.n3)):
+                out.update({name + k: v for k, v in norm.weight_specs().items()})
+            for part in (self.mixer, self.ffn, self.ffn_b):
+                out.update(part.weight_specs())
+            return out
+
+        def load(self, tensors, compute_dtype):
+            for name, norm in (("ln_a.", self.n1), ("ln_b.", self.n2), ("ln_c.", self.n3)):
+                norm.load({k[len(name):]: v for k, v in tensors.items() if k.startswith(name)}, compute_dtype)
+            for part in (self.mixer, self.ffn, self.ffn_b):
+                part.load(tensors, compute_dtype)
+
+        def entry_norm(self):
+            return splittable_entry(self.n1, self.mixer)
+
+        def forward(self, ctx, run, x, norm_after=None):
+            y = ctx.workspace.get("block_y", tuple(x.shape), ctx.dtype)
+            y1 = read_through_norm(ctx, self.n1, x, y)
+            expect_norm(ctx, self.mixer, self.n2, self.ffn)
+            self.mixer.forward(ctx, run, y1, x)
+            part_done(ctx, self.mixer)
+            y2 = read_through_norm(ctx, self.n2, x, y)
+            expect_norm(ctx, self.ffn, self.n3, self.ffn_b)
+            self.ffn.forward(ctx, y2, x)
+            part_done(ctx, self.ffn)
+            y3 = read_through_norm(ctx, self.n3, x, y)
+            expect_norm(ctx, self.ffn_b, norm_after)
+            self.ffn_b.forward(ctx, y3, x)
+            part_done(ctx, self.ffn_b)
+
+    register_part("block", "three_norms", ThreeNorms)
+    calls = []
+    real = {name: getattr(ops, name) for name in ("rmsnorm", "add_rmsnorm")}
+    try:
+        norm = PartSpec("rmsnorm", {"size": H, "eps": eps})
+        block = PartSpec("three_norms", {"ffn_b": PartSpec("swiglu", {"hidden_size": H, "intermediate_size": Ib, "prefix": "mlp_b."}),
+                                         "norm_b": norm})
+        layers = [LayerSpec(prefix=f"model.layers.{i}.",
+                            mixer=PartSpec("attention", {"hidden_size": H, "n_heads": nq, "n_kv_heads": nkv, "head_dim": d,
+                                                         "window": 24, "position": PartSpec("rotary", {"head_dim": d, "theta": 100.0})}),
+                            ffn=PartSpec("swiglu", {"hidden_size": H, "intermediate_size": I}),
+                            mixer_norm=norm, ffn_norm=norm, block=block) for i in range(L)]
+        spec = _toy_model(layers, H, V, eps)
+        assert "model.layers.1.ln_c.weight" in spec.weight_specs() and "model.layers.1.mlp_b.down_proj.weight" in spec.weight_specs()
+        w = random_tensors(spec.weight_specs(), seed=31, std=0.08, norm_std=0.1, dtype=torch.bfloat16)
+        model = Model(spec, None, DT[dt], DEV)
+        model.load_weights(TensorDict(w))
+        eng = Engine(model, max_tokens=64 * 4, use_graphs=False)
+
+        def plain_forward(ids):
+            wd = {k: v.double() for k, v in w.items()}
+            pos = torch.arange(len(ids))
+            cfg = {"num_attention_heads": nq, "num_key_value_heads": nkv, "head_dim": d, "hidden_size": H,
+                   "rope_theta": 100.0, "sliding_window": 24}
+            x = wd["model.embed_tokens.weight"][ids]
+            for i in range(L):
+                p = f"model.layers.{i}."
+                x = x + plain.attention(plain.rmsnorm(x, wd[p + "ln_a.weight"], eps), wd, p, cfg, pos)
+                x = x + plain.swiglu(plain.rmsnorm(x, wd[p + "ln_b.weight"], eps), wd, p)
+                wb = {p + "mlp." + k: wd[p + "mlp_b." + k] for k in ("gate_proj.weight", "up_proj.weight", "down_proj.weight")}
+                x = x + plain.swiglu(plain.rmsnorm(x, wd[p + "ln_c.weight"], eps), wb, p)
+            return plain.linear(plain.rmsnorm(x, wd["model.norm.weight"], eps), wd["lm_head.weight"])
+
+        g = torch.Generator().manual_seed(32)
+        seqs = [torch.randint(0, V, (n,), generator=g).tolist() for n in (50, 7)]
+        wants = [plain_forward(s) for s in seqs]
+        tol = {"float32": 2e-5, "bfloat16": 3e-2}[dt]
+        slots = [eng.alloc() for _ in seqs]
+        heads = [30, 3]
+        lg = eng.step([SeqInput(sl, s[:h], list(range(h))) for sl, s, h in zip(slots, seqs, heads)]).clone()
+        assert rel_err(lg[:30], wants[0][:30]) < tol and rel_err(lg[30:], wants[1][:3]) < tol
+        for name in real:
+            setattr(ops, name, lambda *a, _n=name, **k: (calls.append(_n), real[_n](*a, **k))[1])
+        for t in range(20):
+            live = [i for i in range(2) if heads[i] + t < len(seqs[i])]
+            calls.clear()
+            lg = eng.step([SeqInput(slots[i], [seqs[i][heads[i] + t]], [0]) for i in live]).clone()
+            for r, i in enumerate(live):
+                assert rel_err(lg[r:r + 1], wants[i][heads[i] + t:heads[i] + t + 1]) < tol, (t, i)
+            if dt == "bfloat16":
+                # the first norm of the first layer (behind the embedding, which is no product) and the
+                # last norm on the gathered rows: the 3 L - 1 norms between them ran inside the products
+                assert calls == ["rmsnorm", "rmsnorm"], calls
+            else:
+                assert len(calls) == 3 * L + 1
+        eng.close()
+    finally:
+        for name, fn in real.items():
+            setattr(ops, name, fn)
+        unregister_part("block", "three_norms")

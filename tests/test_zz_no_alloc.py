@@ -92,3 +92,46 @@ def test_static_scratch_entry_point_refuses_what_does_not_fit():
     assert "static scratch holds" in lib.tl_last_error().decode()
     torch.cuda.synchronize()
     assert (out == 0).all()
+
+
+def test_static_scratch_entry_point_under_graph_capture():
+    """After the set-up call (made outside capture) a call may be captured into a HIP graph: every
+    replay, with the program's own eager work and synchronizations between them and with other inputs
+    written into the same tensors, gives the bits of the eager call."""
+    from torchless_rs_amd.kernels import ops
+    lib = ops.lib()
+    assert lib.tl_static_scratch_ready() == 0, lib.tl_last_error().decode()
+    c = _case(5, 8, 2, 128, None, [130, 700, 64, 65, 1], seed=21)
+    other = _case(5, 8, 2, 128, None, [130, 700, 64, 65, 1], seed=22)      # same shapes, other values
+    B, nq, d, splits = c["B"], c["nq"], c["d"], 3
+    q, pages, table = c["q"].clone(), c["pages"].clone(), c["table"].clone()
+    out = torch.zeros(B, nq, d, dtype=torch.bfloat16, device=DEV)
+
+    def call(stream):
+        rc = lib.tl_attn_decode_bf16_static(_ptr(q), _ptr(pages), _ptr(table), table.shape[1], c["ring"],
+                                            _ptr(c["row_pos"]), B, nq, c["nkv"], d, c["window"],
+                                            ctypes.c_float(c["scale"]), splits, _ptr(out),
+                                            ctypes.c_void_p(stream.cuda_stream))
+        assert rc == 0, lib.tl_last_error().decode()
+
+    eager = {}
+    for name, src in (("a", c), ("b", other)):
+        q.copy_(src["q"]); pages.copy_(src["pages"]); table.copy_(src["table"])
+        call(torch.cuda.current_stream())
+        torch.cuda.synchronize()
+        eager[name] = out.clone()
+    assert not torch.equal(eager["a"], eager["b"])
+    graph = torch.cuda.CUDAGraph()
+    q.copy_(c["q"]); pages.copy_(c["pages"]); table.copy_(c["table"])
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph):
+        call(torch.cuda.current_stream())
+    for name in ("a", "b", "b", "a", "a"):
+        src = c if name == "a" else other
+        q.copy_(src["q"]); pages.copy_(src["pages"]); table.copy_(src["table"])
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager[name]), name
+        # the array is shared: an eager call between the replays, with its own output, disturbs nothing
+        _both(lib, _case(2, 6, 1, 48, 100, [40, 333], seed=12), 2)

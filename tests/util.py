@@ -67,6 +67,22 @@ def within_the_format(got, rounded, exact):
     return ok, dict(rms=rms, rms_of_roundings=rms_cost, largest=top, largest_of_roundings=top_cost)
 
 
+def held_to_the_format(dtype, got, exact, w, cfg, ids, step_rows, what=""):
+    """The stricter of the measures for a schedule's logits (lists, one tensor a request): float32
+    within the fixed tolerance; bfloat16 within what the format costs the plain implementation that
+    rounds where the engine does, on these very requests cut into these very steps (`step_rows`:
+    for every position the number of rows of the step it came in), so that a stale or misplaced row
+    of little weight, far below the fixed tolerance, still shows."""
+    import plain_mistral as plain
+    if dtype == "float32":
+        worst = max(rel_err(g, x) for g, x in zip(got, exact))
+        assert worst < TOL[dtype], (what, worst)
+        return
+    rounded = [plain.forward_rounded(w, cfg, p, r) for p, r in zip(ids, step_rows)]
+    ok, numbers = within_the_format(got, rounded, exact)
+    assert ok, (what, numbers)
+
+
 def make_model_dir(tmp, name: str, dtype=torch.bfloat16) -> str:
     from torchless_rs_amd import write_random_model
     d = os.path.join(str(tmp), f"tiny_{name}_{str(dtype).split('.')[-1]}")

@@ -68,7 +68,8 @@ def generate(model_dir: str, prompts: Sequence[Sequence[int]], max_tokens: Optio
         raise ValueError(f"a request needs {longest} positions, " +
                          (f"--max-seq-len allows {limit}" if max_seq_len is not None else
                           f"the model's max_position_embeddings is {limit}; raise --max-seq-len to go beyond"))
-    per_seq = -(-longest // 64) * 64
+    from .kernels.page import round_up
+    per_seq = round_up(longest)
     engine = Engine(model, max_tokens=per_seq * len(prompts), max_slots=len(prompts), freeze_gc=freeze_gc)
     try:
         cfg = SamplingConfig(temperature=temperature, top_k=top_k, top_p=top_p, seed=seed)

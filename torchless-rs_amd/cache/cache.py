@@ -33,10 +33,10 @@ import ctypes
 
 import numpy as np
 
+from ..kernels.page import PAGE                  # noqa: F401  (positions in a page: csrc/page.h)
 from . import native
 from .native import CacheFull, CacheMisuse      # noqa: F401
 
-PAGE = 64
 NO_RING = 1 << 24          # "ring" of a group that keeps every position: never wraps
 
 
@@ -76,11 +76,21 @@ class _Books:
     def __init__(self, max_slots: int, n_pages: int, rings, pages):
         self.max_slots, self.n_pages = int(max_slots), int(n_pages)
         rings, pages = _ints(rings), _ints(pages)
-        self.h = ctypes.c_void_p(native.lib().tl_books_new(self.max_slots, len(rings), rings.ctypes.data,
-                                                           pages.ctypes.data))
+        self._handle = ctypes.c_void_p(native.lib().tl_books_new(self.max_slots, len(rings), rings.ctypes.data,
+                                                                 pages.ctypes.data))
+
+    @property
+    def h(self):
+        """The handle of the books in the host library, for every call into it: the cache and all
+        its views (slots, lengths, pools, pages of a slot) come through here, so that none of
+        them hands the library a null handle once the cache is closed."""
+        h = getattr(self, "_handle", None)
+        if h is None:
+            raise CacheMisuse("the cache is closed")
+        return h
 
     def close(self) -> None:
-        h, self.h = getattr(self, "h", None), None
+        h, self._handle = getattr(self, "_handle", None), None
         if h:
             try:
                 native.lib().tl_books_delete(h)
@@ -262,9 +272,7 @@ class Cache:
 
     @property
     def _h(self):
-        """The handle of the books in the host library."""
-        if self._books.h is None:
-            raise CacheMisuse("the cache is closed")
+        """The handle of the books in the host library (`CacheMisuse` once the cache is closed)."""
         return self._books.h
 
     def close(self) -> None:

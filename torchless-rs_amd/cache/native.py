@@ -57,6 +57,8 @@ def lib() -> ctypes.CDLL:
         l.tl_aligned_columns.restype = ctypes.c_long
         l.tl_pack_step.argtypes = [ctypes.c_void_p, ctypes.c_int] + [ctypes.c_void_p] * 5 + [ctypes.c_int] + \
             [ctypes.c_void_p] * 2 + [ctypes.c_long] + [ctypes.c_void_p] * 3
+        from ..kernels.page import require_same
+        require_same(l.tl_host_page(), "the host library")
         _lib = l
     return _lib
 

@@ -779,6 +779,8 @@ float* static_scratch() {
 
 extern "C" size_t tl_static_scratch_bytes(void) { return TL_STATIC_SCRATCH_BYTES; }
 
+extern "C" int tl_static_scratch_ready(void) { return static_scratch() == nullptr ? 2 : 0; }
+
 extern "C" int tl_attn_decode_bf16_static(const void* q, const void* pages, const int* table, int table_stride,
                                           int ring_pages, const int* row_pos, int B, int nq, int nkv, int d,
                                           int window, float scale, int n_splits, void* out, hipStream_t st) {

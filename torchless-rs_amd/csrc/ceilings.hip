@@ -26,6 +26,75 @@ stream_read_kernel(const f32x4* __restrict__ src, size_t n_vec, float* __restric
   if (threadIdx.x == 0) sink[blockIdx.x] = s;
 }
 
+// The same read in other shapes, to see whether the machine gives more to any of them: U loads
+// in flight a lane; SPAN: a workgroup reads one contiguous share of the buffer (U * 4 KB an
+// iteration) instead of pieces a grid stride apart; NT: loads marked non-temporal.
+template <int U, bool SPAN, bool NT>
+__global__ void __launch_bounds__(256)
+stream_read_shape_kernel(const f32x4* __restrict__ src, size_t n_vec, float* __restrict__ sink) {
+  size_t i, end, step, apart;
+  if (SPAN) {
+    const size_t share = (n_vec / gridDim.x) / (256 * U) * (256 * U);     // whole iterations; the rest is left unread
+    i = (size_t)blockIdx.x * share + threadIdx.x;
+    end = (size_t)(blockIdx.x + 1) * share;
+    step = (size_t)256 * U;
+    apart = 256;
+  } else {
+    apart = (size_t)gridDim.x * 256;
+    i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    end = n_vec;
+    step = apart * U;
+  }
+  f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (; i + (U - 1) * apart < end; i += step) {
+    f32x4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) v[u] = NT ? __builtin_nontemporal_load(src + i + u * apart) : src[i + u * apart];
+#pragma unroll
+    for (int u = 0; u < U; ++u) acc += v[u];
+  }
+  __shared__ float sh[4];
+  const float s = block_sum<256>(acc[0] + acc[1] + acc[2] + acc[3], sh);
+  if (threadIdx.x == 0) sink[blockIdx.x] = s;
+}
+
+// The read with the data going from memory straight into LDS (16 bytes a lane, no register in
+// between), U loads a wave under way; nothing reads the LDS but one value at the end.
+template <int U>
+__global__ void __launch_bounds__(256)
+stream_read_lds_kernel(const f32x4* __restrict__ src, size_t n_vec, float* __restrict__ sink) {
+  __shared__ __attribute__((aligned(16))) f32x4 buf[4][U][WAVE];
+  const int w = threadIdx.x / WAVE, l = threadIdx.x % WAVE;
+  const size_t apart = (size_t)gridDim.x * 256;
+  size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  for (; i + (U - 1) * apart < n_vec; i += apart * U) {
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + i + u * apart),
+                                       (__attribute__((address_space(3))) void*)&buf[w][u][0], 16, 0, 0);
+  }
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
+  const f32x4 v = buf[w][l % U][l];
+  if (v[0] == 12345.678f) sink[blockIdx.x] = v[1];      // never true in practice
+}
+
+// A copy: as many bytes written as read, a cross-check of the total traffic the memory takes.
+template <int U>
+__global__ void __launch_bounds__(256)
+stream_copy_kernel(const f32x4* __restrict__ src, f32x4* __restrict__ dst, size_t n_vec) {
+  const size_t apart = (size_t)gridDim.x * 256;
+  size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  for (; i + (U - 1) * apart < n_vec; i += apart * U) {
+    f32x4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) v[u] = src[i + u * apart];
+#pragma unroll
+    for (int u = 0; u < U; ++u) dst[i + u * apart] = v[u];
+  }
+  for (; i < n_vec; i += apart) dst[i] = src[i];
+}
+
 // Eight independent accumulators a wave, 32x32x16 bfloat16 MFMAs back to back.
 __global__ void __launch_bounds__(256)
 mfma_chain_kernel(int iters, float* __restrict__ sink) {
@@ -64,6 +133,40 @@ int tl_stream_read(const void* src, size_t n_bytes, float* sink, int blocks, hip
              n_bytes, blocks);
   stream_read_kernel<<<blocks, 256, 0, st>>>((const f32x4*)src, n_bytes / 16, sink);
   TL_LAUNCH_CHECK("stream_read");
+  return 0;
+}
+
+// The read in another shape (see the kernels): 1: 16 loads in flight a lane; 2: 32; 3: 8, a contiguous share a
+// workgroup; 4: 16, contiguous; 5: 8, non-temporal; 6: 16, non-temporal, contiguous; 7: 8 a wave straight into
+// LDS; 8: 16 a wave straight into LDS.  (0 is tl_stream_read's.)  The shapes read whole iterations only: up to
+// blocks * 256 * 32 * 16 bytes at the end are left out, which the caller's sizes make negligible.
+int tl_stream_read_shape(const void* src, size_t n_bytes, float* sink, int blocks, int shape, hipStream_t st) {
+  TL_REQUIRE(n_bytes % 16 == 0 && blocks > 0 && ((uintptr_t)src % 16 == 0), "stream_read: %zu bytes in %d blocks",
+             n_bytes, blocks);
+  const f32x4* s = (const f32x4*)src;
+  const size_t n = n_bytes / 16;
+  switch (shape) {
+    case 0: stream_read_kernel<<<blocks, 256, 0, st>>>(s, n, sink); break;
+    case 1: stream_read_shape_kernel<16, false, false><<<blocks, 256, 0, st>>>(s, n, sink); break;
+    case 2: stream_read_shape_kernel<32, false, false><<<blocks, 256, 0, st>>>(s, n, sink); break;
+    case 3: stream_read_shape_kernel<8, true, false><<<blocks, 256, 0, st>>>(s, n, sink); break;
+    case 4: stream_read_shape_kernel<16, true, false><<<blocks, 256, 0, st>>>(s, n, sink); break;
+    case 5: stream_read_shape_kernel<8, false, true><<<blocks, 256, 0, st>>>(s, n, sink); break;
+    case 6: stream_read_shape_kernel<16, true, true><<<blocks, 256, 0, st>>>(s, n, sink); break;
+    case 7: stream_read_lds_kernel<8><<<blocks, 256, 0, st>>>(s, n, sink); break;
+    case 8: stream_read_lds_kernel<16><<<blocks, 256, 0, st>>>(s, n, sink); break;
+    default: TL_REQUIRE(false, "stream_read: unknown shape %d", shape);
+  }
+  TL_LAUNCH_CHECK("stream_read_shape");
+  return 0;
+}
+
+// copies n_bytes (a multiple of 16) from src to dst, which must not overlap
+int tl_stream_copy(const void* src, void* dst, size_t n_bytes, int blocks, hipStream_t st) {
+  TL_REQUIRE(n_bytes % 16 == 0 && blocks > 0 && ((uintptr_t)src % 16 == 0) && ((uintptr_t)dst % 16 == 0),
+             "stream_copy: %zu bytes in %d blocks", n_bytes, blocks);
+  stream_copy_kernel<8><<<blocks, 256, 0, st>>>((const f32x4*)src, (f32x4*)dst, n_bytes / 16);
+  TL_LAUNCH_CHECK("stream_copy");
   return 0;
 }
 

@@ -5,6 +5,8 @@
 #include <stdint.h>
 #include <stdio.h>
 
+#include "page.h"
+
 namespace tl {
 
 typedef __bf16 bf16;
@@ -15,7 +17,8 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 
 constexpr int WAVE = 64;
-constexpr int PAGE = 64;          // positions per cache page
+constexpr int PAGE = TL_PAGE;     // positions per cache page
+static_assert(PAGE == 64, "the attention kernels tile a page by 64 positions");
 
 // dtype codes of the C interface
 constexpr int DT_F32 = 0;

@@ -485,6 +485,7 @@ using namespace tl;
 extern "C" {
 
 const char* tl_last_error() { return g_err; }
+int tl_page_size() { return PAGE; }      // what this library was compiled with (csrc/page.h)
 
 int tl_embed(const void* table, int table_dt, const int* ids, int n, int H, float* out,
              hipStream_t st) {

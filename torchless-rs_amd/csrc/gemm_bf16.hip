@@ -17,8 +17,8 @@
 //    single-token steps, with rotation and the write into the cache's pages.
 //  * gemm_mid: 17..128 rows.  The activations of a k-step are shared by the four
 //    waves through LDS; K may be cut over workgroups into partial sums.
-//  * gemm_tiled, gemm_big: more rows (prefill).  128x128x64 and 256x128x64 tiles
-//    staged through LDS, 32x32x16 MFMA, next tile prefetched into registers.
+// Products with more rows (prefill, large decode batches) are the BLAS library's, as the
+// reference hands its products to the vendor's library.
 //
 // All need K % 8 == 0 and 16-byte aligned rows; callers fall back to the
 // plain kernel otherwise.
@@ -730,262 +730,6 @@ static int launch_mid(const bf16* A, const bf16* W, float* C, int M, int N, int 
   return 0;
 }
 
-// ----------------------------------------------------------------- tiled ----
-constexpr int TM = 128, TN = 128, TK = 64, TPAD = 8, TLD = TK + TPAD;
-
-__global__ void __launch_bounds__(256)
-gemm_tiled_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float* __restrict__ C, int M,
-                  int N, int K, int epilogue) {
-  __shared__ __attribute__((aligned(16))) bf16 As[TM * TLD];
-  __shared__ __attribute__((aligned(16))) bf16 Ws[TN * TLD];
-  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
-  const int wm = (wave / 2) * 64, wn = (wave % 2) * 64;     // this wave's 64x64 corner in the tile
-  const int m0 = blockIdx.y * TM, n0 = blockIdx.x * TN;
-  const int l32 = lane % 32, kh = lane / 32;
-
-  // global -> register staging: 128 rows x 8 chunks of 8; thread takes chunk (tid%8) of rows tid/8 + 32*i
-  const int lc = (tid % 8) * 8, lr = tid / 8;
-  const bf16* ap[4];
-  const bf16* wp[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    ap[i] = A + (size_t)min(m0 + lr + 32 * i, M - 1) * K + lc;
-    wp[i] = W + (size_t)min(n0 + lr + 32 * i, N - 1) * K + lc;
-  }
-  bf16x8 ra[4], rw[4];
-  auto fetch = [&](int k0) {
-    const bool ok = k0 + lc + 8 <= K;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      ra[i] = ok ? load8(ap[i] + k0) : zero8();
-      rw[i] = ok ? load8(wp[i] + k0) : zero8();
-    }
-  };
-  auto stash = [&]() {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      *reinterpret_cast<bf16x8*>(&As[(lr + 32 * i) * TLD + lc]) = ra[i];
-      *reinterpret_cast<bf16x8*>(&Ws[(lr + 32 * i) * TLD + lc]) = rw[i];
-    }
-  };
-
-  f32x16 acc[2][2];
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-
-  fetch(0);
-  for (int k0 = 0; k0 < K; k0 += TK) {
-    __syncthreads();                 // everyone is done reading the previous tile
-    stash();
-    __syncthreads();
-    if (k0 + TK < K) fetch(k0 + TK);
-    // operands of the next 16 k are read from LDS while the MFMAs of these 16 run
-    bf16x8 a[2][2], b[2][2];
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      a[0][i] = *reinterpret_cast<const bf16x8*>(&As[(wm + 32 * i + l32) * TLD + 8 * kh]);
-      b[0][i] = *reinterpret_cast<const bf16x8*>(&Ws[(wn + 32 * i + l32) * TLD + 8 * kh]);
-    }
-#pragma unroll
-    for (int ks = 0; ks < TK / 16; ++ks) {
-      const int cur = ks & 1, nxt = cur ^ 1;
-      if (ks + 1 < TK / 16) {
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-          a[nxt][i] = *reinterpret_cast<const bf16x8*>(&As[(wm + 32 * i + l32) * TLD + (ks + 1) * 16 + 8 * kh]);
-          b[nxt][i] = *reinterpret_cast<const bf16x8*>(&Ws[(wn + 32 * i + l32) * TLD + (ks + 1) * 16 + 8 * kh]);
-        }
-      }
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[cur][i], b[cur][j], acc[i][j], 0, 0, 0);
-    }
-  }
-  // acc[i][j][r]: row = 8*(r/4) + 4*kh + r%4, column = l32 of the 32x32 block
-  if (epilogue == EPI_SILU_PAIR) {
-    // the wave's 64 columns are one group: block j=0 gate, block j=1 up
-    bf16* H = reinterpret_cast<bf16*>(C);
-    const int NH = N / 2;
-    const int n = (n0 + wn) / 2 + l32;
-    if (n < NH) {
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int m = m0 + wm + 32 * i + 8 * (r / 4) + 4 * kh + (r % 4);
-          if (m < M) {
-            const float g = acc[i][0][r], u = acc[i][1][r];
-            H[(size_t)m * NH + n] = (bf16)((g / (1.0f + expf(-g))) * u);
-          }
-        }
-    }
-    return;
-  }
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int n = n0 + wn + 32 * j + l32;
-      if (n >= N) continue;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int m = m0 + wm + 32 * i + 8 * (r / 4) + 4 * kh + (r % 4);
-        if (m < M) {
-          float* c = C + (size_t)m * N + n;
-          *c = (epilogue == EPI_ACCUMULATE) ? *c + acc[i][j][r] : acc[i][j][r];
-        }
-      }
-    }
-}
-
-// ------------------------------------------------------------------- big ----
-// 256x128x64 tiles staged through LDS (two workgroups a CU), 4 waves of 128x64.
-// Workgroups are numbered so that those that follow each other on one XCD
-// (every 8th id) take neighbouring row blocks of the same weight tile.
-constexpr int GM = 256, GN = 128, GK = 64, GLD = GK + 8;
-constexpr int G_BUF = (GM + GN) * GLD;                 // elements of one buffer
-
-__global__ void __launch_bounds__(256, 2)
-gemm_big_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float* __restrict__ C, int M,
-                int N, int K, int epilogue, int tiles_m, int tiles_n) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char g_smem[];
-  bf16* smem = reinterpret_cast<bf16*>(g_smem);
-  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
-  const int l32 = lane % 32, kh = lane / 32;
-  const int wm = (wave / 2) * 128, wn = (wave % 2) * 64;
-  // id -> tile: ids 8 apart run on one XCD; give them consecutive tiles, rows fastest
-  const int total = tiles_m * tiles_n;
-  const int bid = blockIdx.x;
-  const int per_xcd = (total + 7) / 8;
-  const int logical = (bid % 8) * per_xcd + bid / 8;
-  if (logical >= total) return;
-  const int m0 = (logical % tiles_m) * GM, n0 = (logical / tiles_m) * GN;
-
-  const int lc = (tid % 8) * 8, lr = tid / 8;
-  const bf16* ap[8];
-  const bf16* wp[4];
-#pragma unroll
-  for (int i = 0; i < 8; ++i) ap[i] = A + (size_t)min(m0 + lr + 32 * i, M - 1) * K + lc;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) wp[i] = W + (size_t)min(n0 + lr + 32 * i, N - 1) * K + lc;
-  bf16x8 ra[8], rw[4];
-  auto fetch = [&](int k0) {
-    const bool ok = k0 + lc + 8 <= K;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) ra[i] = ok ? load8(ap[i] + k0) : zero8();
-#pragma unroll
-    for (int i = 0; i < 4; ++i) rw[i] = ok ? load8(wp[i] + k0) : zero8();
-  };
-  auto stash = [&](int buf) {
-    bf16* As = smem + buf * G_BUF;
-    bf16* Ws = As + GM * GLD;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) *reinterpret_cast<bf16x8*>(&As[(lr + 32 * i) * GLD + lc]) = ra[i];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) *reinterpret_cast<bf16x8*>(&Ws[(lr + 32 * i) * GLD + lc]) = rw[i];
-  };
-
-  f32x16 acc[4][2];
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-
-  const int nk = (K + GK - 1) / GK;
-  const bf16* As = smem;
-  const bf16* Ws = As + GM * GLD;
-  fetch(0);
-  for (int kt = 0; kt < nk; ++kt) {
-    __syncthreads();                 // everyone is done reading the previous tile
-    stash(0);
-    __syncthreads();
-    if (kt + 1 < nk) fetch((kt + 1) * GK);
-    bf16x8 a[2][4], b[2][2];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) a[0][i] = *reinterpret_cast<const bf16x8*>(&As[(wm + 32 * i + l32) * GLD + 8 * kh]);
-#pragma unroll
-    for (int j = 0; j < 2; ++j) b[0][j] = *reinterpret_cast<const bf16x8*>(&Ws[(wn + 32 * j + l32) * GLD + 8 * kh]);
-#pragma unroll
-    for (int ks = 0; ks < GK / 16; ++ks) {
-      const int cur = ks & 1, nxt = cur ^ 1;
-      if (ks + 1 < GK / 16) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          a[nxt][i] = *reinterpret_cast<const bf16x8*>(&As[(wm + 32 * i + l32) * GLD + (ks + 1) * 16 + 8 * kh]);
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-          b[nxt][j] = *reinterpret_cast<const bf16x8*>(&Ws[(wn + 32 * j + l32) * GLD + (ks + 1) * 16 + 8 * kh]);
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[cur][i], b[cur][j], acc[i][j], 0, 0, 0);
-    }
-  }
-  if (epilogue == EPI_SILU_PAIR) {
-    bf16* H = reinterpret_cast<bf16*>(C);
-    const int NH = N / 2;
-    const int n = (n0 + wn) / 2 + l32;
-    if (n < NH) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int m = m0 + wm + 32 * i + 8 * (r / 4) + 4 * kh + (r % 4);
-          if (m < M) {
-            const float g = acc[i][0][r], u = acc[i][1][r];
-            H[(size_t)m * NH + n] = (bf16)((g / (1.0f + expf(-g))) * u);
-          }
-        }
-    }
-    return;
-  }
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int n = n0 + wn + 32 * j + l32;
-      if (n >= N) continue;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int m = m0 + wm + 32 * i + 8 * (r / 4) + 4 * kh + (r % 4);
-        if (m < M) {
-          float* c = C + (size_t)m * N + n;
-          *c = (epilogue == EPI_ACCUMULATE) ? *c + acc[i][j][r] : acc[i][j][r];
-        }
-      }
-    }
-}
-
-static int launch_big(const bf16* A, const bf16* W, float* C, int M, int N, int K, int epilogue,
-                      hipStream_t st) {
-  constexpr int smem = G_BUF * (int)sizeof(bf16);
-  static bool raised = false;
-  if (!raised) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_big_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-    if (e != hipSuccess) {
-      set_error("gemm_big: cannot have %d bytes of LDS: %s", smem, hipGetErrorString(e));
-      return 2;
-    }
-    raised = true;
-  }
-  const int tiles_m = (M + GM - 1) / GM, tiles_n = (N + GN - 1) / GN;
-  const int grid = ((tiles_m * tiles_n + 7) / 8) * 8;
-  gemm_big_kernel<<<grid, 256, smem, st>>>(A, W, C, M, N, K, epilogue, tiles_m, tiles_n);
-  TL_LAUNCH_CHECK("gemm_big");
-  return 0;
-}
-
 }  // namespace tl
 
 using namespace tl;
@@ -1020,15 +764,11 @@ extern "C" int tl_gemm_bf16(const void* A, const void* W, const void* Wt, void* 
     if (wide) return launch_skinny<4, 4, 4>(a, w, c, M, N, K, epilogue, st);
     return launch_skinny<1, 4, 8>(a, w, c, M, N, K, epilogue, st);
   }
-  if (M > 128 && (long long)((M + GM - 1) / GM) * ((N + GN - 1) / GN) >= 512)
-    return launch_big(a, w, c, M, N, K, epilogue, st);      // enough tiles to fill the chip twice
-  dim3 grid((N + TN - 1) / TN, (M + TM - 1) / TM);
-  gemm_tiled_kernel<<<grid, 256, 0, st>>>(a, w, c, M, N, K, epilogue);
-  TL_LAUNCH_CHECK("gemm_tiled");
-  return 0;
+  TL_REQUIRE(false, "gemm_bf16: %d rows; this entry point serves at most 64 (tl_gemm_mid_bf16 takes up to 128, "
+             "the BLAS library more)", M);
 }
 
-// For tests and tuning: force one kernel whatever M is.  variant 0: tiled; 1: big; 2: rows; 1000 + R: the kernel for at
+// For tests and tuning: force one kernel whatever M is.  variant 2: rows; 1000 + R: the kernel for at
 // most 16 rows with R channels a workgroup (1 to 32); else NT*100 + MT*10 + waves/4.
 extern "C" int tl_gemm_bf16_variant(const void* A, const void* W, void* C, int M, int N, int K,
                                     int epilogue, int variant, hipStream_t st) {
@@ -1038,13 +778,6 @@ extern "C" int tl_gemm_bf16_variant(const void* A, const void* W, void* C, int M
   const bf16* a = (const bf16*)A;
   const bf16* w = (const bf16*)W;
   float* c = (float*)C;
-  if (variant == 0) {
-    dim3 grid((N + TN - 1) / TN, (M + TM - 1) / TM);
-    gemm_tiled_kernel<<<grid, 256, 0, st>>>(a, w, c, M, N, K, epilogue);
-    TL_LAUNCH_CHECK("gemm_tiled");
-    return 0;
-  }
-  if (variant == 1) return launch_big(a, w, c, M, N, K, epilogue, st);
   if (variant == 2) {
     TL_REQUIRE(rows_fit(M, N, K), "gemm_rows: M=%d N=%d K=%d (at most 16 rows, N a multiple of 64, K of %d)", M, N,
                K, ROWS_CHUNK);

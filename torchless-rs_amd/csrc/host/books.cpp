@@ -13,9 +13,11 @@
 #include <string>
 #include <vector>
 
+#include "../page.h"
+
 namespace {
 
-constexpr int PAGE = 64;
+constexpr int PAGE = TL_PAGE;
 
 // return codes of the interface; the message of the last failure is kept per thread
 constexpr int OK = 0, FULL = 1, MISUSE = 2, BAD_VALUE = 3, BAD_STEP = 4;

@@ -19,6 +19,16 @@ extern "C" {
 
 size_t tl_static_scratch_bytes(void);
 
+// Looks up the array's device address for the current device (hipGetDevice,
+// hipGetSymbolAddress; the latter may load the code object on that device) and
+// keeps it.  Returns 0, or non-zero with a message in tl_last_error().  Call it
+// once per device at set-up, OUTSIDE any stream capture: the lookup is no
+// stream operation and must not happen while a stream of the device is
+// capturing.  tl_attn_decode_bf16_static does the same lookup at its first call
+// on a device if this was not called, so that first call then has to be made
+// outside capture too (a warm-up step before the capture is enough).
+int tl_static_scratch_ready(void);
+
 // tl_attn_decode_bf16 without its `part` argument: bfloat16 attention of one
 // new token per sequence over its pages (the token's own key is already
 // committed), the keys cut into `n_splits` parts whose partial results
@@ -35,7 +45,9 @@ size_t tl_static_scratch_bytes(void);
 // whose partial results, B * nq * n_splits * (d + 2) floats, exceed
 // TL_STATIC_SCRATCH_BYTES.  It calls no hipMalloc, hipFree or allocating
 // library routine; the array's device address is looked up once per device
-// (hipGetSymbolAddress), at the first call with that device current.
+// (tl_static_scratch_ready, or the first call with that device current, which
+// therefore must not be made under stream capture).  Later calls may be
+// captured into a HIP graph: they only launch kernels on `stream`.
 //
 // Every call on a GPU shares that GPU's array, which keeps the contents of the
 // last call.  Nothing in it has to start at zero: each call's first kernel

@@ -268,10 +268,7 @@ class Engine:
             raise StepError("token_rows without device_tokens")
         packed = pack_step(self.cache, batch, self.vocab_size, token_rows)
         growth = [(s.slot, len(s.tokens)) for s in batch]
-        from ..kernels.ops import LIBRARY_ROWS
-        # (above LIBRARY_ROWS rows the products are the BLAS library's, whose launches are kept
-        # out of captured graphs; such a step is no longer bound by launches anyway)
-        if self.use_graphs and packed.all_single and self.model.graph_safe and packed.n_rows <= LIBRARY_ROWS:
+        if self.use_graphs and packed.all_single and self.model.may_capture(packed.n_rows):
             logits = self._graph_step(packed, device_tokens)
         else:
             dev = torch.from_numpy(packed.flat).to(self.device, non_blocking=False)

@@ -174,10 +174,13 @@ class BatchRun:
             return False
         # a request that is alive and whose budget this token does not use up goes on, unless
         # the token is a stop id, which the host does not know yet
-        ahead = [i for i in order if i in slots and self.count[i] + 1 < self.max_tokens]
+        rows, ahead = [], []
+        for row, i in enumerate(order):
+            if i in slots and self.count[i] + 1 < self.max_tokens:
+                rows.append(row)
+                ahead.append(i)
         nxt_drawn = None
         if ahead:
-            rows = [order.index(i) for i in ahead]
             logits = engine.step([SeqInput(slots[i], [0], [0]) for i in ahead],
                                  device_tokens=drawn.device, token_rows=rows)
             nxt_drawn = self.sampler.draw(logits, ahead, [self.count[i] + 1 for i in ahead])

@@ -41,6 +41,12 @@ class Model:
         self.loaded = False
         self.graph_safe = all(p.graph_safe for p in [self.embedding, self.final_norm, self.head] + self.blocks)
 
+    def may_capture(self, n_rows: int) -> bool:
+        """May a single-token step of `n_rows` rows be captured as a graph and replayed?  Every
+        part answers for itself; the step function knows nothing of their kernels."""
+        return self.loaded and all(p.may_capture(n_rows)
+                                   for p in [self.embedding, self.final_norm, self.head] + self.blocks)
+
     # ---- weights -----------------------------------------------------------
     def load_weights(self, source, tiled_copies: bool = True) -> None:
         """`source`: anything with names/shape/dtype/tensor (a model folder's

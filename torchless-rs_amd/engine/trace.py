@@ -35,7 +35,7 @@ def main(argv=None) -> int:
     ap.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
     ap.add_argument("--out", required=True, help="folder that receives <step>.f32")
     ap.add_argument("--max-tokens", type=int, required=True,
-                    help="most tokens live requests hold at any time (each rounded up to 64)")
+                    help="most tokens live requests hold at any time (each rounded up to whole pages of the cache, 64)")
     args = ap.parse_args(argv)
 
     print("[trace_run] loading torch and the kernels", file=sys.stderr, flush=True)
@@ -43,7 +43,8 @@ def main(argv=None) -> int:
 
     os.makedirs(args.out, exist_ok=True)
     model = load_model(args.model, args.dtype, "cuda:0")
-    engine = Engine(model, max_tokens=max(args.max_tokens, 64))
+    from ..kernels.page import PAGE
+    engine = Engine(model, max_tokens=max(args.max_tokens, PAGE))
     print("[trace_run] ready", file=sys.stderr, flush=True)
 
     slot_of: Dict[str, int] = {}

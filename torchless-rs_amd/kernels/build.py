@@ -74,7 +74,7 @@ def kernels_digest() -> str:
 
 
 def host_digest() -> str:
-    return _digest(host_sources(), HOST_FLAGS)
+    return _digest(host_sources() + [os.path.join(_CSRC, "page.h")], HOST_FLAGS)
 
 
 def _write_stamp(lib: str, digest: str) -> None:
@@ -206,15 +206,20 @@ def build(verbose: bool = True) -> str:
     return lib
 
 
-def built_library(name: str = LIB_NAME) -> Optional[str]:
+def built_library(name: str = LIB_NAME, digest: Optional[str] = None) -> Optional[str]:
     """The library `name` if one is there: in the package's own folder, or in this user's
-    private folder under the temporary directory (never in one that others can write to)."""
+    private folder under the temporary directory (never in one that others can write to).
+    With `digest`, one that was built from the sources of that digest goes before one that was
+    not, wherever it lies: a stale library in a package folder that cannot be written must not
+    hide the current one that an earlier process built into the private folder."""
     pkg, tmp = build_dirs()
-    for d in (pkg, tmp):
-        p = os.path.join(d, name)
-        if os.path.isfile(p) and (d == pkg or _own_private_dir(d)):
-            return p
-    return None
+    found = [p for d in (pkg, tmp) for p in [os.path.join(d, name)]
+             if os.path.isfile(p) and (d == pkg or _own_private_dir(d))]
+    if digest is not None:
+        for p in found:
+            if _is_current(p, digest):
+                return p
+    return found[0] if found else None
 
 
 def _current_or_rebuilt(path: Optional[str], digest: str, rebuild, what: str) -> str:
@@ -238,7 +243,8 @@ def load() -> ctypes.CDLL:
     with _lock:
         if _lib is not None:
             return _lib
-        path = _current_or_rebuilt(built_library(), kernels_digest(), build, "the kernels' library")
+        digest = kernels_digest()
+        path = _current_or_rebuilt(built_library(LIB_NAME, digest), digest, build, "the kernels' library")
         try:
             _lib = ctypes.CDLL(path)
         except OSError as e:
@@ -252,7 +258,8 @@ def load_host() -> ctypes.CDLL:
     with _lock:
         if _host_lib is not None:
             return _host_lib
-        path = _current_or_rebuilt(built_library(HOST_LIB_NAME), host_digest(), build_host, "the host library")
+        digest = host_digest()
+        path = _current_or_rebuilt(built_library(HOST_LIB_NAME, digest), digest, build_host, "the host library")
         try:
             _host_lib = ctypes.CDLL(path)
         except OSError as e:

@@ -15,6 +15,7 @@ from typing import Optional
 import torch
 
 from .build import load
+from .page import PAGE, require_same
 
 DT_F32, DT_BF16 = 0, 1
 _CODES = {torch.float32: DT_F32, torch.bfloat16: DT_BF16}
@@ -32,6 +33,7 @@ def lib() -> ctypes.CDLL:
     L = load()
     if not _configured:
         L.tl_last_error.restype = ctypes.c_char_p
+        require_same(L.tl_page_size(), "the kernels' library")
         _configured = True
     return L
 
@@ -157,8 +159,8 @@ def kv_commit(k: torch.Tensor, v: torch.Tensor, row_seq, row_pos, len_after, tab
     _req(len_after, "kv_commit.len_after", torch.int32)
     _req(table, "kv_commit.table", torch.int32)
     _req(pages, "kv_commit.pages")
-    if pages.dim() != 5 or tuple(pages.shape[1:]) != (2, nkv, 64, d):
-        raise KernelError(f"kv_commit.pages: shape {tuple(pages.shape)}, kernel needs [*, 2, {nkv}, 64, {d}]")
+    if pages.dim() != 5 or tuple(pages.shape[1:]) != (2, nkv, PAGE, d):
+        raise KernelError(f"kv_commit.pages: shape {tuple(pages.shape)}, kernel needs [*, 2, {nkv}, {PAGE}, {d}]")
     if table.dim() != 2 or table.shape[0] != len_after.shape[0]:
         raise KernelError("kv_commit.table: needs one row per sequence")
     _check(lib().tl_kv_commit(_p(k), _p(v), _code(k.dtype), _p(row_seq), _p(row_pos), _p(len_after),
@@ -181,8 +183,8 @@ def v_tiles(qkv: torch.Tensor, nq: int, nkv: int, d: int, vt: torch.Tensor, cu_s
     n = qkv.shape[0]
     _req(qkv, "v_tiles.qkv", torch.float32, (n, (nq + 2 * nkv) * d))
     _req(vt, "v_tiles.vt")
-    if vt.dim() != 3 or tuple(vt.shape[:2]) != (nkv, d) or vt.shape[2] % 64:
-        raise KernelError(f"v_tiles.vt: shape {tuple(vt.shape)}, kernel needs [{nkv}, {d}, a multiple of 64]")
+    if vt.dim() != 3 or tuple(vt.shape[:2]) != (nkv, d) or vt.shape[2] % PAGE:
+        raise KernelError(f"v_tiles.vt: shape {tuple(vt.shape)}, kernel needs [{nkv}, {d}, a multiple of {PAGE}]")
     B = tile_off.shape[0]
     _tiles_args(B, cu_seqlens, tile_off, n_cached, len_after, "v_tiles")
     _check(lib().tl_v_tiles(_p(qkv), n, nq, nkv, d, _p(vt), vt.shape[2], _code(vt.dtype), B, _p(cu_seqlens),
@@ -199,8 +201,8 @@ def rope_v_tiles(qkv: torch.Tensor, row_pos, rotation, nq: int, nkv: int, d: int
     _req(q, "rope_v_tiles.q", None, (n, nq, d))
     _req(k, "rope_v_tiles.k", q.dtype, (n, nkv, d))
     _req(vt, "rope_v_tiles.vt", q.dtype)
-    if vt.dim() != 3 or tuple(vt.shape[:2]) != (nkv, d) or vt.shape[2] % 64:
-        raise KernelError(f"rope_v_tiles.vt: shape {tuple(vt.shape)}, kernel needs [{nkv}, {d}, a multiple of 64]")
+    if vt.dim() != 3 or tuple(vt.shape[:2]) != (nkv, d) or vt.shape[2] % PAGE:
+        raise KernelError(f"rope_v_tiles.vt: shape {tuple(vt.shape)}, kernel needs [{nkv}, {d}, a multiple of {PAGE}]")
     B = tile_off.shape[0]
     _tiles_args(B, cu_seqlens, tile_off, n_cached, len_after, "rope_v_tiles")
     if cu_seqlens is None:
@@ -217,16 +219,16 @@ def kv_commit_tiles(k: torch.Tensor, vt: torch.Tensor, row_seq, row_pos, tile_of
     n, nkv, d = k.shape
     _req(k, "kv_commit.k", pages.dtype)
     _req(vt, "kv_commit.vt", pages.dtype)
-    if vt.dim() != 3 or tuple(vt.shape[:2]) != (nkv, d) or vt.shape[2] % 64:
-        raise KernelError(f"kv_commit.vt: shape {tuple(vt.shape)}, kernel needs [{nkv}, {d}, a multiple of 64]")
+    if vt.dim() != 3 or tuple(vt.shape[:2]) != (nkv, d) or vt.shape[2] % PAGE:
+        raise KernelError(f"kv_commit.vt: shape {tuple(vt.shape)}, kernel needs [{nkv}, {d}, a multiple of {PAGE}]")
     _req(row_seq, "kv_commit.row_seq", torch.int32, (n,))
     _req(row_pos, "kv_commit.row_pos", torch.int32, (n,))
     B = tile_off.shape[0]
     _tiles_args(B, None, tile_off, n_cached, len_after, "kv_commit")
     _req(table, "kv_commit.table", torch.int32)
     _req(pages, "kv_commit.pages")
-    if pages.dim() != 5 or tuple(pages.shape[1:]) != (2, nkv, 64, d):
-        raise KernelError(f"kv_commit.pages: shape {tuple(pages.shape)}, kernel needs [*, 2, {nkv}, 64, {d}]")
+    if pages.dim() != 5 or tuple(pages.shape[1:]) != (2, nkv, PAGE, d):
+        raise KernelError(f"kv_commit.pages: shape {tuple(pages.shape)}, kernel needs [*, 2, {nkv}, {PAGE}, {d}]")
     if table.dim() != 2 or table.shape[0] != B:
         raise KernelError("kv_commit.table: needs one row per sequence")
     _check(lib().tl_kv_commit_tiles(_p(k), _p(vt), vt.shape[2], _code(k.dtype), _p(row_seq), _p(row_pos), B,
@@ -246,8 +248,8 @@ def attn_plain(q, k_new, v_new, pages, table, ring_pages: int, row_seq, row_pos,
         _req(k_new, "attn.k_new", pages.dtype, (n, nkv, d))
         _req(v_new, "attn.v_new", pages.dtype, (n, nkv, d))
     _req(pages, "attn.pages")
-    if pages.dim() != 5 or tuple(pages.shape[1:]) != (2, nkv, 64, d):
-        raise KernelError(f"attn.pages: shape {tuple(pages.shape)}, kernel needs [*, 2, nkv, 64, {d}]")
+    if pages.dim() != 5 or tuple(pages.shape[1:]) != (2, nkv, PAGE, d):
+        raise KernelError(f"attn.pages: shape {tuple(pages.shape)}, kernel needs [*, 2, nkv, {PAGE}, {d}]")
     _req(table, "attn.table", torch.int32)
     _req(row_seq, "attn.row_seq", torch.int32, (n,))
     _req(row_pos, "attn.row_pos", torch.int32, (n,))
@@ -460,7 +462,7 @@ def compute_units(device) -> int:
     return _UNITS[key]
 
 
-def mid_splits(M: int, N: int, K: int, units: int = 256) -> int:
+def mid_splits(M: int, N: int, K: int, units: int) -> int:
     """For 17..MID_ROWS rows: into how many slices K is cut so that some 400
     workgroups or more (64 output channels each) are at work, a power of two
     (which shares the k-steps out evenly at the usual sizes; measured best at
@@ -584,8 +586,8 @@ def rope_commit(qkv: torch.Tensor, row_pos, rotation, table, ring_pages: int, nq
     _req(q, "rope.q", pages.dtype, (n, nq, d))
     _req(table, "rope.table", torch.int32)
     _req(pages, "rope.pages")
-    if pages.dim() != 5 or tuple(pages.shape[1:]) != (2, nkv, 64, d):
-        raise KernelError(f"rope.pages: shape {tuple(pages.shape)}, kernel needs [*, 2, {nkv}, 64, {d}]")
+    if pages.dim() != 5 or tuple(pages.shape[1:]) != (2, nkv, PAGE, d):
+        raise KernelError(f"rope.pages: shape {tuple(pages.shape)}, kernel needs [*, 2, {nkv}, {PAGE}, {d}]")
     if table.dim() != 2 or table.shape[0] != n:
         raise KernelError("rope.table: needs one row per sequence")
     _check(lib().tl_rope_commit(_p(qkv), n_parts, _p(row_pos), _p(rot.inv_freq), rot.rotary_dim,
@@ -617,8 +619,8 @@ def qkv_rope_commit(a: torch.Tensor, w: torch.Tensor, row_pos, rotation, table, 
     _req(q, "qkv_rope_commit.q", torch.bfloat16, (n, nq, d))
     _req(table, "qkv_rope_commit.table", torch.int32)
     _req(pages, "qkv_rope_commit.pages", torch.bfloat16)
-    if pages.dim() != 5 or tuple(pages.shape[1:]) != (2, nkv, 64, d):
-        raise KernelError(f"qkv_rope_commit.pages: shape {tuple(pages.shape)}, kernel needs [*, 2, {nkv}, 64, {d}]")
+    if pages.dim() != 5 or tuple(pages.shape[1:]) != (2, nkv, PAGE, d):
+        raise KernelError(f"qkv_rope_commit.pages: shape {tuple(pages.shape)}, kernel needs [*, 2, {nkv}, {PAGE}, {d}]")
     if table.dim() != 2 or table.shape[0] != n:
         raise KernelError("qkv_rope_commit.table: needs one row per sequence")
     ssq_in, n_part, inv_h, eps = None, 0, 0.0, 0.0
@@ -662,12 +664,12 @@ def attn_prefill_bf16(q, k_new, vt_new, tile_off, pages, table, ring_pages: int,
     _req(q, "attn.q", torch.bfloat16)
     _req(k_new, "attn.k_new", torch.bfloat16, (n, nkv, d))
     _req(vt_new, "attn.vt_new", torch.bfloat16)
-    if vt_new.dim() != 3 or tuple(vt_new.shape[:2]) != (nkv, d) or vt_new.shape[2] % 64:
-        raise KernelError(f"attn.vt_new: shape {tuple(vt_new.shape)}, kernel needs [{nkv}, {d}, 64 k]")
+    if vt_new.dim() != 3 or tuple(vt_new.shape[:2]) != (nkv, d) or vt_new.shape[2] % PAGE:
+        raise KernelError(f"attn.vt_new: shape {tuple(vt_new.shape)}, kernel needs [{nkv}, {d}, a multiple of {PAGE}]")
     _req(tile_off, "attn.tile_off", torch.int32, (B,))
     _req(pages, "attn.pages", torch.bfloat16)
-    if pages.dim() != 5 or tuple(pages.shape[1:]) != (2, nkv, 64, d):
-        raise KernelError(f"attn.pages: shape {tuple(pages.shape)}, kernel needs [*, 2, nkv, 64, {d}]")
+    if pages.dim() != 5 or tuple(pages.shape[1:]) != (2, nkv, PAGE, d):
+        raise KernelError(f"attn.pages: shape {tuple(pages.shape)}, kernel needs [*, 2, nkv, {PAGE}, {d}]")
     _req(table, "attn.table", torch.int32)
     _req(row_pos, "attn.row_pos", torch.int32, (n,))
     _req(cu_seqlens, "attn.cu_seqlens", torch.int32, (B + 1,))
@@ -690,8 +692,8 @@ def attn_decode_bf16(q, pages, table, ring_pages: int, row_pos, window: Optional
     nkv = pages.shape[2]
     _req(q, "attn.q", torch.bfloat16)
     _req(pages, "attn.pages", torch.bfloat16)
-    if pages.dim() != 5 or tuple(pages.shape[1:]) != (2, nkv, 64, d):
-        raise KernelError(f"attn.pages: shape {tuple(pages.shape)}, kernel needs [*, 2, nkv, 64, {d}]")
+    if pages.dim() != 5 or tuple(pages.shape[1:]) != (2, nkv, PAGE, d):
+        raise KernelError(f"attn.pages: shape {tuple(pages.shape)}, kernel needs [*, 2, nkv, {PAGE}, {d}]")
     _req(table, "attn.table", torch.int32)
     _req(row_pos, "attn.row_pos", torch.int32, (B,))
     _req(part, "attn.part", torch.float32)
@@ -712,7 +714,11 @@ def decode_groups(B: int, nq: int, nkv: int) -> int:
 
 
 SPLIT_PAGES = 4             # fewest pages a part of the keys has
-SPLIT_COST = 0.15           # what a part more costs in the merge, in pages of a workgroup's way
+SPLIT_COST = 0.15           # what a part more costs in the merge, in pages of a workgroup's way (8 sequences of
+                            # 8 KV heads over 4,096 keys: 4 parts 3.91 ms a step, 8 parts 3.96, 6 parts 4.08)
+FULL_UNIT_HEAD = 128        # the head size from which one workgroup has enough bytes under way to keep a compute
+                            # unit streaming; smaller heads get FULL_UNIT_HEAD // head_dim workgroups a unit
+                            # (heads of 64 at batch 32: 52.5 against 55.7 us with two a unit)
 
 
 @functools.lru_cache(maxsize=4096)
@@ -723,7 +729,7 @@ def _decode_splits(groups: int, max_pages: int, units: int) -> int:
     return min(range(1, most + 1), key=lambda s: (cost(s), s))
 
 
-def decode_splits(B: int, nq: int, nkv: int, max_pages: int, units: int = 256, head_dim: int = 128) -> int:
+def decode_splits(B: int, nq: int, nkv: int, max_pages: int, units: int, head_dim: int) -> int:
     """Into how many parts the keys of a decode step are cut.  A compute unit streams at a rate of
     its own, so the step's attention takes as long as the unit with the most to read: rounds of
     workgroups over the `units` compute units times the pages a workgroup has, plus the merge's
@@ -732,7 +738,7 @@ def decode_splits(B: int, nq: int, nkv: int, max_pages: int, units: int = 256, h
     four pages.  With heads of 64 or less a workgroup has too few bytes under way to keep a unit
     busy alone, and a round is two workgroups a unit (four with heads of 32: 32 sequences of 4 KV
     heads of 32 take 19.2 us in 4 parts, 27.2 in 2)."""
-    return _decode_splits(decode_groups(B, nq, nkv), int(max_pages), int(units) * max(1, 128 // max(1, int(head_dim))))
+    return _decode_splits(decode_groups(B, nq, nkv), int(max_pages), int(units) * max(1, FULL_UNIT_HEAD // max(1, int(head_dim))))
 
 
 def uses_transposed_values(dtype: torch.dtype, d: int, all_single: bool) -> bool:
@@ -764,31 +770,56 @@ def attention(q, k_new, v_new, pages, table, ring_pages: int, ctx, n_cached, win
                    n_cached, window, scale, out)
 
 
-def measure_ceilings(device="cuda:0", gib: float = 8.0) -> dict:
+READ_SHAPES = {0: "8 loads a lane, a grid stride apart", 1: "16 loads a lane", 2: "32 loads a lane",
+               3: "8 loads a lane, a contiguous share a workgroup", 4: "16 loads a lane, contiguous",
+               5: "8 loads a lane, non-temporal", 6: "16 loads a lane, non-temporal, contiguous",
+               7: "8 loads a wave straight into LDS", 8: "16 loads a wave straight into LDS"}
+
+
+def measure_ceilings(device="cuda:0", gib: float = 8.0, shapes=None) -> dict:
     """What the simplest kernels get on this machine: GB/s of one read of a buffer far larger
-    than the caches, and TFLOP/s of independent bfloat16 MFMAs on registers (the best of a
-    few runs and launch shapes each)."""
+    than the caches, in every shape of `READ_SHAPES` (the best is reported with its shape, the
+    others beside it), GB/s of a copy (bytes read plus bytes written), and TFLOP/s of independent
+    bfloat16 MFMAs on registers (the best of a few runs and launch shapes each)."""
     import time
-    n_bytes = int(gib * 2 ** 30) // 16 * 16
+    units = compute_units(device)
+    quantum = units * 32 * 256 * 32 * 16          # whole iterations of every shape at every number of workgroups (1 GiB)
+    n_bytes = max(1, round(gib * 2 ** 30 / quantum)) * quantum
     buf = torch.empty(n_bytes // 4, dtype=torch.float32, device=device).normal_()
-    sink = torch.zeros(256 * 32, dtype=torch.float32, device=device)
-    best_read = 0.0
-    for blocks in (256, 256 * 2, 256 * 4, 256 * 8, 256 * 16, 256 * 32):     # one workgroup a compute unit is the fastest
+    sink = torch.zeros(units * 32, dtype=torch.float32, device=device)
+
+    def timed(launch):
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        _check(launch())
+        torch.cuda.synchronize()
+        return time.perf_counter() - t
+
+    by_shape = {}
+    for shape in (READ_SHAPES if shapes is None else shapes):
+        best = 0.0
+        for blocks in (units, units * 2, units * 4, units * 8, units * 16, units * 32):
+            for _ in range(3):
+                dt = timed(lambda: lib().tl_stream_read_shape(_p(buf), ctypes.c_size_t(n_bytes), _p(sink), blocks,
+                                                              shape, _stream()))
+                best = max(best, n_bytes / dt / 1e9)
+        by_shape[shape] = round(best, 1)
+    top = max(by_shape, key=by_shape.get)
+    half = n_bytes // 2
+    dst = buf.view(-1)[half // 4:]
+    best_copy = 0.0
+    for blocks in (units, units * 2, units * 4, units * 8):
         for _ in range(3):
-            torch.cuda.synchronize()
-            t = time.perf_counter()
-            _check(lib().tl_stream_read(_p(buf), ctypes.c_size_t(n_bytes), _p(sink), blocks, _stream()))
-            torch.cuda.synchronize()
-            best_read = max(best_read, n_bytes / (time.perf_counter() - t) / 1e9)
-    del buf
+            dt = timed(lambda: lib().tl_stream_copy(_p(buf), _p(dst), ctypes.c_size_t(half), blocks, _stream()))
+            best_copy = max(best_copy, 2 * half / dt / 1e9)
+    del buf, dst
     best_mfma = 0.0
-    for blocks in (256, 256 * 2, 256 * 4):
+    for blocks in (units, units * 2, units * 4):
         iters = 8192
         for _ in range(3):
-            torch.cuda.synchronize()
-            t = time.perf_counter()
-            _check(lib().tl_mfma_chain(iters, blocks, _p(sink), _stream()))
-            torch.cuda.synchronize()
+            dt = timed(lambda: lib().tl_mfma_chain(iters, blocks, _p(sink), _stream()))
             flop = blocks * 4 * iters * 8 * 2 * 32 * 32 * 16
-            best_mfma = max(best_mfma, flop / (time.perf_counter() - t) / 1e12)
-    return {"hbm_read_GBs": round(best_read, 1), "mfma_bf16_TFLOPs": round(best_mfma, 1)}
+            best_mfma = max(best_mfma, flop / dt / 1e12)
+    return {"hbm_read_GBs": by_shape[top], "hbm_read_shape": READ_SHAPES[top],
+            "hbm_read_by_shape_GBs": {READ_SHAPES[k]: v for k, v in by_shape.items()},
+            "hbm_copy_GBs": round(best_copy, 1), "mfma_bf16_TFLOPs": round(best_mfma, 1)}

@@ -42,7 +42,9 @@ class AttentionMixer(Mixer):
 
     def __init__(self, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int,
                  position: PartSpec, window: Optional[int] = None, own_kv: bool = True,
-                 prefix: str = "self_attn.", names: Optional[Dict[str, Optional[str]]] = None):
+                 prefix: str = "self_attn.", names: Optional[Dict[str, Optional[str]]] = None,
+                 scale: Optional[float] = None):
+        """`scale`: what a score k.q is multiplied by before the softmax; None: 1 / sqrt(head_dim)."""
         if n_heads % n_kv_heads:
             raise ValueError(f"attention: {n_heads} heads are not a multiple of {n_kv_heads} KV heads")
         unknown = set(names or {}) - set(self.NAMES)
@@ -56,12 +58,15 @@ class AttentionMixer(Mixer):
         self.own_kv = bool(own_kv)
         self.prefix = prefix
         self.position = make_part("position", position)
-        self.scale = 1.0 / math.sqrt(self.d)
+        self.scale = 1.0 / math.sqrt(self.d) if scale is None else float(scale)
         self.qkv = None
         self.o = None
 
     def kv_request(self):
         return KVRequest(self.nkv, self.d, self.window) if self.own_kv else None
+
+    def may_capture(self, n_rows: int) -> bool:
+        return self.qkv is not None and self.qkv.own_kernels(n_rows) and self.o.own_kernels(n_rows)
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
         p, nm = self.prefix, self.names

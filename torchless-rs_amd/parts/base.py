@@ -114,6 +114,12 @@ class Part:
     # device): such a step can be captured once as a HIP graph and replayed.
     graph_safe = False
 
+    def may_capture(self, n_rows: int) -> bool:
+        """May a single-token step of `n_rows` rows through this part go into a captured graph?
+        A part whose kernels depend on the number of rows (a product that hands many rows to
+        the BLAS library, whose launches stay out of graphs) answers for that number."""
+        return self.graph_safe
+
     def weight_specs(self) -> Dict[str, WeightSpec]:
         return {}
 
@@ -198,6 +204,50 @@ def take_row_factor(ctx: "StepContext", usable: bool):
         f = None
     ctx.settle = None
     return f
+
+
+def read_through_norm(ctx: "StepContext", norm: "Norm", x: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
+    """The stream `x` as `norm` gives it to the part behind it (a block calls this for every norm
+    it runs; returns the buffer that holds the result, which is `y` or what a product left).
+    Partial products that a part left pending are added first, by the norm itself if it can
+    (`takes_pending`).  If the product that completed the stream did this norm's first half
+    (`expect_norm` had announced it), the result is what that product left, and the factor per
+    row goes to the part that reads it (`ctx.row_factor`; `ctx.settle` runs the plain norm into
+    the same buffer for a part that cannot apply it)."""
+    pre, ctx.prenormed = ctx.prenormed, None
+    if pre is not None and pre[0] is norm:
+        ctx.row_factor = pre[2]
+        ctx.settle = lambda: norm.forward(ctx, x, pre[1])
+        return pre[1]
+    if not getattr(norm, "takes_pending", False):
+        flush_pending(ctx, x)
+    norm.forward(ctx, x, y)
+    return y
+
+
+def expect_norm(ctx: "StepContext", writer: Part, norm: Optional["Norm"], reader: Optional[Part] = None) -> None:
+    """Before `writer` runs: announce that `norm` reads the stream next and `reader` reads the
+    norm.  If all three can (`writer.closes_stream`, `norm.rms_form()`, `reader.takes_row_factor`)
+    the product that completes the stream may do the norm's first half (steps of at most 16
+    rows); if not, nothing is announced and the norm runs by itself.  `reader` None: the norm
+    is another block's `splittable_entry`, which has asked its reader already."""
+    ok = (norm is not None and getattr(writer, "closes_stream", False) and norm.rms_form() is not None
+          and (reader is None or getattr(reader, "takes_row_factor", False)))
+    ctx.norm_ahead = norm if ok else None
+
+
+def part_done(ctx: "StepContext", part: Part) -> None:
+    """After a part has run: what was announced to it is void, and a factor per row that it was
+    handed must have been taken."""
+    ctx.norm_ahead = None
+    if ctx.row_factor is not None:
+        raise RuntimeError(f"{type(part).__name__} declares takes_row_factor and left the factor untaken")
+
+
+def splittable_entry(norm: "Norm", reader: Part) -> Optional["Norm"]:
+    """`norm` if it is the first reader of the stream in a block and can be cut in two for
+    `reader` (the block before may then do its first half); else None."""
+    return norm if norm.rms_form() is not None and getattr(reader, "takes_row_factor", False) else None
 
 
 def flush_pending(ctx: "StepContext", x: torch.Tensor) -> None:

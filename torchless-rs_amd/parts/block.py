@@ -8,7 +8,8 @@ from typing import Dict
 import torch
 
 from ..weights.binding import WeightSpec
-from .base import LayerSpec, Part, flush_pending, make_part, register_part
+from .base import (LayerSpec, Part, expect_norm, make_part, part_done, read_through_norm, register_part,
+                   splittable_entry)
 
 
 class PreNormBlock(Part):
@@ -39,48 +40,27 @@ class PreNormBlock(Part):
         self.mixer.load(tensors, compute_dtype)
         self.ffn.load(tensors, compute_dtype)
 
+    def may_capture(self, n_rows: int) -> bool:
+        return all(p.may_capture(n_rows) for p in (self.mixer, self.ffn, self.mixer_norm, self.ffn_norm))
+
     def entry_norm(self):
         """The norm that reads the stream first, if the part behind it can take a norm cut in
         two (the block before this one may then do the norm's first half)."""
-        ok = self.mixer_norm.rms_form() is not None and getattr(self.mixer, "takes_row_factor", False)
-        return self.mixer_norm if ok else None
+        return splittable_entry(self.mixer_norm, self.mixer)
 
     def forward(self, ctx, run, x: torch.Tensor, norm_after=None) -> None:
-        """`norm_after`: the `entry_norm` of the block that runs next, if it has one."""
+        """`norm_after`: the `entry_norm` of the block that runs next, if it has one.  The three
+        helpers around each part (`read_through_norm`, `expect_norm`, `part_done`) are all that
+        an arrangement needs for norms cut in two around the products."""
         y = ctx.workspace.get("block_y", tuple(x.shape), ctx.dtype)
-        y1 = self._norm(self.mixer_norm, ctx, x, y)
-        if (self.ffn_norm.rms_form() is not None and getattr(self.ffn, "takes_row_factor", False)
-                and getattr(self.mixer, "closes_stream", False)):
-            ctx.norm_ahead = self.ffn_norm
+        y1 = read_through_norm(ctx, self.mixer_norm, x, y)
+        expect_norm(ctx, self.mixer, self.ffn_norm, self.ffn)
         self.mixer.forward(ctx, run, y1, x)
-        self._after_part(ctx, self.mixer)
-        y2 = self._norm(self.ffn_norm, ctx, x, y)
-        if getattr(self.ffn, "closes_stream", False):
-            ctx.norm_ahead = norm_after
+        part_done(ctx, self.mixer)
+        y2 = read_through_norm(ctx, self.ffn_norm, x, y)
+        expect_norm(ctx, self.ffn, norm_after)
         self.ffn.forward(ctx, y2, x)
-        self._after_part(ctx, self.ffn)
-
-    @staticmethod
-    def _after_part(ctx, part) -> None:
-        ctx.norm_ahead = None
-        if ctx.row_factor is not None:
-            raise RuntimeError(f"{type(part).__name__} declares takes_row_factor and left the factor untaken")
-
-    @staticmethod
-    def _norm(norm, ctx, x, y) -> torch.Tensor:
-        """A norm reads the stream: partial products that a part left pending are
-        added first, by the norm itself if it can (`takes_pending`).  If the product
-        that completed the stream did this norm's first half, the output is what it
-        left, and the factor per row goes to the part that reads it."""
-        pre, ctx.prenormed = ctx.prenormed, None
-        if pre is not None and pre[0] is norm:
-            ctx.row_factor = pre[2]
-            ctx.settle = lambda: norm.forward(ctx, x, pre[1])      # the plain norm into the same buffer
-            return pre[1]
-        if not getattr(norm, "takes_pending", False):
-            flush_pending(ctx, x)
-        norm.forward(ctx, x, y)
-        return y
+        part_done(ctx, self.ffn)
 
 
 register_part("block", "pre_norm", PreNormBlock)

@@ -34,6 +34,8 @@ class LMHead(Part):
     """`tied`: use the embedding table instead of a tensor of its own."""
     graph_safe = True
 
+    def may_capture(self, n_rows: int) -> bool:
+        return self.proj is not None and self.proj.own_kernels(n_rows)
 
     def __init__(self, vocab_size: int, hidden_size: int, tied: bool = False, name: str = "weight"):
         self.V, self.H, self.tied, self.name = int(vocab_size), int(hidden_size), bool(tied), name

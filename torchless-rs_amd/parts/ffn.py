@@ -35,6 +35,9 @@ class SwiGLU(FeedForward):
         self.gate_up = None
         self.down = None
 
+    def may_capture(self, n_rows: int) -> bool:
+        return self.gate_up is not None and self.gate_up.own_kernels(n_rows) and self.down.own_kernels(n_rows)
+
     def weight_specs(self) -> Dict[str, WeightSpec]:
         p, nm = self.prefix, self.names
         if nm["gate_up"]:

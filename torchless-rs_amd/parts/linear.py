@@ -57,6 +57,11 @@ class Linear:
         else:
             ops.gemm(a, self.weight, out, accumulate, tiles=self.tiles)
 
+    def own_kernels(self, n_rows: int) -> bool:
+        """Does a product of `n_rows` rows launch this package's kernels only (never the BLAS
+        library's, which a captured graph must not hold)?"""
+        return n_rows <= ops.LIBRARY_ROWS or self.weight.dtype != torch.bfloat16
+
     def mid(self, a: torch.Tensor) -> bool:
         """17..MID_ROWS rows of bfloat16: the kernel that shares the activations.
         (Above LIBRARY_ROWS rows it beats the library only with K cut into
