@@ -284,7 +284,7 @@ def to_bf16(t: torch.Tensor) -> torch.Tensor:
     return t.to(torch.float32).to(torch.bfloat16).to(t.dtype)
 
 
-def forward_rounded(weights: dict, cfg: dict, ids, step_rows, library_rows=64, matrix_core_heads=None,
+def forward_rounded(weights: dict, cfg: dict, ids, step_rows, library_rows="auto", matrix_core_heads=None,
                     ffn_norm_in_halves=True) -> torch.Tensor:
     """`forward` in float64 with a rounding to bfloat16 at every place where the engine's
     bfloat16 path stores one, and nowhere else: the output of a norm, q and k after the rotation,
@@ -297,7 +297,8 @@ def forward_rounded(weights: dict, cfg: dict, ids, step_rows, library_rows=64, m
       it: bfloat16(x * w) goes into the product and the results are multiplied by
       rsqrt(mean(x^2) + eps) (all but the first layer's first norm and the last norm);
     * above `library_rows` rows, gate and up are themselves stored in bfloat16 before the
-      activation (None: never).
+      activation (None: never; "auto": the engine's rule, 128 rows where the hidden size is a multiple
+      of 128, else 64).
     (The kernels round a probability against the running maximum of the keys seen so far and
     scale float32 sums afterwards; here it is rounded against the row's maximum: another
     realisation of the same rounding.)
@@ -314,6 +315,8 @@ def forward_rounded(weights: dict, cfg: dict, ids, step_rows, library_rows=64, m
     ids = torch.as_tensor(ids)
     T = ids.shape[0]
     step_rows = torch.as_tensor(step_rows, device=dev)
+    if library_rows == "auto":
+        library_rows = 128 if cfg["hidden_size"] % 128 == 0 else 64
     split = (step_rows <= 16)[:, None]
     pre_round = (step_rows > library_rows)[:, None] if library_rows else torch.zeros(T, 1, dtype=torch.bool, device=dev)
     positions = torch.arange(T, device=dev)

@@ -2,19 +2,26 @@
 from torchless_rs_amd.kernels import ops
 
 
-def test_mid_splits_are_powers_of_two_that_fit():
+def test_mid_splits_fit():
     for M in (17, 64, 128):
         for N in (72, 4096, 6144, 28672, 32000):
             for K in (48, 256, 1000, 4096, 14336):
                 S = ops.mid_splits(M, N, K, 256)
-                steps = -(-K // 256)
-                assert S >= 1 and S & (S - 1) == 0, (M, N, K, S)
-                assert S <= max(1, steps) and S <= 16, (M, N, K, S)
-    # the 7B sizes: narrow outputs are cut in 8, the wide one is not cut
-    assert ops.mid_splits(64, 4096, 4096, 256) == 8 and ops.mid_splits(64, 6144, 4096, 256) == 8
+                if K % ops.RING_K == 0:                  # the ring kernel: every slice has a stage of 128 k at least
+                    assert 1 <= S <= max(1, K // 128) and S <= 16, (M, N, K, S)
+                    assert -(-N // 128) * S <= 256 or S == 1, (M, N, K, S)      # one round of workgroups
+                else:                                    # gemm_mid: powers of two, a step of 256 k at least each
+                    steps = -(-K // 256)
+                    assert S >= 1 and S & (S - 1) == 0, (M, N, K, S)
+                    assert S <= max(1, steps) and S <= 16, (M, N, K, S)
+    # the 7B sizes: narrow outputs are cut to one round of workgroups on 256 compute units, the wide one is not cut
+    assert ops.mid_splits(64, 4096, 4096, 256) == 8 and ops.mid_splits(64, 6144, 4096, 256) == 5
     assert ops.mid_splits(128, 4096, 14336, 256) == 8 and ops.mid_splits(64, 28672, 4096, 256) == 1
-    assert ops.mid_splits(20, 72, 48, 256) == 1                  # one step of K: nothing to cut
-    assert ops.mid_splits(64, 5120, 14336, 256) == 16 and ops.mid_splits(64, 5120, 14336, units=320) == 8   # whole rounds of workgroups
+    assert ops.mid_splits(64, 5120, 14336, 256) == 6 and ops.mid_splits(64, 5120, 14336, units=320) == 8
+    assert ops.mid_splits(64, 4096, 256, 256) == 1          # two stages: nothing to cut
+    assert ops.mid_splits(20, 72, 48, 256) == 1             # (gemm_mid) one step of K: nothing to cut
+    assert ops.mid_splits(64, 4096, 4104, 256) == 8         # (gemm_mid) K no multiple of 128: 64 x 8 workgroups
+    assert ops.own_rows(4096) == ops.MID_ROWS and ops.own_rows(4104) == ops.LIBRARY_ROWS
 
 
 def test_decode_splits_follow_batch_and_length():
@@ -45,4 +52,7 @@ def test_rows_choose_the_kernel():
     rows = lambda m: torch.zeros(m, 4096, dtype=torch.bfloat16)
     assert [lin.mid(rows(m)) for m in (1, 16, 17, ops.MID_ROWS, ops.MID_ROWS + 1)] == [False, False, True, True, False]
     assert not lin.mid(torch.zeros(32, 4096))                        # float32 rows: the plain kernel
-    assert ops.LIBRARY_ROWS < ops.MID_ROWS                           # between them only narrow outputs are ours
+    assert [lin.own_kernels(m) for m in (1, 64, 128, 129)] == [True, True, True, False]
+    odd = Linear(torch.zeros(96, 4104, dtype=torch.bfloat16))        # K no multiple of 128: the library from 65 rows on
+    assert [odd.mid(torch.zeros(m, 4104, dtype=torch.bfloat16)) for m in (17, 64, 65)] == [True, True, False]
+    assert [odd.own_kernels(m) for m in (64, 65)] == [True, False]

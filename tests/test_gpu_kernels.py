@@ -933,6 +933,67 @@ def test_gemm_mid_paired_silu_and_row_independence(ops, M):
     assert torch.equal(few, full[:17])
 
 
+@pytest.mark.parametrize("waves,kc", [(4, 128), (7, 128), (8, 128), (4, 64), (7, 64), (8, 64)])
+@pytest.mark.parametrize("M,N,K,S", [(17, 64, 128, 1), (33, 200, 1024, 2), (64, 256, 512, 1), (100, 336, 1152, 3),
+                                     (128, 520, 2048, 4), (5, 40, 384, 1), (96, 130, 256, 2)])
+def test_gemm_ring_bf16(ops, waves, kc, M, N, K, S):
+    """The product whose operands go from memory straight into a ring of LDS stages: every number of
+    waves a workgroup and both stage sizes, rows and channels that fill no tile, K cut into slices
+    of unequal numbers of stages; stored, accumulated, and as partial sums."""
+    a = rnd(M, K, seed=51, dtype=torch.bfloat16)
+    w = rnd(N, K, seed=52, dtype=torch.bfloat16)
+    want = a.double() @ w.double().t()
+    if S == 1:
+        out = torch.full((M, N), float("nan"), device=DEV)
+        ops.gemm_ring_bf16(a.to(DEV), w.to(DEV), out, waves=waves, kc=kc)
+        assert rel_err(out, want) < 3e-6
+        base = rnd(M, N, seed=53)
+        acc = base.clone().to(DEV)
+        ops.gemm_ring_bf16(a.to(DEV), w.to(DEV), acc, accumulate=True, waves=waves, kc=kc)
+        assert rel_err(acc, want + base.double()) < 3e-6
+    else:
+        parts = torch.full((S, M, N), float("nan"), device=DEV)
+        ops.gemm_ring_bf16(a.to(DEV), w.to(DEV), parts, S, waves=waves, kc=kc)
+        assert torch.isfinite(parts).all()
+        assert rel_err(parts.sum(0), want) < 3e-6
+    # a row's result does not depend on the other rows of the batch, nor on how many there are
+    full = torch.empty(M, N, device=DEV)
+    ops.gemm_ring_bf16(a.to(DEV), w.to(DEV), full, waves=waves, kc=kc)
+    few = torch.empty(min(M, 3), N, device=DEV)
+    ops.gemm_ring_bf16(a[:min(M, 3)].contiguous().to(DEV), w.to(DEV), few, waves=waves, kc=kc)
+    assert torch.equal(few, full[:min(M, 3)])
+
+
+@pytest.mark.parametrize("waves,kc", [(4, 128), (8, 128), (8, 64)])
+@pytest.mark.parametrize("M,I,K", [(64, 128, 512), (40, 192, 256), (128, 64, 384), (20, 160, 128)])
+def test_gemm_ring_paired_silu(ops, waves, kc, M, I, K):
+    from torchless_rs_amd.parts.linear import interleave_pairs
+    a = rnd(M, K, seed=54, dtype=torch.bfloat16)
+    g = rnd(I, K, seed=55, dtype=torch.bfloat16, scale=0.3)
+    u = rnd(I, K, seed=56, dtype=torch.bfloat16, scale=0.3)
+    out = torch.full((M, I), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.gemm_ring_bf16(a.to(DEV), interleave_pairs(g, u).to(DEV), out, silu_pair=True, waves=waves, kc=kc)
+    want = plain.silu(a.double() @ g.double().t()) * (a.double() @ u.double().t())
+    assert rel_err(out, want) < KTOL["bfloat16"]
+    with pytest.raises(ops.KernelError, match="groups of four waves"):
+        ops.gemm_ring_bf16(a.to(DEV), interleave_pairs(g, u).to(DEV), out, silu_pair=True, waves=7)
+
+
+def test_gemm_ring_refuses_what_it_does_not_serve(ops):
+    a = torch.zeros(20, 200, dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros(64, 200, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(ops.KernelError, match="multiple of 128"):
+        ops.gemm_ring_bf16(a, w, torch.empty(20, 64, device=DEV))
+    a, w = torch.zeros(20, 256, dtype=torch.bfloat16, device=DEV), torch.zeros(64, 256, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(ops.KernelError, match="waves"):
+        ops.gemm_ring_bf16(a, w, torch.empty(20, 64, device=DEV), waves=5)
+    with pytest.raises(ops.KernelError, match="splits do not fit"):
+        ops.gemm_ring_bf16(a, w, torch.empty(3, 20, 64, device=DEV), n_split=3)
+    big = torch.zeros(129, 256, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(ops.KernelError, match="M at most"):
+        ops.gemm_ring_bf16(big, w, torch.empty(129, 64, device=DEV))
+
+
 def test_rope_commit_adds_partial_products(ops):
     from torchless_rs_amd.parts.position import Rotary
     nq, nkv, d = 6, 2, 48

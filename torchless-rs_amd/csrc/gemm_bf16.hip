@@ -27,6 +27,15 @@
 namespace tl {
 
 __device__ __forceinline__ bf16x8 load8(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
+// A load of weights that a step of at most 16 rows reads once: marked non-temporal.  A plain read of a
+// large buffer reaches 6.7 to 6.95 TB/s with such loads against 6.0 without (csrc/ceilings.hip); gate|up
+// at 8 rows went from 41.6 to 38.0 us, down from 21.9 to 20.4, o from 9.0 to 8.3.  Not for the kernels
+// whose cache lines are shared between load instructions or waves (gemm_mid: a decode step at batch 64
+// 11.9 against 10.85 ms; the keys and values of decode attention: 11.56 against 10.85 ms), and the fused
+// q|k|v kernel gains nothing from it.
+__device__ __forceinline__ bf16x8 load8_once(const bf16* p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(p));
+}
 __device__ __forceinline__ bf16x8 zero8() {
   bf16x8 z;
 #pragma unroll
@@ -157,11 +166,11 @@ gemm_skinny_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       if constexpr (TILED) {
-        wv[t][0] = load8(wrow[t] + (size_t)s * TILE_STEP);
-        wv[t][1] = load8(wrow[t] + (size_t)s * TILE_STEP + TILE_STEP / 2);
+        wv[t][0] = load8_once(wrow[t] + (size_t)s * TILE_STEP);
+        wv[t][1] = load8_once(wrow[t] + (size_t)s * TILE_STEP + TILE_STEP / 2);
       } else {
-        wv[t][0] = ok0 ? load8(wrow[t] + k) : zero8();
-        wv[t][1] = ok1 ? load8(wrow[t] + k + 8) : zero8();
+        wv[t][0] = ok0 ? load8_once(wrow[t] + k) : zero8();
+        wv[t][1] = ok1 ? load8_once(wrow[t] + k + 8) : zero8();
       }
     }
 #pragma unroll
@@ -351,7 +360,7 @@ gemm_rows_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float* 
     asm volatile("" : "+v"(off), "+v"(row_bytes));
 #pragma unroll
     for (int i = 0; i < 16; ++i)
-      w[i] = *reinterpret_cast<const bf16x8*>(reinterpret_cast<const char*>(base) + (off + i * row_bytes));
+      w[i] = load8_once(reinterpret_cast<const bf16*>(reinterpret_cast<const char*>(base) + (off + i * row_bytes)));
   };
   const bool scaled = ns.ssq_in != nullptr;
   RowFactors rf;
@@ -730,6 +739,198 @@ static int launch_mid(const bf16* A, const bf16* W, float* C, int M, int N, int 
   return 0;
 }
 
+// ------------------------------------------------------------------ ring ----
+// 17..128 rows when K is a multiple of 128: the same product as gemm_mid, with both operands going
+// from memory straight into a ring of stages in LDS (global_load_lds, 16 bytes a lane, no register in
+// between), several stages ahead of the matrix cores.  A stage is KC k (64 or 128): KC * 2 bytes of each
+// of the workgroup's channels (16 a wave) and of each row of activations.  A load instruction takes
+// whole runs of that length from four or eight rows (1 KB, which lands in LDS lane after lane); within a
+// row the 16-byte chunk c lies at a swizzled place, so that the operand reads of 16 lanes fall on 16
+// different groups of banks.  The compiler places no waits for such loads: the waves count them (vmcnt)
+// and meet at one barrier a stage.  The weights' loads are marked non-temporal (whole lines, read once).
+constexpr int RING_LDS = 156 * 1024;         // most LDS a workgroup takes
+constexpr int RING_W_AUX = 2;                // cache policy of the weights' loads: non-temporal
+
+template <int N> __device__ __forceinline__ void wait_loads_but() {       // until at most N loads are under way
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+#define TL_AS1 __attribute__((address_space(1)))
+#define TL_AS3 __attribute__((address_space(3)))
+
+template <int MT, int WAVES, int KC, int NS>
+__global__ void __launch_bounds__(WAVES * 64)
+gemm_ring_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float* __restrict__ C, int M, int N,
+                 int K, int stages_per_split, int epilogue) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char ring_smem[];
+  constexpr int ROWB = KC * 2;                              // bytes of a row in a stage
+  constexpr int RPI = 1024 / ROWB;                          // rows a load instruction takes
+  constexpr int CPR = ROWB / 16;                            // 16-byte chunks of a row
+  constexpr int W_INSTR = 16 / RPI;                         // loads of a wave's 16 channels
+  constexpr int A_BYTES = MT * 16 * ROWB, W_BYTES = WAVES * 16 * ROWB, STAGE = A_BYTES + W_BYTES;
+  constexpr int A_INSTR = MT * 16 / RPI;                    // loads of a stage's activations
+  constexpr int A_PER = (A_INSTR + WAVES - 1) / WAVES;      // a wave's share of them
+  constexpr int LPS = W_INSTR + A_PER;                      // loads a wave issues for a stage
+  constexpr int SPARE = NS * STAGE;                         // 1 KB that takes the loads of shares that do not exist
+  constexpr int STEPS = KC / 32;                            // matrix-core steps of a stage
+  static_assert(KC == 64 || KC == 128, "a stage is 64 or 128 k");
+  static_assert((NS - 2) * LPS <= 63 && NS >= 2, "the count of loads under way has six bits");
+  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64, li = lane % 16, kg = lane / 16;
+  const int n0 = blockIdx.x * (WAVES * 16) + wave * 16;
+  const int stages = K / KC;
+  const int t_begin = blockIdx.y * stages_per_split;
+  const int n_t = min(stages, t_begin + stages_per_split) - t_begin;
+  // chunk c of row r lies at place c ^ key(r) of the row: 16 lanes that read the same chunk of 16 rows
+  // then fall on 16 groups of banks (rows of 128 bytes lie two to a line of banks)
+  auto key = [](int r) { return CPR == 16 ? r % 16 : (r / 2) % 8; };
+
+  // this lane's sources: of load i of the weights (row RPI i + lane / CPR of the wave's 16) and of its
+  // shares of the activations
+  const int sub = lane / CPR, place = lane % CPR;
+  const char* wsrc[W_INSTR];
+#pragma unroll
+  for (int i = 0; i < W_INSTR; ++i) {
+    const int r = RPI * i + sub;
+    wsrc[i] = reinterpret_cast<const char*>(W + (size_t)min(n0 + r, N - 1) * K) + (size_t)t_begin * ROWB +
+              ((place ^ key(r)) * 16);
+  }
+  const char* asrc[A_PER];
+  int adst[A_PER];
+#pragma unroll
+  for (int x = 0; x < A_PER; ++x) {
+    const int q = wave + WAVES * x, r = RPI * q + sub;
+    asrc[x] = reinterpret_cast<const char*>(A + (size_t)min(r, M - 1) * K) + (size_t)t_begin * ROWB +
+              ((place ^ key(r)) * 16);
+    adst[x] = q < A_INSTR ? q * 1024 : -1;
+  }
+  auto issue = [&](int i) {                                 // stage i of this split into its place in the ring
+    unsigned char* slot = ring_smem + (i % NS) * STAGE;
+    const size_t off = (size_t)i * ROWB;
+#pragma unroll
+    for (int x = 0; x < A_PER; ++x) {
+      unsigned char* dst = adst[x] >= 0 ? slot + adst[x] : ring_smem + SPARE;
+      __builtin_amdgcn_global_load_lds((const TL_AS1 void*)(asrc[x] + off), (TL_AS3 void*)dst, 16, 0, 0);
+    }
+#pragma unroll
+    for (int j = 0; j < W_INSTR; ++j)
+      __builtin_amdgcn_global_load_lds((const TL_AS1 void*)(wsrc[j] + off),
+                                       (TL_AS3 void*)(slot + A_BYTES + wave * (16 * ROWB) + j * 1024), 16, 0,
+                                       RING_W_AUX);
+  };
+
+  f32x4 acc[MT];
+#pragma unroll
+  for (int u = 0; u < MT; ++u) acc[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+#pragma unroll
+  for (int i = 0; i < NS - 1; ++i)
+    if (i < n_t) issue(i);
+  const int kl = key(li);
+  for (int i = 0; i < n_t; ++i) {
+    // stage i has arrived for this wave when only the stages behind it are under way
+    if (n_t - 1 - i >= NS - 2) wait_loads_but<(NS - 2) * LPS>();
+    else wait_loads_but<0>();
+    __builtin_amdgcn_s_barrier();                           // ... and for all; everyone has left stage i - 1
+    if (i + NS - 1 < n_t) issue(i + NS - 1);                // into the place of stage i - 1
+    const unsigned char* slot = ring_smem + (i % NS) * STAGE;
+    const unsigned char* wrow = slot + A_BYTES + wave * (16 * ROWB) + li * ROWB;
+    // all operands of the stage are asked for before the first product: a wave is alone on its SIMD, and
+    // nothing else hides the way from LDS
+    bf16x8 wreg[STEPS], areg[MT][STEPS];
+#pragma unroll
+    for (int j = 0; j < STEPS; ++j) wreg[j] = *reinterpret_cast<const bf16x8*>(wrow + (((4 * j + kg) ^ kl) * 16));
+#pragma unroll
+    for (int u = 0; u < MT; ++u)
+#pragma unroll
+      for (int j = 0; j < STEPS; ++j)
+        areg[u][j] = *reinterpret_cast<const bf16x8*>(slot + (u * 16 + li) * ROWB + (((4 * j + kg) ^ kl) * 16));
+#pragma unroll
+    for (int u = 0; u < MT; ++u)
+#pragma unroll
+      for (int j = 0; j < STEPS; ++j)
+        acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(areg[u][j], wreg[j], acc[u], 0, 0, 0);
+  }
+  // acc[u][r] = D[m = 16 u + 4 kg + r][n = n0 + li]
+  if (epilogue == EPI_SILU_PAIR) {
+    // the workgroup's channels are groups of 64: of a group's four waves, the first two hold gate
+    // rows, the other two their up rows
+    __builtin_amdgcn_s_barrier();                           // the ring is free
+    float* ex = reinterpret_cast<float*>(ring_smem);        // [up wave][MT][4][64] floats
+    const int grp = wave / 4, wq = wave % 4;
+    if (wq >= 2) {
+#pragma unroll
+      for (int u = 0; u < MT; ++u)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) ex[(((grp * 2 + wq - 2) * MT + u) * 4 + r) * 64 + lane] = acc[u][r];
+    }
+    __syncthreads();
+    if (wq < 2) {
+      bf16* H = reinterpret_cast<bf16*>(C);
+      const int NH = N / 2;
+      const int n = (blockIdx.x * (WAVES / 4) + grp) * 32 + wq * 16 + li;
+#pragma unroll
+      for (int u = 0; u < MT; ++u)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int m = 16 * u + 4 * kg + r;
+          if (m < M && n < NH) {
+            const float g = acc[u][r], up = ex[(((grp * 2 + wq) * MT + u) * 4 + r) * 64 + lane];
+            H[(size_t)m * NH + n] = (bf16)((g / (1.0f + expf(-g))) * up);
+          }
+        }
+    }
+    return;
+  }
+  float* dst = C + (size_t)blockIdx.y * M * N;              // the split's own partial (split 0: C itself)
+  const int n = n0 + li;
+  if (n < N) {
+#pragma unroll
+    for (int u = 0; u < MT; ++u)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int m = 16 * u + 4 * kg + r;
+        if (m < M) {
+          float* c = dst + (size_t)m * N + n;
+          *c = (epilogue == EPI_ACCUMULATE) ? *c + acc[u][r] : acc[u][r];
+        }
+      }
+  }
+}
+
+template <int MT, int WAVES, int KC>
+static int launch_ring(const bf16* A, const bf16* W, float* C, int M, int N, int K, int n_split, int epilogue,
+                       hipStream_t st) {
+  constexpr int STAGE = (MT + WAVES) * 16 * KC * 2;
+  constexpr int FIT = (RING_LDS - 1024) / STAGE;
+  constexpr int NS = FIT > 8 ? 8 : FIT;
+  static_assert(NS >= 2, "two stages at least");
+  constexpr int LDS = NS * STAGE + 1024;
+  static bool raised = false;
+  if (!raised) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_ring_kernel<MT, WAVES, KC, NS>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+    if (e != hipSuccess) {
+      set_error("gemm_ring: cannot have %d bytes of LDS: %s", LDS, hipGetErrorString(e));
+      return 2;
+    }
+    raised = true;
+  }
+  const int stages = K / KC, per = (stages + n_split - 1) / n_split;
+  dim3 grid((N + WAVES * 16 - 1) / (WAVES * 16), n_split);
+  gemm_ring_kernel<MT, WAVES, KC, NS><<<grid, WAVES * 64, LDS, st>>>(A, W, C, M, N, K, per, epilogue);
+  TL_LAUNCH_CHECK("gemm_ring");
+  return 0;
+}
+
+template <int WAVES, int KC>
+static int launch_ring_rows(const bf16* A, const bf16* W, float* C, int M, int N, int K, int n_split, int epilogue,
+                            hipStream_t st) {
+  if (M <= 32) return launch_ring<2, WAVES, KC>(A, W, C, M, N, K, n_split, epilogue, st);
+  if (M <= 64) return launch_ring<4, WAVES, KC>(A, W, C, M, N, K, n_split, epilogue, st);
+  if (M <= 96) return launch_ring<6, WAVES, KC>(A, W, C, M, N, K, n_split, epilogue, st);
+  return launch_ring<8, WAVES, KC>(A, W, C, M, N, K, n_split, epilogue, st);
+}
+
 }  // namespace tl
 
 using namespace tl;
@@ -807,11 +1008,16 @@ extern "C" int tl_gemm_bf16_variant(const void* A, const void* W, void* C, int M
   TL_REQUIRE(false, "gemm_bf16: unknown variant %d", variant);
 }
 
+extern "C" int tl_gemm_ring_bf16(const void* A, const void* W, void* C, int M, int N, int K, int n_split,
+                                 int epilogue, int waves, int kc, hipStream_t st);
+
 // 17..128 rows.  n_split == 1: C as in tl_gemm_bf16 (all three epilogues).  n_split > 1: C is
-// float [n_split][M][N] and receives partial sums (epilogue must be 0); every split gets at
-// least one k-step of 256.
+// float [n_split][M][N] and receives partial sums (epilogue must be 0).  K a multiple of 128: the
+// ring kernel, 8 waves (128 channels) a workgroup, stages of 128 k, every split with one stage at
+// least; other K: gemm_mid, every split with one k-step of 256 at least.
 extern "C" int tl_gemm_mid_bf16(const void* A, const void* W, void* C, int M, int N, int K, int n_split,
                                 int epilogue, hipStream_t st) {
+  if (K > 0 && K % 128 == 0) return tl_gemm_ring_bf16(A, W, C, M, N, K, n_split, epilogue, 8, 128, st);
   TL_REQUIRE(M > 0 && M <= MID_ROWS && N > 0 && K > 0 && K % 8 == 0, "gemm_mid: bad sizes M=%d N=%d K=%d (M at most "
              "%d, K a multiple of 8)", M, N, K, MID_ROWS);
   TL_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "gemm_mid: operands must be 16-byte aligned");
@@ -832,6 +1038,35 @@ extern "C" int tl_gemm_mid_bf16(const void* A, const void* W, void* C, int M, in
   if (M <= 96) return launch_mid<6>(a, w, c, M, N, K, n_split, epilogue, st);
   if (M <= 112) return launch_mid<7>(a, w, c, M, N, K, n_split, epilogue, st);
   return launch_mid<8>(a, w, c, M, N, K, n_split, epilogue, st);
+}
+
+// The same product through the ring kernel (see gemm_ring_kernel): K a multiple of 128.  waves: the waves of a
+// workgroup, each with 16 channels: 4, 7 or 8 (the paired epilogue needs whole groups of 64 channels: 4 or 8);
+// kc: the k of a stage, 64 or 128.
+extern "C" int tl_gemm_ring_bf16(const void* A, const void* W, void* C, int M, int N, int K, int n_split,
+                                 int epilogue, int waves, int kc, hipStream_t st) {
+  TL_REQUIRE(M > 0 && M <= MID_ROWS && N > 0 && K > 0 && K % 128 == 0, "gemm_ring: bad sizes M=%d N=%d K=%d (M at "
+             "most %d, K a multiple of 128)", M, N, K, MID_ROWS);
+  TL_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "gemm_ring: operands must be 16-byte aligned");
+  TL_REQUIRE(kc == 64 || kc == 128, "gemm_ring: a stage of %d k (64 or 128)", kc);
+  TL_REQUIRE(n_split >= 1 && n_split <= K / kc && n_split <= 65535,
+             "gemm_ring: %d splits do not fit K=%d (one stage of %d at least each)", n_split, K, kc);
+  TL_REQUIRE(epilogue >= 0 && epilogue <= 2 && (n_split == 1 || epilogue == EPI_STORE),
+             "gemm_ring: epilogue %d cannot go with %d splits", epilogue, n_split);
+  TL_REQUIRE(epilogue != EPI_SILU_PAIR || (N % 64 == 0 && waves % 4 == 0), "gemm_ring: the paired epilogue needs N=%d "
+             "to be a multiple of 64 and whole groups of four waves (%d)", N, waves);
+  const bf16* a = (const bf16*)A;
+  const bf16* w = (const bf16*)W;
+  float* c = (float*)C;
+#define TL_RING(WV)                                                                                     \
+  if (waves == WV)                                                                                      \
+    return kc == 64 ? launch_ring_rows<WV, 64>(a, w, c, M, N, K, n_split, epilogue, st)                 \
+                    : launch_ring_rows<WV, 128>(a, w, c, M, N, K, n_split, epilogue, st)
+  TL_RING(4);
+  TL_RING(7);
+  TL_RING(8);
+#undef TL_RING
+  TL_REQUIRE(false, "gemm_ring: %d waves a workgroup (4, 7 or 8)", waves);
 }
 
 // q|k|v of a step with one token a sequence (row m is sequence m, at position row_pos[m]):

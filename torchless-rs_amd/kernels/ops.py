@@ -448,7 +448,15 @@ def gemm_bf16_norm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumula
     return groups.value
 
 
-MID_ROWS = 128      # most rows of the kernel that shares a k-step's activations through LDS
+MID_ROWS = 128      # most rows of the kernels that share a step's activations through LDS
+RING_K = 128        # the kernel that brings both operands into a ring of LDS stages takes K in multiples of this
+LIBRARY_ROWS = 64   # where K is no such multiple, the BLAS library's product beats ours above this many rows
+
+
+def own_rows(K: int) -> int:
+    """The most rows for which a bfloat16 product over K runs in this package's own kernels (more
+    go to the BLAS library)."""
+    return MID_ROWS if K % RING_K == 0 else LIBRARY_ROWS
 
 
 _UNITS: dict = {}
@@ -463,12 +471,19 @@ def compute_units(device) -> int:
 
 
 def mid_splits(M: int, N: int, K: int, units: int) -> int:
-    """For 17..MID_ROWS rows: into how many slices K is cut so that some 400
-    workgroups or more (64 output channels each) are at work, a power of two
-    (which shares the k-steps out evenly at the usual sizes; measured best at
-    the 7B sizes); 1 where N alone gives them.  Twice as many where only that fills
-    the `units` compute units evenly (5,120 channels: 80 x 16 workgroups are 5 a
-    unit, 80 x 8 two and a half; down at 128 rows 50.6 against 56.7 us)."""
+    """For 17..MID_ROWS rows: into how many slices K is cut, each a workgroup's own, whose partial
+    sums the next kernel adds up; 1 where N alone gives the workgroups.
+
+    K a multiple of RING_K (the ring kernel: 128 channels a workgroup, which holds a compute unit by
+    itself): as many slices as make one round of workgroups over the `units` compute units, each
+    with four stages of 128 k at least (o and down of the 7B shape at 64 rows: 8 slices, 256
+    workgroups, 9.4 and 22.2 us; q|k|v: 5).
+
+    Other K (gemm_mid: 64 channels a workgroup, steps of 256 k): so that some 400 workgroups or more
+    are at work, a power of two; twice as many where only that fills the compute units evenly."""
+    if K % RING_K == 0:
+        blocks = -(-N // 128)
+        return max(1, min(units // blocks, (K // RING_K) // 4, 16))
     blocks = -(-N // 64)
     steps = -(-K // 256)
     want = -(-400 // blocks)
@@ -484,9 +499,10 @@ def mid_splits(M: int, N: int, K: int, units: int) -> int:
 
 def gemm_mid_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, n_split: int = 1,
                   accumulate: bool = False, silu_pair: bool = False) -> None:
-    """The product for 17..MID_ROWS rows.  n_split == 1: out as in `gemm_bf16`.
-    n_split > 1: out is float32 [n_split, M, N] and receives partial sums that
-    the next kernel adds up (`add_rmsnorm`, `add_partials`, `rope_commit`)."""
+    """The product for 17..MID_ROWS rows (the ring kernel where K is a multiple of RING_K, else
+    gemm_mid).  n_split == 1: out as in `gemm_bf16`.  n_split > 1: out is float32 [n_split, M, N]
+    and receives partial sums that the next kernel adds up (`add_rmsnorm`, `add_partials`,
+    `rope_commit`)."""
     M, K = a.shape
     N = w.shape[0]
     _req(a, "gemm.a", torch.bfloat16)
@@ -503,6 +519,29 @@ def gemm_mid_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, n_split: 
         _req(out, "gemm.out", torch.float32, (M, N))
         epi = EPI_ACCUMULATE if accumulate else EPI_STORE
     _check(lib().tl_gemm_mid_bf16(_p(a), _p(w), _p(out), M, N, K, int(n_split), epi, _stream()))
+
+
+def gemm_ring_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, n_split: int = 1, accumulate: bool = False,
+                   silu_pair: bool = False, waves: int = 4, kc: int = 128) -> None:
+    """`gemm_mid_bf16` through the kernel that brings both operands into a ring of stages in LDS
+    (K a multiple of 128); `waves`: 4, 7 or 8 waves a workgroup with 16 channels each; `kc`: the k
+    of a stage, 64 or 128."""
+    M, K = a.shape
+    N = w.shape[0]
+    _req(a, "gemm.a", torch.bfloat16)
+    _req(w, "gemm.w", torch.bfloat16, (N, K))
+    if n_split > 1:
+        if accumulate or silu_pair:
+            raise KernelError("gemm_ring: partial sums cannot be accumulated or paired")
+        _req(out, "gemm.out", torch.float32, (n_split, M, N))
+        epi = EPI_STORE
+    elif silu_pair:
+        _req(out, "gemm.out", torch.bfloat16, (M, N // 2))
+        epi = EPI_SILU_PAIR
+    else:
+        _req(out, "gemm.out", torch.float32, (M, N))
+        epi = EPI_ACCUMULATE if accumulate else EPI_STORE
+    _check(lib().tl_gemm_ring_bf16(_p(a), _p(w), _p(out), M, N, K, int(n_split), epi, int(waves), int(kc), _stream()))
 
 
 def add_rmsnorm(x: torch.Tensor, parts: torch.Tensor, w: torch.Tensor, eps: float, out: torch.Tensor) -> None:
@@ -526,10 +565,6 @@ def add_partials(x: torch.Tensor, parts: torch.Tensor) -> None:
     if parts.dim() != 3 or tuple(parts.shape[1:]) != (n, H):
         raise KernelError(f"add_partials.parts: shape {tuple(parts.shape)}, kernel needs [S, {n}, {H}]")
     _check(lib().tl_add_partials(_p(x), _p(parts), parts.shape[0], n, H, _stream()))
-
-
-LIBRARY_ROWS = 64           # above this many rows the library's product beats ours (measured at the 7B sizes),
-                            # but for small N up to MID_ROWS rows, where ours wins with K cut into partial sums
 
 
 def gemm_library(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False) -> None:
@@ -562,11 +597,13 @@ def gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool =
          tiles: Optional[torch.Tensor] = None) -> None:
     """out[M,N] (+)= a[M,K] @ w[N,K]^T with float32 accumulation.  The kernel
     follows from the operand types: bfloat16 x bfloat16 goes to the matrix
-    cores (our kernels up to LIBRARY_ROWS rows, the library's above), anything
+    cores (our kernels up to `own_rows(K)` rows, the library's above), anything
     with float32 in it to the plain FMA kernel.  `tiles`: see `gemm_bf16`."""
     if bf16_gemm_ok(a, w):
-        if a.shape[0] > LIBRARY_ROWS:
+        if a.shape[0] > own_rows(a.shape[1]):
             gemm_library(a, w, out, accumulate)
+        elif a.shape[0] > LIBRARY_ROWS:
+            gemm_mid_bf16(a, w, out, 1, accumulate)
         else:
             gemm_bf16(a, w, out, accumulate, tiles=tiles)
     else:

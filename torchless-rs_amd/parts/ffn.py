@@ -67,7 +67,7 @@ class SwiGLU(FeedForward):
         factor = take_row_factor(ctx, usable=self.paired and ops.norm_split_ok(y, self.gate_up.weight))
         if factor is not None:
             ops.gemm_bf16_norm(y, self.gate_up.weight, h, silu_pair=True, factor=factor)
-        elif self.paired and n <= ops.LIBRARY_ROWS and self.gate_up.mid(y):
+        elif self.paired and self.gate_up.mid(y):
             ops.gemm_mid_bf16(y, self.gate_up.weight, h, 1, silu_pair=True)
         elif self.paired and ops.bf16_gemm_ok(y, self.gate_up.weight):
             if n > ops.LIBRARY_ROWS:

@@ -52,7 +52,7 @@ class Linear:
         second half of the norm that made `a`, a factor per row (at most 16 rows)."""
         if factor is not None:
             ops.gemm_bf16_norm(a, self.weight, out, accumulate, factor=factor, tiles=self.tiles)
-        elif self.mid(a) and a.shape[0] <= ops.LIBRARY_ROWS:
+        elif self.mid(a):
             ops.gemm_mid_bf16(a, self.weight, out, 1, accumulate)
         else:
             ops.gemm(a, self.weight, out, accumulate, tiles=self.tiles)
@@ -60,13 +60,12 @@ class Linear:
     def own_kernels(self, n_rows: int) -> bool:
         """Does a product of `n_rows` rows launch this package's kernels only (never the BLAS
         library's, which a captured graph must not hold)?"""
-        return n_rows <= ops.LIBRARY_ROWS or self.weight.dtype != torch.bfloat16
+        return n_rows <= ops.own_rows(self.in_features) or self.weight.dtype != torch.bfloat16
 
     def mid(self, a: torch.Tensor) -> bool:
-        """17..MID_ROWS rows of bfloat16: the kernel that shares the activations.
-        (Above LIBRARY_ROWS rows it beats the library only with K cut into
-        partial sums, which `partial` does.)"""
-        return 16 < a.shape[0] <= ops.MID_ROWS and ops.bf16_gemm_ok(a, self.weight)
+        """17..`ops.own_rows(K)` rows of bfloat16: the kernels that share the activations
+        through LDS."""
+        return 16 < a.shape[0] <= ops.own_rows(self.in_features) and ops.bf16_gemm_ok(a, self.weight)
 
     def partial(self, a: torch.Tensor, ctx, name: str):
         """The product as partial sums [S, M, N] (float32) for a reader that adds
