@@ -26,15 +26,20 @@ def test_mid_splits_fit():
 
 def test_decode_splits_follow_batch_and_length():
     assert ops.decode_groups(8, 32, 8) == 64 and ops.decode_groups(1, 34, 2) == 4      # 17 heads a group: two tiles
+    # heads of 128 (and 64): the kernel that stages pages in LDS, two workgroups a compute unit
+    assert ops.decode_workgroups_per_unit(128) == 2 and ops.decode_workgroups_per_unit(64) == 2
+    assert ops.decode_workgroups_per_unit(256) == 1 and ops.decode_workgroups_per_unit(96) == 1
+    assert ops.decode_workgroups_per_unit(32) == 4 and ops.decode_workgroups_per_unit(48) == 2
     assert ops.decode_splits(64, 32, 8, 32, 256, 128) == 1            # enough workgroups without a cut
-    assert ops.decode_splits(32, 32, 8, 65, 256, 128) == 1            # one workgroup a compute unit already
-    assert ops.decode_splits(8, 32, 8, 65, 256, 128) == 4             # 64 groups: four parts are one workgroup a unit
-    assert ops.decode_splits(16, 32, 8, 65, 256, 128) == 2
-    assert ops.decode_splits(3, 32, 8, 65, 256, 128) == 10            # 24 groups: 11 parts would start a second round
-    assert ops.decode_splits(20, 32, 8, 65, 256, 128) == 3            # 160 groups: two rounds of thirds beat one of wholes
+    assert ops.decode_splits(32, 32, 8, 65, 256, 128) == 2            # 256 groups: two parts are two workgroups a unit
+    assert ops.decode_splits(8, 32, 8, 65, 256, 128) == 8             # 64 groups: eight parts fill the round of 512
+    assert ops.decode_splits(16, 32, 8, 65, 256, 128) == 4
+    assert ops.decode_splits(3, 32, 8, 65, 256, 128) == 17            # 24 groups: at least four pages a part
+    assert ops.decode_splits(20, 32, 8, 65, 256, 128) == 3            # 160 groups: 480 workgroups in one round
     assert ops.decode_splits(1, 32, 8, 64, 256, 128) == 16            # at least four pages a part
-    assert ops.decode_splits(1, 32, 8, 513, 256, 128) == 31           # a long context: one round of workgroups, 17 pages each
-    assert ops.decode_splits(8, 32, 8, 65, 128, 128) == 2  # by the device's compute units
+    assert ops.decode_splits(1, 32, 8, 513, 256, 128) == 57           # a long context: one round of workgroups, 9 pages each
+    assert ops.decode_splits(8, 32, 8, 65, 128, 128) == 4             # by the device's compute units
+    assert ops.decode_splits(8, 32, 8, 65, 256, 96) == 4              # a head size of the kernel that reads into registers: one a unit
     assert ops.decode_splits(8, 32, 8, 65, 256, 64) == 8 and ops.decode_splits(32, 16, 4, 64, 256, 32) == 8   # small heads: more workgroups a unit
     assert ops.decode_splits(1, 32, 8, 1, 256, 128) == 1
     for B in (1, 3, 8, 64):

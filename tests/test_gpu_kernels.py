@@ -485,18 +485,44 @@ def test_attention_prefill_bf16(ops, nq, nkv, d, window):
     assert rel_err(a["out"], plain_out.double()) < KTOL["bfloat16"]
 
 
+@pytest.mark.parametrize("through_lds", [True, False])
 @pytest.mark.parametrize("splits", [1, 3, 8])
 @pytest.mark.parametrize("nq,nkv,d,window", SHAPES)
-def test_attention_decode_bf16(ops, nq, nkv, d, window, splits):
+def test_attention_decode_bf16(ops, nq, nkv, d, window, splits, through_lds):
+    """Both decode kernels: the one that stages whole pages in LDS (head sizes 64, 128, 256) and the one that
+    reads them into registers (every head size; the switch sends those three through it too)."""
+    if not through_lds and d not in (64, 128, 256):
+        pytest.skip("this head size has one kernel")
     lens = [0, 63, 64, 300, 191, 31, 32, 700]
     a = paged_case(ops, "bfloat16", nq, nkv, d, window, lens_cached=lens, lens_new=[1] * len(lens), seed=3,
                    n_pages=60)
     ops.kv_commit(a["k"], a["v"], a["row_seq"], a["row_pos"], a["after"], a["table"], a["ring"], a["pages"])
     B = len(lens)
     part = torch.full((B * nq * splits * (d + 2),), float("nan"), device=DEV)
-    ops.attn_decode_bf16(a["q"], a["pages"], a["table"], a["ring"], a["row_pos"], window, a["scale"], splits,
-                         part, a["out"])
+    was = ops.decode_through_lds(through_lds)
+    try:
+        ops.attn_decode_bf16(a["q"], a["pages"], a["table"], a["ring"], a["row_pos"], window, a["scale"], splits,
+                             part, a["out"])
+    finally:
+        ops.decode_through_lds(was)
+    assert was is True                                     # the default
     assert rel_err(a["out"], a["want"]) < KTOL["bfloat16"]
+
+
+def test_attention_decode_through_lds_over_many_pages(ops):
+    """More than 64 pages to one workgroup (its page ids are fetched 64 at a time), a ring that wraps, a window
+    that begins inside a page, and stale rows of NaN behind every sequence's end."""
+    nq, nkv, d = 8, 2, 128
+    for window, lens in ((None, [4500, 64 * 70 - 1, 1]), (2100, [4500, 2099, 2200])):
+        a = paged_case(ops, "bfloat16", nq, nkv, d, window, lens_cached=lens, lens_new=[1] * len(lens), seed=9,
+                       n_pages=230)
+        ops.kv_commit(a["k"], a["v"], a["row_seq"], a["row_pos"], a["after"], a["table"], a["ring"], a["pages"])
+        for splits in (1, 2):
+            part = torch.full((len(lens) * nq * splits * (d + 2),), float("nan"), device=DEV)
+            out = torch.full_like(a["out"], float("nan"))
+            ops.attn_decode_bf16(a["q"], a["pages"], a["table"], a["ring"], a["row_pos"], window, a["scale"], splits,
+                                 part, out)
+            assert rel_err(out, a["want"]) < KTOL["bfloat16"], (window, splits)
 
 
 def test_attention_bf16_far_key_and_edge(ops):

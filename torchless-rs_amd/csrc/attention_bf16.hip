@@ -558,6 +558,220 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
   }
 }
 
+// ------------------------------------------------------ decode, through LDS --
+// The same step for head sizes 64, 128 and 256, with the pages going from memory straight into a
+// ring of stages in LDS (global_load_lds, 16 bytes a lane), several pages ahead of the matrix cores.
+// A stage is one page of one KV head: its keys [64][d] and its values [d][64], each one run of
+// memory, so that every load instruction takes 1 KB of whole lines, which may then be marked
+// non-temporal (a plain read gains a seventh from that, csrc/ceilings.hip; with the loads of
+// attn_decode_kernel, which take a line in halves, it loses).  The workgroup's four waves take 16
+// keys of the page each: S^T = K Q^T (16x16x32), softmax with the wave's own running maximum,
+// O^T += V^T P (16x16x16: the scores leave the first product in the second's operand layout).
+// In LDS the 16-byte chunk c of a row lies at a swizzled place, so that the operand reads of 16
+// lanes fall on 16 groups of banks.  The compiler places no waits for such loads: the waves count
+// them (vmcnt) and meet at one barrier a page.  Partial results as attn_decode_kernel writes them.
+#define TL_AS1 __attribute__((address_space(1)))
+#define TL_AS3 __attribute__((address_space(3)))
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+template <int N> __device__ __forceinline__ void wait_page_loads_but() {     // until at most N loads are under way
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+template <int D, int NS>
+__global__ void __launch_bounds__(DC_WAVES * 64)
+attn_decode_ring_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
+                        const int* __restrict__ table, int table_stride, int ring_pages,
+                        const int* __restrict__ row_pos, int nq, int nkv, int window, float scale,
+                        int n_splits, int head_groups, float* __restrict__ part, bf16* __restrict__ out) {
+  extern __shared__ __attribute__((aligned(1024))) unsigned char dr_smem[];
+  constexpr int KB = D / 32, VB = D / 16;
+  constexpr int K_BYTES = PAGE * D * 2, STAGE = 2 * K_BYTES;   // keys, then values, as many bytes each
+  constexpr int K_CPR = D / 8;                        // 16-byte chunks of a key's row
+  constexpr int K_RPI = 64 / K_CPR;                   // keys a load instruction takes
+  constexpr int K_INSTR = PAGE / K_RPI, V_INSTR = D / 8;       // (a load of values takes 8 rows of 128 bytes)
+  constexpr int LPS = (K_INSTR + V_INSTR) / DC_WAVES; // loads a wave issues for a page
+  static_assert(D == 64 || D == 128 || D == 256, "head sizes whose rows have a power of two of chunks");
+  static_assert((K_INSTR + V_INSTR) % DC_WAVES == 0 && (NS - 2) * LPS <= 63 && NS >= 2, "loads a wave counts");
+  const int g = nq / nkv;
+  const int hg = blockIdx.x % head_groups;
+  const int kvh = (blockIdx.x / head_groups) % nkv;
+  const int b = blockIdx.x / (head_groups * nkv);
+  const int split = blockIdx.y;
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64, li = lane % 16, kg = lane / 16;
+  const int hl = hg * 16 + li;
+  const int h = kvh * g + min(hl, g - 1);
+  const int p = row_pos[b];
+  const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  const int pg_lo = lo / PAGE, pg_hi = p / PAGE, n_pg = pg_hi - pg_lo + 1;
+  const int my_lo = pg_lo + (int)((long long)split * n_pg / n_splits);
+  const int my_hi = pg_lo + (int)((long long)(split + 1) * n_pg / n_splits);
+  const int n_st = my_hi - my_lo;                     // this split's pages: the stages
+  const size_t head_elems = (size_t)PAGE * D, page_elems = 2 * (size_t)nkv * head_elems;
+  auto kkey = [](int r) { return K_CPR >= 16 ? r % 16 : (r / 2) % 8; };   // swizzle of a key's row
+  auto vkey = [](int r) { return (r / 2) % 8; };                          // ... of a row of values (128 bytes)
+
+  bf16x8 qreg[KB];
+  {
+    const bf16* qp = q + ((size_t)b * nq + h) * D;
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb) qreg[kb] = ld8(qp + kb * 32 + 8 * kg);
+  }
+  // this lane's share of a page's loads: where in the page's keys or values (bytes from the KV head's keys)
+  unsigned src_off[LPS];
+#pragma unroll
+  for (int x = 0; x < LPS; ++x) {
+    const int i = wave + DC_WAVES * x;
+    if (i < K_INSTR) {
+      const int r = i * K_RPI + lane / K_CPR, place = lane % K_CPR;
+      src_off[x] = (unsigned)(r * (2 * D) + ((place ^ kkey(r)) * 16));
+    } else {
+      const int r = (i - K_INSTR) * 8 + lane / 8, place = lane % 8;
+      src_off[x] = (unsigned)((size_t)nkv * head_elems * 2 + r * 128 + ((place ^ vkey(r)) * 16));
+    }
+  }
+  // the page ids of this split's stages lie in LDS behind the ring (a load from memory inside the loop
+  // would make the compiler wait for every load under way, the pages' among them)
+  int* ids = reinterpret_cast<int*>(dr_smem + NS * STAGE);
+  {
+    const int* trow = table + (size_t)b * table_stride;
+    for (int st = threadIdx.x; st < n_st; st += DC_WAVES * 64) ids[st] = trow[(my_lo + st) % ring_pages];
+  }
+  __syncthreads();
+  auto issue = [&](int st) {
+    const int page = __builtin_amdgcn_readfirstlane(ids[st]);
+    const char* base = reinterpret_cast<const char*>(pages + (size_t)page * page_elems + (size_t)kvh * head_elems);
+    unsigned char* slot = dr_smem + (st % NS) * STAGE;
+#pragma unroll
+    for (int x = 0; x < LPS; ++x)
+      __builtin_amdgcn_global_load_lds((const TL_AS1 void*)(base + src_off[x]),
+                                       (TL_AS3 void*)(slot + (wave + DC_WAVES * x) * 1024), 16, 0, 2);
+  };
+
+  f32x4 o[VB];
+#pragma unroll
+  for (int vb = 0; vb < VB; ++vb) o[vb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+
+#pragma unroll
+  for (int st = 0; st < NS - 1; ++st)
+    if (st < n_st) issue(st);
+  const int krow = 16 * wave + li;                    // this lane's key of a page (row of the first product)
+  const int kk = kkey(krow), vk = vkey(li);           // (16 vb + li has li's swizzle: 16 rows are a whole period)
+  for (int st = 0; st < n_st; ++st) {
+    if (n_st - 1 - st >= NS - 2) wait_page_loads_but<(NS - 2) * LPS>();
+    else wait_page_loads_but<0>();
+    __builtin_amdgcn_s_barrier();                     // the page is there for all; everyone has left the one before
+    if (st + NS - 1 < n_st) issue(st + NS - 1);
+    const int j0 = (my_lo + st) * PAGE + 16 * wave;   // this wave's 16 keys
+    if (j0 > p || j0 + 15 < lo) continue;             // none of them visible
+    const unsigned char* slot = dr_smem + (st % NS) * STAGE;
+    bf16x8 kreg[KB];
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb)
+      kreg[kb] = *reinterpret_cast<const bf16x8*>(slot + krow * (2 * D) + (((4 * kb + kg) ^ kk) * 16));
+    s16x4 vreg[VB];
+#pragma unroll
+    for (int vb = 0; vb < VB; ++vb)
+      vreg[vb] = *reinterpret_cast<const s16x4*>(slot + K_BYTES + (16 * vb + li) * 128 +
+                                                 (((2 * wave + kg / 2) ^ vk) * 16) + 8 * (kg % 2));
+    f32x4 s = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[kb], qreg[kb], s, 0, 0, 0);
+    // s[r]: key j0 + 4 kg + r against head li
+    float sv[4];
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int j = j0 + 4 * kg + r;
+      sv[r] = (j <= p && j >= lo) ? s[r] * scale : -INFINITY;
+      tmax = fmaxf(tmax, sv[r]);
+    }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, WAVE));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
+    const float m_new = fmaxf(m, tmax);               // finite: one of the 16 keys is visible
+    const float alpha = __expf(m - m_new);
+    float psum = 0.f;
+    bf16x4 pb;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float pv = __expf(sv[r] - m_new);
+      psum += pv;
+      pb[r] = (bf16)pv;
+    }
+    psum += __shfl_xor(psum, 16, WAVE);
+    psum += __shfl_xor(psum, 32, WAVE);
+    l = l * alpha + psum;
+    m = m_new;
+    if (j0 + 15 > p) {                                // rows past the sequence's end were never written: 0 * garbage
+      typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+      u32x2 keep;
+#pragma unroll
+      for (int w2 = 0; w2 < 2; ++w2)
+        keep[w2] = (j0 + 4 * kg + 2 * w2 <= p ? 0x0000ffffu : 0u) | (j0 + 4 * kg + 2 * w2 + 1 <= p ? 0xffff0000u : 0u);
+#pragma unroll
+      for (int vb = 0; vb < VB; ++vb)
+        vreg[vb] = __builtin_bit_cast(s16x4, __builtin_bit_cast(u32x2, vreg[vb]) & keep);
+    }
+    if (__ballot(alpha != 1.0f) != 0ull) {
+#pragma unroll
+      for (int vb = 0; vb < VB; ++vb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[vb][r] *= alpha;
+    }
+    const s16x4 pbits = __builtin_bit_cast(s16x4, pb);
+#pragma unroll
+    for (int vb = 0; vb < VB; ++vb) o[vb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vreg[vb], pbits, o[vb], 0, 0, 0);
+  }
+  // o[vb][r] = O[dv = 16 vb + 4 kg + r][head li]; m, l are per head li (equal in the 4 kg lanes).
+  // Merge the waves in the ring's memory: common maximum, then every wave's scaled share.
+  __builtin_amdgcn_s_barrier();                       // everyone has left the last page
+  float* red_o = reinterpret_cast<float*>(dr_smem);                              // [waves][VB * 4 * 64]
+  float* red_ml = red_o + DC_WAVES * VB * 4 * 64;                               // [waves][2][16]
+  if (kg == 0) {
+    red_ml[(wave * 2 + 0) * 16 + li] = m;
+    red_ml[(wave * 2 + 1) * 16 + li] = l;
+  }
+  __syncthreads();
+  float mm = -INFINITY;
+#pragma unroll
+  for (int w = 0; w < DC_WAVES; ++w) mm = fmaxf(mm, red_ml[(w * 2) * 16 + li]);
+  const float f = (m == -INFINITY) ? 0.f : __expf(m - mm);
+#pragma unroll
+  for (int vb = 0; vb < VB; ++vb)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) red_o[wave * (VB * 4 * 64) + (vb * 4 + r) * 64 + lane] = o[vb][r] * f;
+  __syncthreads();
+  for (int e = threadIdx.x; e < 16 * D; e += DC_WAVES * 64) {
+    const int hd = e / D, dv = e % D;
+    if (hg * 16 + hd >= g) continue;
+    float mh = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < DC_WAVES; ++w) mh = fmaxf(mh, red_ml[(w * 2) * 16 + hd]);
+    float ll = 0.f;
+#pragma unroll
+    for (int w = 0; w < DC_WAVES; ++w) {
+      const float mw = red_ml[(w * 2) * 16 + hd];
+      ll += (mw == -INFINITY) ? 0.f : red_ml[(w * 2 + 1) * 16 + hd] * __expf(mw - mh);
+    }
+    const int idx = ((dv / 16) * 4 + (dv % 4)) * 64 + ((dv % 16) / 4) * 16 + hd;
+    float osum = red_o[idx];
+#pragma unroll
+    for (int w = 1; w < DC_WAVES; ++w) osum += red_o[w * (VB * 4 * 64) + idx];
+    const size_t bh = (size_t)b * nq + kvh * g + hg * 16 + hd;
+    if (n_splits == 1) {
+      out[bh * D + dv] = (bf16)(osum / ll);
+      continue;
+    }
+    float* dst = part + (bh * n_splits + split) * (D + 2);
+    dst[2 + dv] = osum;
+    if (dv == 0) {
+      dst[0] = mh;
+      dst[1] = ll;
+    }
+  }
+}
+
 // Merge the splits of one (sequence, head): common maximum, weighted sums, in the order of the
 // splits.  (A second kernel and not the last workgroup of the first: what other XCDs wrote is
 // only sure to be seen across a kernel boundary or after a device-wide fence, and that fence
@@ -661,12 +875,41 @@ static int launch_prefill(const bf16* q, const bf16* k_new, const bf16* vt_new, 
   return 0;
 }
 
+// which decode kernel serves head sizes 64, 128 and 256 (tests and measurements may switch)
+static bool decode_through_lds = true;
+constexpr int DR_MAX_PAGES = 2048;      // most pages of a sequence that the kernel through LDS keeps the ids of (8 KB)
+
 template <int DPAD>
 static int launch_decode(const bf16* q, const bf16* pages, const int* table, int table_stride,
                          int ring_pages, const int* row_pos, int B, int nq, int nkv, int d, int window,
                          float scale, int n_splits, float* part, bf16* out, hipStream_t st) {
   const int g = nq / nkv, head_groups = (g + 15) / 16;
   dim3 grid(B * nkv * head_groups, n_splits);
+  if constexpr (DPAD == 64 || DPAD == 128 || DPAD == 256) {
+    if (d == DPAD && decode_through_lds && table_stride <= DR_MAX_PAGES) {
+      constexpr int NS = DPAD == 64 ? 4 : 2;         // 64 KB of LDS, two workgroups a compute unit; heads of 256: 128 KB, one
+      constexpr int LDS = NS * PAGE * DPAD * 4 + DR_MAX_PAGES * 4;              // the ring, and the page ids of a split
+      static bool raised = false;
+      if (!raised) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_decode_ring_kernel<DPAD, NS>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+        if (e != hipSuccess) {
+          set_error("attn_decode: cannot have %d bytes of LDS: %s", LDS, hipGetErrorString(e));
+          return 2;
+        }
+        raised = true;
+      }
+      attn_decode_ring_kernel<DPAD, NS><<<grid, DC_WAVES * 64, LDS, st>>>(q, pages, table, table_stride, ring_pages,
+                                                                          row_pos, nq, nkv, window, scale, n_splits,
+                                                                          head_groups, part, out);
+      TL_LAUNCH_CHECK("attn_decode_ring");
+      if (n_splits > 1) {
+        attn_decode_combine_kernel<<<B * nq, 64, 0, st>>>(part, n_splits, d, out);
+        TL_LAUNCH_CHECK("attn_decode_combine");
+      }
+      return 0;
+    }
+  }
   if (d == DPAD)
     attn_decode_kernel<DPAD, true><<<grid, DC_WAVES * 64, 0, st>>>(q, pages, table, table_stride, ring_pages,
                                                                     row_pos, nq, nkv, d, window, scale, n_splits,
@@ -724,6 +967,14 @@ extern "C" int tl_attn_prefill_bf16(const void* q, const void* k_new, const void
              (const bf16*)pages, table, table_stride, ring_pages, row_pos, cu_seqlens, n_cached, B,
              n_tiles, nq, nkv, d, window, scale, (bf16*)out, st);
   return 1;
+}
+
+// For tests and measurements: 1 (the default) lets head sizes 64, 128 and 256 go through the kernel that stages the
+// pages in LDS, 0 sends every head size through the kernel that reads them into registers.  Returns the old setting.
+extern "C" int tl_attn_decode_through_lds(int on) {
+  const int was = decode_through_lds ? 1 : 0;
+  decode_through_lds = on != 0;
+  return was;
 }
 
 // part: float scratch of B * nq * n_splits * (d + 2) elements (not touched when n_splits is 1)

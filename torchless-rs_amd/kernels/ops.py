@@ -744,6 +744,13 @@ def attn_decode_bf16(q, pages, table, ring_pages: int, row_pos, window: Optional
                                      int(n_splits), _p(part), _p(out), _stream()))
 
 
+def decode_through_lds(on: bool) -> bool:
+    """For tests and measurements: whether single-token attention with heads of 64, 128 or 256 goes
+    through the kernel that stages the pages in LDS (the default) or, like every other head size,
+    through the one that reads them into registers.  Returns the setting before the call."""
+    return bool(lib().tl_attn_decode_through_lds(int(bool(on))))
+
+
 def decode_groups(B: int, nq: int, nkv: int) -> int:
     """Workgroups of a decode step's attention before splitting: one per
     (sequence, KV head, 16 query heads of its group)."""
@@ -753,9 +760,18 @@ def decode_groups(B: int, nq: int, nkv: int) -> int:
 SPLIT_PAGES = 4             # fewest pages a part of the keys has
 SPLIT_COST = 0.15           # what a part more costs in the merge, in pages of a workgroup's way (8 sequences of
                             # 8 KV heads over 4,096 keys: 4 parts 3.91 ms a step, 8 parts 3.96, 6 parts 4.08)
-FULL_UNIT_HEAD = 128        # the head size from which one workgroup has enough bytes under way to keep a compute
-                            # unit streaming; smaller heads get FULL_UNIT_HEAD // head_dim workgroups a unit
-                            # (heads of 64 at batch 32: 52.5 against 55.7 us with two a unit)
+FULL_UNIT_HEAD = 128        # the kernel that reads the pages into registers: the head size from which one workgroup
+                            # has enough bytes under way to keep a compute unit streaming; smaller heads get
+                            # FULL_UNIT_HEAD // head_dim workgroups a unit (heads of 48 ...)
+LDS_DECODE_PER_UNIT = {64: 2, 128: 2, 256: 1}    # the kernel that stages the pages in LDS (these head sizes): its
+                            # workgroups hold 64 KB of LDS each (128 KB with heads of 256), so two share a unit, and
+                            # a round of workgroups is twice the units (64 sequences of 8 KV heads of 128 over 4,096
+                            # keys, 512 workgroups: 162 us with two a unit, 169 with one holding 128 KB)
+
+
+def decode_workgroups_per_unit(head_dim: int) -> int:
+    """How many workgroups of a decode step's attention a compute unit holds at a time."""
+    return LDS_DECODE_PER_UNIT.get(int(head_dim), max(1, FULL_UNIT_HEAD // max(1, int(head_dim))))
 
 
 @functools.lru_cache(maxsize=4096)
@@ -770,12 +786,13 @@ def decode_splits(B: int, nq: int, nkv: int, max_pages: int, units: int, head_di
     """Into how many parts the keys of a decode step are cut.  A compute unit streams at a rate of
     its own, so the step's attention takes as long as the unit with the most to read: rounds of
     workgroups over the `units` compute units times the pages a workgroup has, plus the merge's
-    share for every part.  Eight sequences with eight KV heads each are 4 parts (256 workgroups,
-    one a unit: 3.91 ms a step against 3.96 with 8 parts and 4.08 with 6); parts have at least
-    four pages.  With heads of 64 or less a workgroup has too few bytes under way to keep a unit
-    busy alone, and a round is two workgroups a unit (four with heads of 32: 32 sequences of 4 KV
+    share for every part; parts have at least four pages.  A round is as many workgroups as the
+    units hold at a time (`decode_workgroups_per_unit`): eight sequences with eight KV heads of 128
+    are 8 parts, 512 workgroups, two a unit (28.2 us a layer over 4,096 keys against 30.3 in 4 parts).
+    With heads of less than 64 the kernel that reads into registers has too few bytes under way to
+    keep a unit busy with one workgroup, and a round is 128 // head size a unit (32 sequences of 4 KV
     heads of 32 take 19.2 us in 4 parts, 27.2 in 2)."""
-    return _decode_splits(decode_groups(B, nq, nkv), int(max_pages), int(units) * max(1, FULL_UNIT_HEAD // max(1, int(head_dim))))
+    return _decode_splits(decode_groups(B, nq, nkv), int(max_pages), int(units) * decode_workgroups_per_unit(head_dim))
 
 
 def uses_transposed_values(dtype: torch.dtype, d: int, all_single: bool) -> bool:
