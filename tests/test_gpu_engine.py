@@ -548,6 +548,45 @@ def test_graph_replays_equal_eager_steps(zoo, dtype):
     assert rel_err(outs[0][:1], want) < TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_steps_of_several_tokens_are_captured_when_their_shape_comes_again(zoo, dtype):
+    """Chunks of the same numbers of tokens step after step (two sequences, 8 and 16 tokens a step, so that the
+    buffers laid out by pages keep their width): the first such step runs in the shared workspace, the second
+    in the graph's own, the third is captured, the rest are replays; every one gives the bits of an engine
+    that never captures, and the plain logits.  Steps of other shapes and synchronisations lie between them."""
+    from torchless_rs_amd.engine import Engine, SeqInput, load_model
+    z = zoo["C"]
+    model = load_model(z["dir"], dtype)
+    eng_g = Engine(model, max_tokens=64 * 16, max_slots=6, use_graphs=True)
+    eng_e = Engine(model, max_tokens=64 * 16, max_slots=6, use_graphs=False)
+    ids = prompts(z["cfg"]["vocab_size"], [8 * 12 + 3, 16 * 12], seed=6)
+    want = [plain.forward(z["w"], z["cfg"], p) for p in ids]
+    got = {id(eng_g): [[], []], id(eng_e): [[], []]}
+    for eng in (eng_g, eng_e):
+        eng.slots_ = [eng.alloc() for _ in ids]
+    for c in range(12):
+        outs = []
+        for eng in (eng_g, eng_e):
+            batch = [SeqInput(eng.slots_[0], ids[0][8 * c:8 * c + 8], list(range(8))),
+                     SeqInput(eng.slots_[1], ids[1][16 * c:16 * c + 16], list(range(16)))]
+            lg = eng.step(batch).clone()
+            got[id(eng)][0].append(lg[:8]); got[id(eng)][1].append(lg[8:])
+            outs.append(lg)
+            if c % 4 == 1:                                 # a step of another shape in between
+                extra = eng.alloc()
+                eng.step([SeqInput(extra, ids[1][:30 + c], [0])])
+                eng.free(extra)
+            torch.cuda.synchronize()
+        assert torch.equal(outs[0], outs[1]), c
+    several = [g for k, g in eng_g._graphs.items() if len(k) > 5]
+    assert several and any(g.graph is not None for g in several) and not eng_e._graphs      # (page tables widen once)
+    lg = eng_g.step([SeqInput(eng_g.slots_[0], ids[0][96:], [0, 1, 2])]).clone()       # the first request's last three tokens
+    got[id(eng_g)][0].append(lg)
+    assert rel_err(torch.cat(got[id(eng_g)][0]), want[0]) < TOL[dtype]
+    assert rel_err(torch.cat(got[id(eng_g)][1]), want[1]) < TOL[dtype]
+    eng_g.close(); eng_e.close()
+
+
 # ---- other storage widths and real layer sizes ------------------------------------------
 
 def test_float32_checkpoint_in_bfloat16_mode(tmp_path):

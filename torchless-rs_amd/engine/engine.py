@@ -97,7 +97,14 @@ class PackedStep:
 
     @property
     def key(self):
-        return (self.n_seqs, self.n_rows, self.n_want, self.strides)
+        """What a captured step of this shape must have in common with this one: every number that
+        reaches a kernel from the host (sizes, page-table widths and, where sequences bring several
+        tokens, how many each and the width of the buffers laid out by `aligned_columns`);
+        everything else the kernels read on the device."""
+        if self.all_single:
+            return (self.n_seqs, self.n_rows, self.n_want, self.strides)
+        return (self.n_seqs, self.n_rows, self.n_want, self.strides, tuple(int(n) for n in self.host["n_new"]),
+                int(self.host["aligned_cols"]))
 
 
 def pack_step(cache: Cache, batch: Sequence[SeqInput], vocab_size: int,
@@ -211,6 +218,7 @@ class Engine:
         self.use_graphs = use_graphs
         self.max_graphs = 32
         self._graphs: Dict[tuple, _Graph] = {}
+        self._seen: Dict[tuple, int] = {}            # shapes of steps with several tokens a sequence: times seen
         if freeze_gc:
             gc.collect()
             gc.freeze()
@@ -219,6 +227,7 @@ class Engine:
         """Give back the cache's storage, the captured graphs and the workspace now.  The engine
         cannot step afterwards; the model stays loaded."""
         self._graphs.clear()
+        self._seen.clear()
         self.workspace.clear()
         self.runs = []
         self.cache.close()
@@ -254,9 +263,15 @@ class Engine:
         that a step can be launched before the host has seen the last one's
         tokens.  Ids outside the vocabulary are read as 0.
 
-        Steps in which every sequence brings one token are launch-bound; the
-        second time a shape of such a step (batch size, page-table widths) is
-        seen it is captured as a HIP graph, and from then on replayed."""
+        Steps of few rows are launch-bound (the host needs some 15 us a kernel, a
+        step of 32 layers 5 ms whatever its rows).  Where the model's parts allow
+        (`Model.may_capture`: their own kernels only, up to 128 rows), a step in
+        which every sequence brings one token is captured as a HIP graph the second
+        time its shape (batch size, page-table widths) is seen, and from then on
+        replayed; a step in which sequences bring several tokens (a short prompt, a
+        chunk) likewise from the third time its shape is seen, the first time
+        running in the engine's shared workspace, since most such shapes never come
+        again."""
         if device_tokens is not None:
             if token_rows is None:
                 token_rows = list(range(len(batch)))
@@ -268,7 +283,7 @@ class Engine:
             raise StepError("token_rows without device_tokens")
         packed = pack_step(self.cache, batch, self.vocab_size, token_rows)
         growth = [(s.slot, len(s.tokens)) for s in batch]
-        if self.use_graphs and packed.all_single and self.model.may_capture(packed.n_rows):
+        if self.use_graphs and self.model.may_capture(packed.n_rows) and (packed.all_single or self._seen_before(packed)):
             logits = self._graph_step(packed, device_tokens)
         else:
             dev = torch.from_numpy(packed.flat).to(self.device, non_blocking=False)
@@ -278,6 +293,15 @@ class Engine:
             logits = self.model.forward(ctx, self.runs, want_rows, n_want)
         self.cache.commit(growth)
         return logits
+
+    def _seen_before(self, packed: PackedStep) -> bool:
+        """Count a shape of a step with several tokens a sequence; has it been seen before?"""
+        key = packed.key
+        n = self._seen.get(key, 0)
+        if n == 0 and len(self._seen) >= 4096:
+            self._seen.clear()
+        self._seen[key] = n + 1
+        return n > 0
 
     def _take_tokens(self, packed: PackedStep, dev: torch.Tensor, device_tokens: Optional[torch.Tensor]) -> None:
         """Fill the token section of the uploaded array from tokens on the device."""
