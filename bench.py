@@ -59,14 +59,19 @@ def main() -> int:
                     help="the baseline's configurations as it words them (unequal prompt lengths drawn from a seed, "
                          "256/128/128 new tokens, temperature 0.7 for the NeMo shape) run through the generation "
                          "loop, under 'workloads' (the default; --no-workloads skips them)")
-    ap.add_argument("--only", choices=["prefill", "decode"], default=None,
-                    help="measure one phase only and print its line to stderr (for profiling)")
+    ap.add_argument("--only", choices=["prefill", "decode", "pipes"], default=None,
+                    help="measure one phase only and print its line to stderr (for profiling); pipes: whether a "
+                         "SIMD's matrix and vector pipes overlap (ops.measure_pipes)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not served")
         return 2
 
     import torch
+    if args.only == "pipes":
+        from torchless_rs_amd.kernels import ops as _o
+        print(json.dumps({"pipes_ns_per_iteration": _o.measure_pipes("cuda:0")}), flush=True)
+        return 0
     from torchless_rs_amd import SamplingConfig, config_from_dict
     from torchless_rs_amd.engine import Engine, SeqInput, model_from_tensors
     from torchless_rs_amd.engine.generate import BatchRun

@@ -17,6 +17,9 @@
 
 namespace tl {
 
+#define TL_AS1 __attribute__((address_space(1)))      // global memory and LDS, as global_load_lds takes them
+#define TL_AS3 __attribute__((address_space(3)))
+
 __device__ __forceinline__ bf16x8 ld8(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
 __device__ __forceinline__ bf16x4 ld4(const bf16* p) { return *reinterpret_cast<const bf16x4*>(p); }
 // 16 bytes at a uniform base plus a lane's offset in bytes (32 bits: one address register)
@@ -570,8 +573,6 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
 // In LDS the 16-byte chunk c of a row lies at a swizzled place, so that the operand reads of 16
 // lanes fall on 16 groups of banks.  The compiler places no waits for such loads: the waves count
 // them (vmcnt) and meet at one barrier a page.  Partial results as attn_decode_kernel writes them.
-#define TL_AS1 __attribute__((address_space(1)))
-#define TL_AS3 __attribute__((address_space(3)))
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 
 template <int N> __device__ __forceinline__ void wait_page_loads_but() {     // until at most N loads are under way

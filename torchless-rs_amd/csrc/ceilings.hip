@@ -121,6 +121,54 @@ mfma_chain_kernel(int iters, float* __restrict__ sink) {
   if (s == 12345.678f) sink[0] = s;          // never true in practice: keeps the chain alive
 }
 
+// Do the matrix pipe and the vector pipe of a SIMD work at the same time?  Per iteration a wave issues four
+// 32x32x16 MFMAs (independent accumulators), or 32 FMAs and 8 exponentials (the vector work of a softmax), or
+// both one after the other.  ROLE 0: every wave the MFMAs only; 1: every wave the vector work only; 2: every
+// wave both; 3: the first half of a workgroup's waves the MFMAs, the second half the vector work (waves go
+// round the four SIMDs, so with 8 waves every SIMD holds one wave of each kind).
+template <int ROLE>
+__global__ void __launch_bounds__(512)
+pipes_kernel(int iters, float* __restrict__ sink) {
+  const int wave = threadIdx.x / 64, n_waves = blockDim.x / 64;
+  const bool mfmas = ROLE == 0 || ROLE == 2 || (ROLE == 3 && wave < n_waves / 2);
+  const bool vectors = ROLE == 1 || ROLE == 2 || (ROLE == 3 && wave >= n_waves / 2);
+  bf16x8 a, b;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    a[i] = (bf16)(0.001f * (threadIdx.x % 7 + i));
+    b[i] = (bf16)(0.002f * (threadIdx.x % 5 + i));
+  }
+  f32x16 acc[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[j][r] = 0.f;
+  float v[32];
+#pragma unroll
+  for (int i = 0; i < 32; ++i) v[i] = 0.001f * (float)(threadIdx.x + i);
+  const float c0 = 0.999f, c1 = 1e-4f;
+  for (int it = 0; it < iters; ++it) {
+    if (mfmas) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[j], 0, 0, 0);
+    }
+    if (vectors) {
+#pragma unroll
+      for (int i = 0; i < 32; ++i) v[i] = fmaf(v[i], c0, c1);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[i] = __builtin_amdgcn_exp2f(-v[i] * v[i]);
+    }
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s += acc[j][r];
+#pragma unroll
+  for (int i = 0; i < 32; ++i) s += v[i];
+  if (s == 12345.678f) sink[0] = s;          // never true in practice: keeps the work alive
+}
+
 }  // namespace tl
 
 using namespace tl;
@@ -167,6 +215,20 @@ int tl_stream_copy(const void* src, void* dst, size_t n_bytes, int blocks, hipSt
              "stream_copy: %zu bytes in %d blocks", n_bytes, blocks);
   stream_copy_kernel<8><<<blocks, 256, 0, st>>>((const f32x4*)src, (f32x4*)dst, n_bytes / 16);
   TL_LAUNCH_CHECK("stream_copy");
+  return 0;
+}
+
+// `blocks` workgroups of `waves` waves (4 or 8), `iters` iterations each, in one of the roles of pipes_kernel
+int tl_pipes(int role, int waves, int iters, int blocks, float* sink, hipStream_t st) {
+  TL_REQUIRE(iters > 0 && blocks > 0 && (waves == 4 || waves == 8) && role >= 0 && role <= 3,
+             "pipes: role=%d waves=%d iters=%d blocks=%d", role, waves, iters, blocks);
+  switch (role) {
+    case 0: pipes_kernel<0><<<blocks, waves * 64, 0, st>>>(iters, sink); break;
+    case 1: pipes_kernel<1><<<blocks, waves * 64, 0, st>>>(iters, sink); break;
+    case 2: pipes_kernel<2><<<blocks, waves * 64, 0, st>>>(iters, sink); break;
+    default: pipes_kernel<3><<<blocks, waves * 64, 0, st>>>(iters, sink); break;
+  }
+  TL_LAUNCH_CHECK("pipes");
   return 0;
 }
 

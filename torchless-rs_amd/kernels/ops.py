@@ -877,3 +877,28 @@ def measure_ceilings(device="cuda:0", gib: float = 8.0, shapes=None) -> dict:
     return {"hbm_read_GBs": by_shape[top], "hbm_read_shape": READ_SHAPES[top],
             "hbm_read_by_shape_GBs": {READ_SHAPES[k]: v for k, v in by_shape.items()},
             "hbm_copy_GBs": round(best_copy, 1), "mfma_bf16_TFLOPs": round(best_mfma, 1)}
+
+
+def measure_pipes(device="cuda:0", iters: int = 20000) -> dict:
+    """Whether a SIMD's matrix pipe and vector pipe work at the same time (`pipes_kernel` in
+    csrc/ceilings.hip): nanoseconds an iteration of one workgroup a compute unit, for the same work a
+    SIMD laid out in five ways.  `mfma_only`, `vector_only`: one wave a SIMD with one kind of work
+    (4 MFMAs 32x32x16, or 32 FMAs and 8 exponentials, an iteration); `both_in_one_wave`: one wave a SIMD
+    does both; `both_in_two_waves`: two waves a SIMD, each both, half the iterations (what the prefill
+    attention does); `split_roles`: two waves a SIMD, one with the MFMAs and one with the vector work."""
+    import time
+    units = compute_units(device)
+    sink = torch.zeros(16, dtype=torch.float32, device=device)
+
+    def run(role, waves, n):
+        best = float("inf")
+        for _ in range(3):
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            _check(lib().tl_pipes(role, waves, n, units, _p(sink), _stream()))
+            torch.cuda.synchronize()
+            best = min(best, time.perf_counter() - t)
+        return round(best / iters * 1e9, 2)
+
+    return {"mfma_only": run(0, 4, iters), "vector_only": run(1, 4, iters), "both_in_one_wave": run(2, 4, iters),
+            "both_in_two_waves": run(2, 8, iters // 2), "split_roles": run(3, 8, iters)}
