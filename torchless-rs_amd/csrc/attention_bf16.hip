@@ -49,28 +49,30 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
                     const bf16* __restrict__ vt_new, int vt_cols, const int* __restrict__ tile_off,
                     const bf16* __restrict__ pages, const int* __restrict__ table, int table_stride,
                     int ring_pages, const int* __restrict__ row_pos, const int* __restrict__ cu_seqlens,
-                    const int* __restrict__ n_cached, int B, int n_tiles, int cus_per_xcd, int nq, int nkv,
-                    int d, int window, float scale, bf16* __restrict__ out) {
+                    const int* __restrict__ n_cached, int B, int n_tiles, int nq, int nkv, int d,
+                    int window, float scale, bf16* __restrict__ out) {
   constexpr int KB = DPAD / 16, VB = DPAD / 32, KLD = DPAD + 8, CH = DPAD / 8;
   constexpr int PT = DPAD / 32;        // 16-byte chunks of keys, and of values, per thread and tile
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   bf16* Ks = reinterpret_cast<bf16*>(smem);          // [PF_BN][KLD]
   bf16* Vt = Ks + PF_BN * KLD;                       // [DPAD][PF_VLD]
 
-  // Which head and which block of rows.  The (head, block) pairs, heads in their order, are cut
-  // into 8 equal runs, and workgroup L takes pair L / 8 of run L % 8: workgroups are dealt round
-  // to the 8 XCDs, so an XCD works on a run of neighbouring heads, and the keys and values of
-  // their one or two KV heads stay in its L2 while the blocks of rows pass over them.  Inside a
-  // head the late blocks (most keys) come first, or last: the direction turns every `turn`
-  // heads, chosen so that the workgroups an XCD's compute units get in the first and in the
-  // second round (cus_per_xcd pairs apart) run in opposite directions and a long one meets a
-  // short one.
-  const int total = n_tiles * nq, per_xcd = (total + 7) / 8;
-  const int item = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
-  if ((int)(blockIdx.x / 8) >= per_xcd || item >= total) return;
-  const int h = item / n_tiles;
-  const int turn = max(1, cus_per_xcd / n_tiles);
-  int t = ((h / turn) % 2 == 0) ? n_tiles - 1 - item % n_tiles : item % n_tiles, b = 0;
+  // Which head and which block of rows.  Workgroups are dealt round to the 8 XCDs and start in the order
+  // of their numbers.  An XCD takes nq / 8 neighbouring heads, whose one or two KV heads stay in its L2,
+  // and goes through the step's blocks of rows from the last to the first, those heads side by side: they
+  // read the same tiles of keys at the same time, and under a causal mask the blocks with the most tiles
+  // start first and the short ones fill the compute units as they come free.  The nq % 8 heads that are
+  // left over are dealt to all XCDs in the same order, ahead of the others.
+  const int hpx = nq / 8, rest = nq % 8;
+  int h, t, b = 0;
+  if ((int)blockIdx.x < rest * n_tiles) {
+    h = 8 * hpx + (int)blockIdx.x % rest;
+    t = n_tiles - 1 - (int)blockIdx.x / rest;
+  } else {
+    const int i = (int)blockIdx.x - rest * n_tiles, idx = i / 8;
+    h = (i % 8) * hpx + idx % hpx;
+    t = n_tiles - 1 - idx / hpx;
+  }
   for (; b < B; ++b) {
     const int tiles = (cu_seqlens[b + 1] - cu_seqlens[b] + PF_BM - 1) / PF_BM;
     if (t < tiles) break;
@@ -82,13 +84,19 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
   const int row0 = cu_seqlens[b], n_new = cu_seqlens[b + 1] - row0;
   const int cached = n_cached[b];
   const int p_first = row_pos[row0];
+  const size_t head_elems = (size_t)PAGE * d, page_elems = 2 * (size_t)nkv * head_elems;
+  const int j_base = (cached / PAGE) * PAGE;
+  const bf16* vt_head = vt_new + (size_t)kvh * d * vt_cols + tile_off[b];
+  const int seq_end = p_first + n_new;               // one past the sequence's last position
+  static_assert(PF_BN == PAGE, "a tile of keys below n_cached is one page");
+  static_assert(!LEAN || 256 % CH == 0, "the short way needs every thread's chunks in one column of chunks");
+  const unsigned k_row = tid / CH, k_col = (tid % CH) * 16;                        // offsets in bytes
+  const unsigned v_row = tid / (PF_BN / 8), v_col = (tid % (PF_BN / 8)) * 16;
+
   const int qt0 = t * PF_BM;
   const int qr = qt0 + wave * 32 + l32;               // this lane's query row among the new rows
   const bool q_ok = qr < n_new;
   const int p_me = p_first + qr;
-  const size_t head_elems = (size_t)PAGE * d, page_elems = 2 * (size_t)nkv * head_elems;
-  const int j_base = (cached / PAGE) * PAGE;
-  const bf16* vt_head = vt_new + (size_t)kvh * d * vt_cols + tile_off[b];
 
   bf16x8 qreg[KB];
   {
@@ -112,13 +120,8 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
 
   bf16x8 kfetch[PT], vfetch[PT];
   // tile j0 -> registers: keys as rows [key][d], values as rows [dv][key]
-  const int seq_end = p_first + n_new;               // one past the sequence's last position
   // Whole tiles of a head that fills its padded size take the short way: the workgroup's base
   // address is uniform and a thread's chunks lie at fixed offsets from it, one stride apart.
-  static_assert(PF_BN == PAGE, "a tile of keys below n_cached is one page");
-  static_assert(!LEAN || 256 % CH == 0, "the short way needs every thread's chunks in one column of chunks");
-  const unsigned k_row = tid / CH, k_col = (tid % CH) * 16;                        // offsets in bytes
-  const unsigned v_row = tid / (PF_BN / 8), v_col = (tid % (PF_BN / 8)) * 16;
   auto fetch_lean = [&](const bf16* kbase, unsigned k_stride, const bf16* vbase, unsigned v_stride) {
     // the offsets are worked out anew for every tile (a multiply-add each): kept across the loop
     // they would take sixteen registers that the loop does not have
@@ -853,25 +856,15 @@ static int launch_prefill(const bf16* q, const bf16* k_new, const bf16* vt_new, 
     set_error("attn_prefill: %lld (head, block of rows) pairs are too many", total);
     return 1;
   }
-  const unsigned grid = (unsigned)((total + 7) / 8 * 8);
-  static int cus_per_xcd = 0;
-  if (cus_per_xcd == 0) {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 8)
-      n = 256;
-    cus_per_xcd = n / 8;
-  }
+  const unsigned grid = (unsigned)total;
   if (can_lean && d == DPAD)
     attn_prefill_kernel<DPAD, can_lean><<<grid, 256, smem, st>>>(q, k_new, vt_new, vt_cols, tile_off, pages, table,
                                                              table_stride, ring_pages, row_pos, cu_seqlens,
-                                                             n_cached, B, n_tiles, cus_per_xcd, nq, nkv, d,
-                                                             window, scale, out);
+                                                             n_cached, B, n_tiles, nq, nkv, d, window, scale, out);
   else
     attn_prefill_kernel<DPAD, false><<<grid, 256, smem, st>>>(q, k_new, vt_new, vt_cols, tile_off, pages, table,
                                                               table_stride, ring_pages, row_pos, cu_seqlens,
-                                                              n_cached, B, n_tiles, cus_per_xcd, nq, nkv, d,
-                                                              window, scale, out);
+                                                              n_cached, B, n_tiles, nq, nkv, d, window, scale, out);
   TL_LAUNCH_CHECK("attn_prefill");
   return 0;
 }
