@@ -63,6 +63,10 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
   // read the same tiles of keys at the same time, and under a causal mask the blocks with the most tiles
   // start first and the short ones fill the compute units as they come free.  The nq % 8 heads that are
   // left over are dealt to all XCDs in the same order, ahead of the others.
+  // A wave raises its priority while it issues the MFMAs of a tile's two products, so that of the two
+  // waves of a SIMD the one that feeds the matrix cores goes first and the other's exponentials fill in:
+  // up to a tenth faster where tiles are many (4 x 512 rows over 65,536 cached keys 1.85 against 2.03 ms),
+  // 3 us slower for one prompt of 2,048 tokens, whose longest chain of tiles decides.
   const int hpx = nq / 8, rest = nq % 8;
   int h, t, b = 0;
   if ((int)blockIdx.x < rest * n_tiles) {
@@ -247,6 +251,7 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
     for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
       for (int r = 0; r < 16; ++r) s[nb][r] = 0.f;
+    __builtin_amdgcn_s_setprio(1);       // see above: first among the SIMD's waves while it feeds the matrix cores
 #pragma unroll
     for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
@@ -254,6 +259,7 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
         const bf16x8 a = *reinterpret_cast<const bf16x8*>(&Ks[(nb * 32 + l32) * KLD + kb * 16 + 8 * half]);
         s[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qreg[kb], s[nb], 0, 0, 0);
       }
+    __builtin_amdgcn_s_setprio(0);
     // s[nb][r] = k.q of key j0 + 32 nb + 8 (r/4) + 4 half + r%4 with this lane's query.
     // Only tiles that cross the wave's causal edge, the window's edge or the rows' end need masks.
     const bool edge = j0 + PF_BN - 1 > pw_lo || (window > 0 && j0 <= pw_hi - window) ||
@@ -314,6 +320,7 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
     // pinned, one MFMA and its share of the next quarter's eight probabilities at a time.
 #pragma unroll
     for (int e = 0; e < 8; ++e) soft(e);
+    __builtin_amdgcn_s_setprio(1);
 #pragma unroll
     for (int qd = 0; qd < 4; ++qd) {
 #pragma unroll
@@ -325,6 +332,7 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
         }
       }
     }
+    __builtin_amdgcn_s_setprio(0);
     psum += __shfl_xor(psum, 32, WAVE);
     l += psum;
   }
