@@ -766,29 +766,44 @@ def test_qkv_rope_commit_with_row_factor(ops):
 
 # ---- the tiled copy of a weight that steps of at most 16 rows stream from ---------------------
 
-def tiled_by_formula(w, rows=None):
-    """[N/16, K/64, 2, 4, 16, 8] with (T, s, c, g, r, e) = w[rows[16 T + r], 64 s + 16 g + 8 c + e]."""
+def tiled_by_formula(w, rows=None, R=16):
+    """[ceil(N/R), K/64, 2, 4, R, 8] with (T, s, c, g, r, e) = w[rows[R T + r], 64 s + 16 g + 8 c + e]; the
+    places of the last tile behind row N are zero."""
     N, K = w.shape
     src = w if rows is None else w[rows.long()]
-    return src.view(N // 16, 16, K // 64, 4, 2, 8).permute(0, 2, 4, 3, 1, 5).contiguous()
+    T = -(-N // R)
+    if T * R != N:
+        src = torch.cat([src, torch.zeros(T * R - N, K, dtype=w.dtype, device=w.device)])
+    return src.view(T, R, K // 64, 4, 2, 8).permute(0, 2, 4, 3, 1, 5).contiguous()
 
 
-@pytest.mark.parametrize("N,K", [(16, 64), (48, 192), (4112, 320)])
+@pytest.mark.parametrize("N,K", [(16, 64), (48, 192), (4112, 320), (5120, 128)])
 def test_tile_weights(ops, N, K):
+    """Tiles as high as a workgroup's share of the channels (16 while the device has a compute unit for
+    every 16 channels, N over the units beyond), 16 for a copy with its own order of rows, any asked for."""
     w = rnd(N, K, seed=61, dtype=torch.bfloat16).to(DEV)
-    assert torch.equal(ops.tile_weights(w), tiled_by_formula(w))
+    R = ops.tile_height(N)
+    units = ops.compute_units(DEV)
+    assert R == (16 if N // 16 <= units else -(-N // (units * -(-N // (32 * units)))))
+    assert torch.equal(ops.tile_weights(w), tiled_by_formula(w, R=R))
     rows = torch.randperm(N, generator=torch.Generator().manual_seed(62)).to(torch.int32).to(DEV)
     assert torch.equal(ops.tile_weights(w, rows), tiled_by_formula(w, rows))
+    for h in (16, 17, 20, 32):
+        assert torch.equal(ops.tile_weights(w, rows, height=h), tiled_by_formula(w, rows, R=h))
     for bad in (w[:, : K - 8].contiguous(), w[: N - 8].contiguous()):
         with pytest.raises(ops.KernelError, match="multiple of 16"):
             ops.tile_weights(bad)
+    for h in (8, 15, 33):
+        with pytest.raises(ops.KernelError, match="16 to 32"):
+            ops.tile_weights(w, height=h)
     assert ops.tiles_fit(N, K) and not ops.tiles_fit(N + 8, K) and not ops.tiles_fit(N, K + 32)
 
 
 @pytest.mark.parametrize("M", [1, 7, 16])
-@pytest.mark.parametrize("N,K", [(16, 64), (48, 192), (4112, 320), (96, 4096), (8208, 128)])
+@pytest.mark.parametrize("N,K", [(16, 64), (48, 192), (4112, 320), (96, 4096), (8208, 128), (5120, 256), (6144, 128)])
 def test_products_from_the_tiled_copy_give_the_same_bits(ops, M, N, K):
-    """The same values meet in the same MFMAs in the same order, wherever they were read from."""
+    """The same values meet in the same MFMAs in the same order, wherever they were read from (the last
+    four sizes: more tiles of 16 channels than compute units, so shares and tiles of 17, 17, 20 and 24 rows)."""
     a = rnd(M, K, seed=63, dtype=torch.bfloat16).to(DEV)
     w = rnd(N, K, seed=64, dtype=torch.bfloat16).to(DEV)
     tiles = ops.tile_weights(w)
@@ -817,9 +832,12 @@ def test_products_from_the_tiled_copy_give_the_same_bits(ops, M, N, K):
     ops.gemm_bf16_norm(a, w, o1, factor=factor)
     ops.gemm_bf16_norm(a, w, o2, factor=factor, tiles=tiles)
     assert torch.equal(o1, o2)
-    # a copy of another weight's shape is refused
+    # a copy of another weight's shape is refused, and one with tiles of another height than the kernel reads
     with pytest.raises(ops.KernelError, match="tiles"):
         ops.gemm_bf16(a, w, o1, tiles=tiles.view(-1)[: tiles.numel() // 2].clone())
+    other = 24 if ops.tile_height(N) != 24 else 16
+    with pytest.raises(ops.KernelError, match="tiles of"):
+        ops.gemm_bf16(a, w, o1, tiles=ops.tile_weights(w, height=other))
 
 
 @pytest.mark.parametrize("nq,nkv,d,K,lens", [(6, 2, 48, 64, [0, 63, 64, 300]), (4, 4, 16, 320, [5]), (3, 1, 256, 128, [7, 200]),

@@ -104,21 +104,27 @@ struct RowFactors {
 
 // ----------------------------------------------------------- tiled copy ----
 // The copy of W [N, K] that the kernels for at most 16 rows stream from, when N % 16 == 0 and
-// K % 64 == 0: [N/16 tiles][K/64 steps][2 halves][4 groups][16 rows][8], where element
-// (tile T, step s, half c, group g, row r, e) is W[rows[16 T + r]][64 s + 16 g + 8 c + e]
-// (`rows`: a permutation of the rows, or null for none).  One MFMA operand of a wave (row r
-// = lane % 16, group g = lane / 16, 8 values) is then 1 KB of consecutive memory in the order of
-// the lanes, a step 2 KB, and a tile's steps follow each other.
-constexpr int TILE_STEP = 1024;        // elements of one tile's step
+// K % 64 == 0: [tiles of R rows][K/64 steps][2 halves][4 groups][R rows][8], where element
+// (tile T, step s, half c, group g, row r, e) is W[rows[R T + r]][64 s + 16 g + 8 c + e]
+// (`rows`: a permutation of the rows, or null for none; the last tile may have fewer rows than
+// places).  R is 16, or the share of channels of a workgroup of the kernel that reads the copy where
+// that is more (20 for 5,120 channels on 256 compute units): a workgroup's weights are then one run of
+// memory, and no line of it is another workgroup's as well.  With R = 16 one MFMA operand of a wave
+// (row r = lane % 16, group g = lane / 16, 8 values) is 1 KB of consecutive memory in the order of the
+// lanes, a step 2 KB, and a tile's steps follow each other.
+constexpr int TILE_STEP = 1024;        // elements of one step of a tile of 16 rows
 
 __global__ void __launch_bounds__(256)
-tile_weights_kernel(const bf16* __restrict__ W, const int* __restrict__ rows, int N, int K, bf16* __restrict__ Wt) {
+tile_weights_kernel(const bf16* __restrict__ W, const int* __restrict__ rows, int N, int K, int R,
+                    bf16* __restrict__ Wt) {
   const size_t chunks = (size_t)N * K / 8;
+  const size_t per_row = K / 8, steps = K / 64;
   for (size_t c = (size_t)blockIdx.x * 256 + threadIdx.x; c < chunks; c += (size_t)gridDim.x * 256) {
-    const int r = c % 16, g = (c / 16) % 4, half = (c / 64) % 2;
-    const size_t step = (c / 128) % (K / 64), tile = c / 128 / (K / 64);
-    const int row = rows ? rows[tile * 16 + r] : (int)(tile * 16 + r);
-    *reinterpret_cast<bf16x8*>(Wt + c * 8) = load8(W + (size_t)row * K + step * 64 + 16 * g + 8 * half);
+    const size_t n = c / per_row, kc = c % per_row;              // row of the copy, chunk of 8 along k
+    const size_t step = kc / 8, g = (kc % 8) / 2, half = kc % 2, tile = n / R, r = n % R;
+    const size_t src = rows ? (size_t)rows[n] : n;
+    *reinterpret_cast<bf16x8*>(Wt + (((((tile * steps + step) * 2 + half) * 4 + g) * R + r) * 8)) =
+        load8(W + src * K + kc * 8);
   }
 }
 
@@ -137,6 +143,7 @@ gemm_skinny_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const int li = lane % 16, kg = lane / 16;
   const int R = rows_per_wg > 0 ? rows_per_wg : 16 * NT;
+  const int TH = R > 16 ? R : 16;                     // rows of a tile of the tiled copy: the workgroup's share
   const int n0 = blockIdx.x * R;
   const int steps = (K + 63) / 64;
   const int per = (steps + SK_WAVES - 1) / SK_WAVES;
@@ -148,7 +155,7 @@ gemm_skinny_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
     const int gr = min(n0 + min(t * 16 + li, R - 1), N - 1);          // this lane's channel (clamped: never a branch)
-    wrow[t] = TILED ? W + (size_t)(gr / 16) * 16 * K + kg * 128 + (gr % 16) * 8 : W + (size_t)gr * K;
+    wrow[t] = TILED ? W + (size_t)(gr / TH) * TH * K + kg * (TH * 8) + (gr % TH) * 8 : W + (size_t)gr * K;
   }
 #pragma unroll
   for (int u = 0; u < MT; ++u) arow[u] = A + (size_t)min(u * 16 + li, M - 1) * K;
@@ -159,6 +166,7 @@ gemm_skinny_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float
 #pragma unroll
     for (int u = 0; u < MT; ++u) acc[t][u] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+  const int tile_step = TH * 64;                      // elements of one step of such a tile
   // this lane's 16 consecutive k of a step: two chunks of 8
   auto load_step = [&](int s, bf16x8 (&wv)[NT][2], bf16x8 (&av)[MT][2]) {
     const int k = s * 64 + kg * 16;
@@ -166,13 +174,13 @@ gemm_skinny_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       if constexpr (TILED && NT == 1) {
-        wv[t][0] = load8_once(wrow[t] + (size_t)s * TILE_STEP);
-        wv[t][1] = load8_once(wrow[t] + (size_t)s * TILE_STEP + TILE_STEP / 2);
+        wv[t][0] = load8_once(wrow[t] + (size_t)s * tile_step);
+        wv[t][1] = load8_once(wrow[t] + (size_t)s * tile_step + tile_step / 2);
       } else if constexpr (TILED) {
         // two tiles a workgroup (widths whose share of channels is above 16): the mark loses here, a decode
         // step of 40 layers 5,120 wide takes 6.0 instead of 6.3 ms at 16 rows without it
-        wv[t][0] = load8(wrow[t] + (size_t)s * TILE_STEP);
-        wv[t][1] = load8(wrow[t] + (size_t)s * TILE_STEP + TILE_STEP / 2);
+        wv[t][0] = load8(wrow[t] + (size_t)s * tile_step);
+        wv[t][1] = load8(wrow[t] + (size_t)s * tile_step + tile_step / 2);
       } else {
         wv[t][0] = ok0 ? load8_once(wrow[t] + k) : zero8();
         wv[t][1] = ok1 ? load8_once(wrow[t] + k + 8) : zero8();
@@ -276,14 +284,19 @@ gemm_skinny_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W, float
 }
 
 static bool tiles_fit(int N, int K) { return N % 16 == 0 && K % 64 == 0; }
+// rows of a tile of the copy that a workgroup with R channels reads
+static int tile_height(int R) { return R > 16 ? R : 16; }
 
 template <int NT, int MT, int SK_WAVES = 8>
 static int launch_skinny(const bf16* A, const bf16* W, float* C, int M, int N, int K, int epilogue,
-                         hipStream_t st, NormSplit ns = NormSplit{}, const bf16* Wt = nullptr, int rows_per_wg = 0) {
+                         hipStream_t st, NormSplit ns = NormSplit{}, const bf16* Wt = nullptr, int rows_per_wg = 0,
+                         int wt_height = 16) {
   const int R = rows_per_wg > 0 ? rows_per_wg : 16 * NT;
   const int grid = (N + R - 1) / R;
   if constexpr (MT == 1 && SK_WAVES == 8 && NT <= 2) {
     if (Wt != nullptr && tiles_fit(N, K)) {
+      TL_REQUIRE(wt_height == tile_height(R), "gemm: the tiled copy has tiles of %d rows, the kernel reads tiles of %d",
+                 wt_height, tile_height(R));
       gemm_skinny_kernel<NT, MT, SK_WAVES, true, true><<<grid, SK_WAVES * 64, 0, st>>>(A, Wt, C, M, N, K, epilogue, ns, R);
       TL_LAUNCH_CHECK("gemm_skinny");
       return 0;
@@ -322,10 +335,10 @@ static int balanced_share(int N) {
 }
 
 // the product for at most 16 rows and not many channels, in balanced shares
-static int launch_shares(const bf16* A, const bf16* W, const bf16* Wt, float* C, int M, int N, int K, int epilogue,
-                         hipStream_t st, NormSplit ns, int share) {
-  if (share <= 16) return launch_skinny<1, 1, 8>(A, W, C, M, N, K, epilogue, st, ns, Wt, share);
-  return launch_skinny<2, 1, 8>(A, W, C, M, N, K, epilogue, st, ns, Wt, share);
+static int launch_shares(const bf16* A, const bf16* W, const bf16* Wt, int wt_height, float* C, int M, int N, int K,
+                         int epilogue, hipStream_t st, NormSplit ns, int share) {
+  if (share <= 16) return launch_skinny<1, 1, 8>(A, W, C, M, N, K, epilogue, st, ns, Wt, share, wt_height);
+  return launch_skinny<2, 1, 8>(A, W, C, M, N, K, epilogue, st, ns, Wt, share, wt_height);
 }
 
 // ------------------------------------------------------- rows, 1 KB at a time ----
@@ -942,9 +955,9 @@ using namespace tl;
 
 // epilogue: 0 store float, 1 accumulate into float, 2 silu(gate) * up into bfloat16 [M, N/2]
 // (W's rows in groups of 64: 32 gate rows and their 32 up rows; N a multiple of 64).
-// Wt (or null): the tiled copy of W, see tl_gemm_bf16_norm.
-extern "C" int tl_gemm_bf16(const void* A, const void* W, const void* Wt, void* C, int M, int N, int K, int epilogue,
-                            hipStream_t st) {
+// Wt (or null): the tiled copy of W with tiles of wt_height rows, see tl_gemm_bf16_norm.
+extern "C" int tl_gemm_bf16(const void* A, const void* W, const void* Wt, int wt_height, void* C, int M, int N, int K,
+                            int epilogue, hipStream_t st) {
   TL_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm_bf16: bad sizes M=%d N=%d K=%d", M, N, K);
   TL_REQUIRE(K % 8 == 0, "gemm_bf16: K=%d must be a multiple of 8", K);
   TL_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0) && ((uintptr_t)Wt % 16 == 0),
@@ -960,7 +973,7 @@ extern "C" int tl_gemm_bf16(const void* A, const void* W, const void* Wt, void* 
   if (M <= 16) {
     if (wide && rows_fit(M, N, K)) return launch_rows(a, w, c, M, N, K, epilogue, st);
     if (wide && (M > 4 || epilogue == EPI_SILU_PAIR)) return launch_skinny<4, 1, 4>(a, w, c, M, N, K, epilogue, st);
-    return launch_shares(a, w, (const bf16*)Wt, c, M, N, K, epilogue, st, NormSplit{}, balanced_share(N));
+    return launch_shares(a, w, (const bf16*)Wt, wt_height, c, M, N, K, epilogue, st, NormSplit{}, balanced_share(N));
   }
   if (M <= 32) {
     if (wide) return launch_skinny<4, 2, 4>(a, w, c, M, N, K, epilogue, st);
@@ -1133,9 +1146,11 @@ extern "C" int tl_gemm_qkv_rope_commit(const void* A, const void* W, const void*
 // ssq_out [16][workgroups] (or all null): with the accumulate epilogue, also write
 // xt = bfloat16(C * norm_w) and the workgroups' sums of C^2; *n_groups receives the number
 // of workgroups, which is the n_part of the product that reads xt.  Wt (or null): the tiled
-// copy of W (rows in their own order), read instead of W by the kernel with 16 channels a
-// workgroup when N % 16 == 0 and K % 64 == 0.
-extern "C" int tl_gemm_bf16_norm(const void* A, const void* W, const void* Wt, void* C, int M, int N, int K, int epilogue,
+// copy of W (rows in their own order, tiles of wt_height = tl_tile_height(N) rows), read instead of W
+// by the kernel with 16 to 32 channels a workgroup when N % 16 == 0 and K % 64 == 0; a copy with tiles
+// of another height is refused.
+extern "C" int tl_gemm_bf16_norm(const void* A, const void* W, const void* Wt, int wt_height, void* C, int M, int N, int K,
+                                 int epilogue,
                                  const float* ssq_in, int n_part, float inv_h, float eps,
                                  const float* norm_w, void* xt, float* ssq_out, int ssq_capacity,
                                  int* n_groups, hipStream_t st) {
@@ -1164,17 +1179,24 @@ extern "C" int tl_gemm_bf16_norm(const void* A, const void* W, const void* Wt, v
   if (rows) return launch_rows((const bf16*)A, (const bf16*)W, (float*)C, M, N, K, epilogue, st, ns);
   if (four) return launch_skinny<4, 1, 4>((const bf16*)A, (const bf16*)W, (float*)C, M, N, K, epilogue, st, ns);
   TL_REQUIRE((uintptr_t)Wt % 16 == 0, "gemm_bf16_norm: operands must be 16-byte aligned");
-  return launch_shares((const bf16*)A, (const bf16*)W, (const bf16*)Wt, (float*)C, M, N, K, epilogue, st, ns, share);
+  return launch_shares((const bf16*)A, (const bf16*)W, (const bf16*)Wt, wt_height, (float*)C, M, N, K, epilogue, st, ns,
+                       share);
 }
 
-// Wt [N/16][K/64][2][4][16][8] = the tiled copy of W [N, K] (N % 16 == 0, K % 64 == 0) with its
-// rows taken in the order `rows` [N] (null: as they are).
-extern "C" int tl_tile_weights(const void* W, const int* rows, int N, int K, void* Wt, hipStream_t st) {
+// The rows of a tile of the copy that the products for at most 16 rows read of a weight with N rows: the
+// share of channels of a workgroup, 16 at least.
+extern "C" int tl_tile_height(int N) { return tile_height(balanced_share(N)); }
+
+// Wt [ceil(N / height)][K/64][2][4][height][8] = the tiled copy of W [N, K] (N % 16 == 0, K % 64 == 0)
+// with its rows taken in the order `rows` [N] (null: as they are).  height: 16 for the kernel that
+// has its own order of rows (tl_gemm_qkv_rope_commit), tl_tile_height(N) for the others.
+extern "C" int tl_tile_weights(const void* W, const int* rows, int N, int K, int height, void* Wt, hipStream_t st) {
   TL_REQUIRE(N > 0 && K > 0 && tiles_fit(N, K), "tile_weights: N=%d must be a multiple of 16 and K=%d of 64", N, K);
+  TL_REQUIRE(height >= 16 && height <= 32, "tile_weights: tiles of %d rows (16 to 32)", height);
   TL_REQUIRE(((uintptr_t)W % 16 == 0) && ((uintptr_t)Wt % 16 == 0), "tile_weights: operands must be 16-byte aligned");
   const size_t chunks = (size_t)N * K / 8;
   const int grid = (chunks + 255) / 256 < 8192 ? (int)((chunks + 255) / 256) : 8192;
-  tile_weights_kernel<<<grid, 256, 0, st>>>((const bf16*)W, rows, N, K, (bf16*)Wt);
+  tile_weights_kernel<<<grid, 256, 0, st>>>((const bf16*)W, rows, N, K, height, (bf16*)Wt);
   TL_LAUNCH_CHECK("tile_weights");
   return 0;
 }

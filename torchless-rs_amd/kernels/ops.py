@@ -338,19 +338,34 @@ def tiles_fit(N: int, K: int) -> bool:
     return N % 16 == 0 and K % 64 == 0
 
 
-def tile_weights(w: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+def tile_height(N: int) -> int:
+    """Rows of a tile of the tiled copy of a weight with N rows: the channels that a workgroup of the
+    products for at most 16 rows owns (16; more where the device has fewer compute units than the
+    weight has tiles of 16, so that the units get equal shares)."""
+    return int(lib().tl_tile_height(int(N)))
+
+
+def tile_weights(w: torch.Tensor, rows: Optional[torch.Tensor] = None, height: Optional[int] = None) -> torch.Tensor:
     """The copy of w [N, K] (bfloat16, N % 16 == 0, K % 64 == 0) that the products for at most
-    16 rows stream from: [N/16, K/64, 2, 4, 16, 8] with element (T, s, c, g, r, e) =
-    w[rows[16 T + r], 64 s + 16 g + 8 c + e], so that what a wave loads at a time lies in one
-    run of memory, lane after lane.  `rows` (int32 [N], on the device): a permutation of the rows; None: none."""
+    16 rows stream from: [ceil(N / R), K/64, 2, 4, R, 8] with element (T, s, c, g, r, e) =
+    w[rows[R T + r], 64 s + 16 g + 8 c + e], so that what a workgroup reads is one run of memory (and
+    with R = 16 what a wave loads at a time, lane after lane).  `rows` (int32 [N], on the device): a
+    permutation of the rows; None: none.  `height`: R; None: `tile_height(N)`, or 16 with `rows`
+    (the kernel that wants its own order reads tiles of 16).  Places of the last tile behind row N are
+    zero."""
     N, K = w.shape
     _req(w, "tile_weights.w", torch.bfloat16)
     if not tiles_fit(N, K):
         raise KernelError(f"tile_weights: N={N} must be a multiple of 16 and K={K} of 64")
     if rows is not None:
         _req(rows, "tile_weights.rows", torch.int32, (N,))
-    out = torch.empty((N // 16, K // 64, 2, 4, 16, 8), dtype=torch.bfloat16, device=w.device)
-    _check(lib().tl_tile_weights(_p(w), _p(rows), N, K, _p(out), _stream()))
+    R = int(height) if height is not None else (16 if rows is not None else tile_height(N))
+    if not 16 <= R <= 32:
+        raise KernelError(f"tile_weights: tiles of {R} rows (16 to 32)")
+    n_tiles = -(-N // R)
+    make = torch.empty if n_tiles * R == N else torch.zeros
+    out = make((n_tiles, K // 64, 2, 4, R, 8), dtype=torch.bfloat16, device=w.device)
+    _check(lib().tl_tile_weights(_p(w), _p(rows), N, K, R, _p(out), _stream()))
     return out
 
 
@@ -365,11 +380,19 @@ def qkv_tile_rows(nq: int, nkv: int, d: int, device, rotation=None) -> torch.Ten
     return torch.tensor(list(buf), dtype=torch.int32, device=device)
 
 
-def _req_tiles(tiles: Optional[torch.Tensor], N: int, K: int) -> None:
-    if tiles is not None:
-        _req(tiles, "gemm.tiles", torch.bfloat16, (N // 16, K // 64, 2, 4, 16, 8))
-        if not tiles_fit(N, K):
-            raise KernelError(f"gemm.tiles: a weight [{N}, {K}] has no tiled copy")
+def _req_tiles(tiles: Optional[torch.Tensor], N: int, K: int, height: Optional[int] = None) -> int:
+    """Check a tiled copy of a weight [N, K] (`height`: the only tile height the caller reads) and
+    return its tile height (16 where there is no copy)."""
+    if tiles is None:
+        return 16
+    if not tiles_fit(N, K):
+        raise KernelError(f"gemm.tiles: a weight [{N}, {K}] has no tiled copy")
+    R = int(tiles.shape[4]) if tiles.dim() == 6 else 0
+    if R < 16 or (height is not None and R != height):
+        raise KernelError(f"gemm.tiles: shape {tuple(tiles.shape)} is no tiled copy"
+                          + (f" with tiles of {height} rows" if height is not None else ""))
+    _req(tiles, "gemm.tiles", torch.bfloat16, (-(-N // R), K // 64, 2, 4, R, 8))
+    return R
 
 
 def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: bool = False,
@@ -385,7 +408,7 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: b
     N = w.shape[0]
     _req(a, "gemm.a", torch.bfloat16)
     _req(w, "gemm.w", torch.bfloat16, (N, K))
-    _req_tiles(tiles, N, K)
+    th = _req_tiles(tiles, N, K)
     if silu_pair:
         if accumulate or N % 64:
             raise KernelError("gemm: the paired epilogue stores, and needs N to be a multiple of 64")
@@ -395,7 +418,7 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumulate: b
         _req(out, "gemm.out", torch.float32, (M, N))
         epi = EPI_ACCUMULATE if accumulate else EPI_STORE
     if variant is None:
-        _check(lib().tl_gemm_bf16(_p(a), _p(w), _p(tiles), _p(out), M, N, K, epi, _stream()))
+        _check(lib().tl_gemm_bf16(_p(a), _p(w), _p(tiles), th, _p(out), M, N, K, epi, _stream()))
     else:
         _check(lib().tl_gemm_bf16_variant(_p(a), _p(w), _p(out), M, N, K, epi, int(variant), _stream()))
 
@@ -427,7 +450,7 @@ def gemm_bf16_norm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumula
     N = w.shape[0]
     _req(a, "gemm.a", torch.bfloat16)
     _req(w, "gemm.w", torch.bfloat16, (N, K))
-    _req_tiles(tiles, N, K)
+    th = _req_tiles(tiles, N, K)
     if silu_pair:
         if accumulate or N % 64:
             raise KernelError("gemm: the paired epilogue stores, and needs N to be a multiple of 64")
@@ -449,7 +472,7 @@ def gemm_bf16_norm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, accumula
         _req(ssq_out, "gemm.ssq_out", torch.float32)
         cap = ssq_out.numel()
     groups = ctypes.c_int(0)
-    _check(lib().tl_gemm_bf16_norm(_p(a), _p(w), _p(tiles), _p(out), M, N, K, epi, _p(ssq_in), n_part,
+    _check(lib().tl_gemm_bf16_norm(_p(a), _p(w), _p(tiles), th, _p(out), M, N, K, epi, _p(ssq_in), n_part,
                                    ctypes.c_float(inv_h), ctypes.c_float(eps), _p(norm_weight), _p(xt),
                                    _p(ssq_out), cap, ctypes.byref(groups), _stream()))
     return groups.value
@@ -657,7 +680,7 @@ def qkv_rope_commit(a: torch.Tensor, w: torch.Tensor, row_pos, rotation, table, 
     n, K = a.shape
     _req(a, "qkv_rope_commit.a", torch.bfloat16)
     _req(w, "qkv_rope_commit.w", torch.bfloat16, ((nq + 2 * nkv) * d, K))
-    _req_tiles(tiles, (nq + 2 * nkv) * d, K)
+    _req_tiles(tiles, (nq + 2 * nkv) * d, K, height=16)
     _req(row_pos, "qkv_rope_commit.row_pos", torch.int32, (n,))
     rot = _rotation(rotation, d, "qkv_rope_commit")
     _req(q, "qkv_rope_commit.q", torch.bfloat16, (n, nq, d))
