@@ -2,7 +2,7 @@
 the product than the usual ones: even head sizes that are no multiple of 16 (in bfloat16 the
 attention, the rotation with its commit and the q|k|v product then leave the matrix-core kernels
 for the plain ones), heads x head size that is no multiple of 8 (the output projection leaves them
-too), `tie_word_embeddings: true`, a float16 checkpoint.  Each under all three schedules (every
+too), `tie_word_embeddings: true`, a float16 checkpoint, a width of 5,120.  Each under all three schedules (every
 request alone and whole; the last 32 tokens one by one; batches of unequal lengths whose shorter
 requests end earlier, a second batch in the same slots), in float32 and bfloat16, against the plain
 implementation.  And the default stop ids: config.json's `eos_token_id` ends a sequence through the
@@ -30,7 +30,10 @@ CASES = [("head6", 6, 4, 2, 40, 96, 130, 2, 7, False, torch.bfloat16),
          ("tied_head32", 32, 4, 2, 96, 160, 300, 2, 40, True, torch.bfloat16),
          ("tied_head40", 40, 2, 2, 80, 96, 130, 2, None, True, torch.bfloat16),
          ("float16_head64", 64, 4, 1, 128, 192, 384, 2, 100, False, torch.float16),
-         ("float16_tied_head6", 6, 4, 4, 40, 64, 130, 1, 7, True, torch.float16)]
+         ("float16_tied_head6", 6, 4, 4, 40, 64, 130, 1, 7, True, torch.float16),
+         # more tiles of 16 channels than the device has compute units: o and down in shares of 20 channels
+         # from tiled copies with tiles of 20 rows
+         ("wide5120", 64, 8, 2, 5120, 192, 300, 2, 100, False, torch.bfloat16)]
 LENS = [70, 9, 33, 1]
 
 
@@ -97,7 +100,9 @@ def test_legal_configurations_under_every_schedule(tmp_path, case):
            "hidden_size": H, "num_attention_heads": nq, "num_key_value_heads": nkv, "head_dim": d,
            "intermediate_size": I, "vocab_size": V, "rope_theta": 10000.0, "sliding_window": window,
            "rms_norm_eps": 1e-5, "max_position_embeddings": 256, "tie_word_embeddings": tie, "hidden_act": "silu"}
-    mdir = write_random_model(str(tmp_path / "m"), cfg, seed=len(name), std=0.06, norm_std=0.1, dtype=stored)
+    # weights of a size that keeps a layer's gain near one at any width (0.06 up to 600 channels), as real ones are
+    std = min(0.06, 1.5 / H ** 0.5)
+    mdir = write_random_model(str(tmp_path / "m"), cfg, seed=len(name), std=std, norm_std=0.1, dtype=stored)
     cfgd, stored_w = read_model_dir(mdir)
     assert ("lm_head.weight" in stored_w) == (not tie)
     assert all(t.dtype == stored for t in stored_w.values())
