@@ -36,7 +36,16 @@ def test_the_digest_follows_sources_and_flags(tmp_path):
     assert d0 == build._digest([str(f)], ["-O3"]) and d0 != build._digest([str(f)], ["-O2"])
     f.write_text("b")
     assert d0 != build._digest([str(f)], ["-O3"])
-    assert build.kernels_digest() != build.host_digest()
+    assert len({build.kernels_digest(), build.host_digest(), build.measure_digest()}) == 3
+
+
+def test_the_measuring_kernels_are_no_part_of_the_library_that_a_step_loads():
+    """What a model's first step compiles is what the model needs: the kernels that measure the
+    machine's ceilings have a folder and a library of their own."""
+    names = [os.path.basename(f) for f in build.sources()]
+    assert names and "ceilings.hip" not in names
+    assert [os.path.basename(f) for f in build.measure_sources()] == ["ceilings.hip"]
+    assert build.LIB_NAME != build.MEASURE_LIB_NAME
 
 
 def test_a_shared_folder_under_tmp_is_not_trusted(tmp_path):

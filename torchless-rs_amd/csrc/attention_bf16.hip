@@ -577,7 +577,7 @@ attn_decode_kernel(const bf16* __restrict__ q, const bf16* __restrict__ pages,
 // ring of stages in LDS (global_load_lds, 16 bytes a lane), several pages ahead of the matrix cores.
 // A stage is one page of one KV head: its keys [64][d] and its values [d][64], each one run of
 // memory, so that every load instruction takes 1 KB of whole lines, which may then be marked
-// non-temporal (a plain read gains a seventh from that, csrc/ceilings.hip; with the loads of
+// non-temporal (a plain read gains a seventh from that, csrc/measure/ceilings.hip; with the loads of
 // attn_decode_kernel, which take a line in halves, it loses).  The workgroup's four waves take 16
 // keys of the page each: S^T = K Q^T (16x16x32), softmax with the wave's own running maximum,
 // O^T += V^T P (16x16x16: the scores leave the first product in the second's operand layout).

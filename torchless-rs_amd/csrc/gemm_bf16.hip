@@ -28,7 +28,7 @@ namespace tl {
 
 __device__ __forceinline__ bf16x8 load8(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
 // A load of weights that a step of at most 16 rows reads once: marked non-temporal.  A plain read of a
-// large buffer reaches 6.7 to 6.95 TB/s with such loads against 6.0 without (csrc/ceilings.hip); gate|up
+// large buffer reaches 6.7 to 6.95 TB/s with such loads against 6.0 without (csrc/measure/ceilings.hip); gate|up
 // at 8 rows went from 41.6 to 38.0 us, down from 21.9 to 20.4, o from 9.0 to 8.3.  Not for the kernels
 // whose cache lines are shared between load instructions or waves (gemm_mid: a decode step at batch 64
 // 11.9 against 10.85 ms; the keys and values of decode attention: 11.56 against 10.85 ms), and the fused

@@ -1,10 +1,20 @@
 // What the machine gives to the simplest possible kernels: a read of a large buffer
 // (the ceiling of every step that is bound by reading weights and cache) and a chain of
 // independent bfloat16 MFMAs on registers (the ceiling of the products).  bench.py quotes
-// both next to the published peaks.
-#include "common.hpp"
+// both next to the published peaks.  A library of its own (libtorchless_measure.so): nothing
+// that a model's step needs is here, and a step's first call does not compile it.
+#include "../common.hpp"
+#include <stdarg.h>
 
 namespace tl {
+
+static thread_local char g_err[512] = "";
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
 
 // Every thread reads 16-byte vectors, 8 in flight, a grid-stride apart; the sums go to one
 // float a workgroup so that nothing is optimised away.
@@ -174,6 +184,8 @@ pipes_kernel(int iters, float* __restrict__ sink) {
 using namespace tl;
 
 extern "C" {
+
+const char* tl_measure_last_error() { return g_err; }
 
 // reads n_bytes (a multiple of 16) once; sink holds at least `blocks` floats
 int tl_stream_read(const void* src, size_t n_bytes, float* sink, int blocks, hipStream_t st) {

@@ -1,10 +1,12 @@
-"""Compiling the sources into two shared libraries, and loading them: the HIP
-kernels for gfx950 (`libtorchless_hip.so`, hipcc) and the host side of cache
-and step (`libtorchless_host.so`, plain C++, no GPU needed).
+"""Compiling the sources into shared libraries, and loading them: the HIP
+kernels for gfx950 that a model's step needs (`libtorchless_hip.so`, hipcc), the host
+side of cache and step (`libtorchless_host.so`, plain C++, no GPU needed) and the
+kernels that only measure the machine (`libtorchless_measure.so`, `csrc/measure/`).
 
-`build()` always compiles both.  `load()` and `load_host()` load the library
-that is there if it was built from the sources as they are now (a digest of
-sources and flags is kept beside each library), and build otherwise.  The
+`build()` always compiles all three.  `load()`, `load_host()` and `load_measure()` load
+the library that is there if it was built from the sources as they are now (a digest of
+sources and flags is kept beside each library), and build that library otherwise: a
+model's first step compiles the first two, never the third.  The
 libraries go to `csrc/_build/` inside the package; if that cannot be written
 (a read-only checkout), to a folder of the user's own (mode 0700) under the
 system's temporary directory.
@@ -26,6 +28,7 @@ from typing import List, Optional
 ARCH = "gfx950"
 LIB_NAME = "libtorchless_hip.so"
 HOST_LIB_NAME = "libtorchless_host.so"
+MEASURE_LIB_NAME = "libtorchless_measure.so"
 _CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
 HIPCC_FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
@@ -35,6 +38,7 @@ HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-Wall"]
 
 _lib: Optional[ctypes.CDLL] = None
 _host_lib: Optional[ctypes.CDLL] = None
+_measure_lib: Optional[ctypes.CDLL] = None
 _lock = threading.Lock()
 
 
@@ -48,6 +52,11 @@ def _say(msg: str) -> None:
 
 def sources() -> List[str]:
     return sorted(os.path.join(_CSRC, f) for f in os.listdir(_CSRC) if f.endswith(".hip"))
+
+
+def measure_sources() -> List[str]:
+    d = os.path.join(_CSRC, "measure")
+    return sorted(os.path.join(d, f) for f in os.listdir(d) if f.endswith(".hip"))
 
 
 def host_sources() -> List[str]:
@@ -71,6 +80,10 @@ def _digest(files: List[str], flags: List[str]) -> str:
 
 def kernels_digest() -> str:
     return _digest(sources() + _headers(), HIPCC_FLAGS)
+
+
+def measure_digest() -> str:
+    return _digest(measure_sources() + _headers(), HIPCC_FLAGS)
 
 
 def host_digest() -> str:
@@ -175,14 +188,28 @@ def _run_with_progress(cmd: List[str], what: str) -> None:
 
 
 def build(verbose: bool = True) -> str:
-    """Compile every source and link both libraries; returns the path of the kernels'."""
+    """Compile every source and link all libraries; returns the path of the kernels'."""
+    lib = build_kernels(verbose)
+    build_measure(verbose)
+    return lib
+
+
+def build_measure(verbose: bool = True) -> str:
+    """Compile the library of the measuring kernels; returns its path."""
+    return _build_hip(measure_sources(), MEASURE_LIB_NAME, measure_digest(), verbose)
+
+
+def build_kernels(verbose: bool = True) -> str:
+    """Compile the host library and the kernels that a step needs; returns the path of the kernels'."""
     build_host(verbose)
+    return _build_hip(sources(), LIB_NAME, kernels_digest(), verbose)
+
+
+def _build_hip(srcs: List[str], name: str, digest: str, verbose: bool) -> str:
     hipcc = find_hipcc()
     out_dir = next((d for d in build_dirs() if _writable_dir(d)), None)
     if out_dir is None:
         raise ExtensionMissing(f"no writable build folder among {build_dirs()}")
-    srcs = sources()
-    digest = kernels_digest()
     if verbose:
         _say(f"compiling {len(srcs)} HIP sources for {ARCH} into {out_dir}")
     objs = [os.path.join(out_dir, os.path.basename(s)[:-4] + ".o") for s in srcs]
@@ -196,7 +223,7 @@ def build(verbose: bool = True) -> str:
 
     with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as ex:
         list(ex.map(one, range(len(srcs))))
-    lib = os.path.join(out_dir, LIB_NAME)
+    lib = os.path.join(out_dir, name)
     tmp = lib + f".tmp{os.getpid()}"
     _run_with_progress([hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", *objs, "-o", tmp], "link")
     os.replace(tmp, lib)
@@ -244,12 +271,28 @@ def load() -> ctypes.CDLL:
         if _lib is not None:
             return _lib
         digest = kernels_digest()
-        path = _current_or_rebuilt(built_library(LIB_NAME, digest), digest, build, "the kernels' library")
+        path = _current_or_rebuilt(built_library(LIB_NAME, digest), digest, build_kernels, "the kernels' library")
         try:
             _lib = ctypes.CDLL(path)
         except OSError as e:
             raise ExtensionMissing(f"cannot load {path}: {e}") from None
         return _lib
+
+
+def load_measure() -> ctypes.CDLL:
+    """The library of the measuring kernels, built first if there is none."""
+    global _measure_lib
+    with _lock:
+        if _measure_lib is not None:
+            return _measure_lib
+        digest = measure_digest()
+        path = _current_or_rebuilt(built_library(MEASURE_LIB_NAME, digest), digest, build_measure,
+                                   "the measuring kernels' library")
+        try:
+            _measure_lib = ctypes.CDLL(path)
+        except OSError as e:
+            raise ExtensionMissing(f"cannot load {path}: {e}") from None
+        return _measure_lib
 
 
 def load_host() -> ctypes.CDLL:

@@ -14,7 +14,7 @@ from typing import Optional
 
 import torch
 
-from .build import load
+from .build import load, load_measure
 from .page import PAGE, require_same
 
 DT_F32, DT_BF16 = 0, 1
@@ -860,6 +860,18 @@ READ_SHAPES = {0: "8 loads a lane, a grid stride apart", 1: "16 loads a lane", 2
                7: "8 loads a wave straight into LDS", 8: "16 loads a wave straight into LDS"}
 
 
+def _measure_lib() -> ctypes.CDLL:
+    """The library of the kernels that only measure the machine (built apart from the model's)."""
+    L = load_measure()
+    L.tl_measure_last_error.restype = ctypes.c_char_p
+    return L
+
+
+def _check_measure(rc: int) -> None:
+    if rc != 0:
+        raise KernelError(_measure_lib().tl_measure_last_error().decode())
+
+
 def measure_ceilings(device="cuda:0", gib: float = 8.0, shapes=None) -> dict:
     """What the simplest kernels get on this machine: GB/s of one read of a buffer far larger
     than the caches, in every shape of `READ_SHAPES` (the best is reported with its shape, the
@@ -875,7 +887,7 @@ def measure_ceilings(device="cuda:0", gib: float = 8.0, shapes=None) -> dict:
     def timed(launch):
         torch.cuda.synchronize()
         t = time.perf_counter()
-        _check(launch())
+        _check_measure(launch())
         torch.cuda.synchronize()
         return time.perf_counter() - t
 
@@ -884,7 +896,7 @@ def measure_ceilings(device="cuda:0", gib: float = 8.0, shapes=None) -> dict:
         best = 0.0
         for blocks in (units, units * 2, units * 4, units * 8, units * 16, units * 32):
             for _ in range(3):
-                dt = timed(lambda: lib().tl_stream_read_shape(_p(buf), ctypes.c_size_t(n_bytes), _p(sink), blocks,
+                dt = timed(lambda: _measure_lib().tl_stream_read_shape(_p(buf), ctypes.c_size_t(n_bytes), _p(sink), blocks,
                                                               shape, _stream()))
                 best = max(best, n_bytes / dt / 1e9)
         by_shape[shape] = round(best, 1)
@@ -894,14 +906,14 @@ def measure_ceilings(device="cuda:0", gib: float = 8.0, shapes=None) -> dict:
     best_copy = 0.0
     for blocks in (units, units * 2, units * 4, units * 8):
         for _ in range(3):
-            dt = timed(lambda: lib().tl_stream_copy(_p(buf), _p(dst), ctypes.c_size_t(half), blocks, _stream()))
+            dt = timed(lambda: _measure_lib().tl_stream_copy(_p(buf), _p(dst), ctypes.c_size_t(half), blocks, _stream()))
             best_copy = max(best_copy, 2 * half / dt / 1e9)
     del buf, dst
     best_mfma = 0.0
     for blocks in (units, units * 2, units * 4):
         iters = 8192
         for _ in range(3):
-            dt = timed(lambda: lib().tl_mfma_chain(iters, blocks, _p(sink), _stream()))
+            dt = timed(lambda: _measure_lib().tl_mfma_chain(iters, blocks, _p(sink), _stream()))
             flop = blocks * 4 * iters * 8 * 2 * 32 * 32 * 16
             best_mfma = max(best_mfma, flop / dt / 1e12)
     return {"hbm_read_GBs": by_shape[top], "hbm_read_shape": READ_SHAPES[top],
@@ -911,7 +923,7 @@ def measure_ceilings(device="cuda:0", gib: float = 8.0, shapes=None) -> dict:
 
 def measure_pipes(device="cuda:0", iters: int = 20000) -> dict:
     """Whether a SIMD's matrix pipe and vector pipe work at the same time (`pipes_kernel` in
-    csrc/ceilings.hip): nanoseconds an iteration of one workgroup a compute unit, for the same work a
+    csrc/measure/ceilings.hip): nanoseconds an iteration of one workgroup a compute unit, for the same work a
     SIMD laid out in five ways.  `mfma_only`, `vector_only`: one wave a SIMD with one kind of work
     (4 MFMAs 32x32x16, or 32 FMAs and 8 exponentials, an iteration); `both_in_one_wave`: one wave a SIMD
     does both; `both_in_two_waves`: two waves a SIMD, each both, half the iterations (what the prefill
@@ -925,7 +937,7 @@ def measure_pipes(device="cuda:0", iters: int = 20000) -> dict:
         for _ in range(3):
             torch.cuda.synchronize()
             t = time.perf_counter()
-            _check(lib().tl_pipes(role, waves, n, units, _p(sink), _stream()))
+            _check_measure(_measure_lib().tl_pipes(role, waves, n, units, _p(sink), _stream()))
             torch.cuda.synchronize()
             best = min(best, time.perf_counter() - t)
         return round(best / iters * 1e9, 2)
