@@ -266,23 +266,36 @@ class Workspace:
     def __init__(self, device):
         self.device = device
         self._bufs: Dict[str, torch.Tensor] = {}
+        self._views: Dict[tuple, torch.Tensor] = {}      # (name, dtype, shape) -> the view handed out last time
 
     def get(self, name: str, shape: Tuple[int, ...], dtype: torch.dtype, zero: bool = False) -> torch.Tensor:
         """`zero`: the buffer is zero when it is first made (not on later calls:
         for counters that their kernels leave at zero)."""
+        shape = tuple(int(s) for s in shape)
+        at = (name, dtype, shape)
+        view = self._views.get(at)
+        if view is not None:                # every layer of a step asks for the same few
+            return view
         n = 1
         for s in shape:
-            n *= int(s)
+            n *= s
         key = f"{name}:{dtype}"
         buf = self._bufs.get(key)
         if buf is None or buf.numel() < n:
             make = torch.zeros if zero else torch.empty
             buf = make(max(n, 1), dtype=dtype, device=self.device)
             self._bufs[key] = buf
-        return buf[:n].view(shape)
+            for k in [k for k in self._views if k[0] == name and k[1] == dtype]:
+                del self._views[k]          # views of the buffer that this one replaces
+        view = buf[:n].view(shape)
+        if len(self._views) > 4096:
+            self._views.clear()
+        self._views[at] = view
+        return view
 
     def clear(self) -> None:
         self._bufs.clear()
+        self._views.clear()
 
 
 @dataclass
