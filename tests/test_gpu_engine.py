@@ -171,6 +171,45 @@ def test_a_prompt_in_chunks_longer_than_the_ring(zoo, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_long_blocks_of_a_small_step_are_cut_into_runs(tmp_path, dtype):
+    """Few heads and a long context: the multi-token attention would run on a handful of compute units, so
+    in bfloat16 the host cuts the keys of every block with 16 tiles or more into runs for workgroups of their
+    own (`ops.prefill_cuts`).  A prompt of 1,500 tokens whole, and its last 200 as a step of their own over
+    the 1,300 that are cached, against the plain implementation; the step's layout is looked at as well."""
+    from torchless_rs_amd import write_random_model
+    from torchless_rs_amd.engine import Engine, SeqInput, load_model
+    from torchless_rs_amd.kernels import ops
+    from util import CONFIGS, INIT
+    cfg = dict(CONFIGS["B"], max_position_embeddings=2048)
+    mdir = write_random_model(str(tmp_path / "m"), cfg, dtype=torch.bfloat16, **INIT["B"])
+    cfgd, w = read_model_dir(mdir)
+    ids = prompts(cfg["vocab_size"], [1500], seed=79)[0]
+    want = plain.forward(w, cfgd, ids)
+    eng = Engine(load_model(mdir, dtype), max_tokens=64 * 26, max_slots=2)
+    for g in eng.cache.groups:
+        g.storage.fill_(float("nan"))
+    units = ops.compute_units("cuda:0")
+    nq = cfg["num_attention_heads"]
+    whole_cuts = ops.prefill_cuts([1500], [0], None, nq, units, "cuda:0")
+    tail_cuts = ops.prefill_cuts([200], [1300], None, nq, units, "cuda:0")
+    assert whole_cuts.n_cut == 12 - 7 and tail_cuts.n_cut == 2          # blocks 7 to 11 see 1,024 keys or more; both of the tail do
+    assert tail_cuts.ways == 3 and whole_cuts.ways == 3                 # the last block has 24 tiles before it: three runs of 8
+    s = eng.alloc()
+    got_whole = eng.step([SeqInput(s, ids, list(range(1500)))]).clone()
+    eng.free(s)
+    s = eng.alloc()
+    head = eng.step([SeqInput(s, ids[:1300], list(range(1300)))]).clone()
+    tail = eng.step([SeqInput(s, ids[1300:], list(range(200)))]).clone()
+    eng.free(s)
+    eng.cache.check()
+    eng.close()
+    got_cut = torch.cat([head, tail])
+    held_to_the_format(dtype, [got_whole, got_cut], [want, want], w, cfgd, [ids, ids],
+                       [[1500] * 1500, [1300] * 1300 + [200] * 200])
+    assert rel_err(got_whole, want) < TOL[dtype] and rel_err(got_cut, want) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", NAMES)
 def test_small_steps_of_several_tokens(zoo, name, dtype):
     """Two sequences together in steps of 1 to 9 tokens each: at most 16 rows a step, where a

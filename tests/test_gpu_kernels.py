@@ -485,6 +485,75 @@ def test_attention_prefill_bf16(ops, nq, nkv, d, window):
     assert rel_err(a["out"], plain_out.double()) < KTOL["bfloat16"]
 
 
+@pytest.mark.parametrize("cut_tiles", [1, 3, 8])
+@pytest.mark.parametrize("nq,nkv,d,window", SHAPES)
+def test_attention_prefill_with_long_blocks_cut_into_runs(ops, monkeypatch, nq, nkv, d, window, cut_tiles):
+    """A launch with fewer workgroups than compute units: the keys of a block with many tiles before it go
+    to several workgroups, a run of tiles each, and a merge; the host lays the work out.  With runs of one or
+    three tiles most blocks of the usual case are cut (cached context page-aligned and not, rows that end
+    inside a block, windows whose edge falls in any run); with the usual eight a long sequence is."""
+    lens_cached, lens_new = [0, 5, 130, 64, 200, 0], [17, 1, 3, 70, 129, 300]
+    if cut_tiles == 8:
+        lens_cached, lens_new = [900, 0, 64], [300, 1200, 5]
+    monkeypatch.setattr(ops, "PREFILL_CUT_TILES", cut_tiles)
+    a = paged_case(ops, "bfloat16", nq, nkv, d, window, lens_cached=lens_cached, lens_new=lens_new, n_pages=60)
+    blocks = [(b, t) for b, n in enumerate(lens_new) for t in range(-(-n // 128))]
+    n_tiles = len(blocks)
+
+    def tiles_of(b, t):       # the tiles of 64 keys that the block's rows see: from the window's edge of its first row to its last row
+        lo = lens_cached[b] + 128 * t
+        hi = lens_cached[b] + min(128 * (t + 1), lens_new[b]) - 1
+        first = max(0, lo - window + 1) // 64 if window else 0
+        return first, hi // 64
+
+    want_ways = {bt: min(ops.PREFILL_MAX_WAYS, (tiles_of(*bt)[1] - tiles_of(*bt)[0] + 1) // cut_tiles) for bt in blocks}
+    vt, off = transposed_values(ops, a, lens_cached, lens_new)
+    units = 2 * n_tiles * nq * ops.PREFILL_MAX_WAYS                     # room for every block in eight runs
+    cuts = ops.prefill_cuts(lens_new, lens_cached, window, nq, units, DEV)
+    if all(w < 2 for w in want_ways.values()):
+        assert cuts is None                   # no block has tiles for two runs
+        return
+    cut_blocks = {bt: w for bt, w in want_ways.items() if w >= 2}
+    assert cuts is not None and cuts.ways == max(cut_blocks.values())
+    assert {(b, t): w for b, t, w, _ in cuts.blocks.cpu().tolist()} == cut_blocks
+    items = cuts.items.cpu().tolist()
+    assert cuts.n_items == len(items) == n_tiles + sum(w - 1 for w in cut_blocks.values())
+    for bt in blocks:                         # a block's runs follow each other from its first tile to its last
+        mine = sorted((lo, w & 0xffffff, (w >> 24) & 7, ((w >> 27) & 7) + 1 if w >> 30 else 0) for b, t, lo, w in items if (b, t) == bt)
+        if bt not in cut_blocks:
+            assert mine == [(0, 0, 0, 0)]
+            continue
+        first, last = tiles_of(*bt)
+        assert [m[2] for m in mine] == list(range(cut_blocks[bt])) and all(m[3] == cut_blocks[bt] for m in mine)
+        assert mine[0][0] == first and mine[-1][1] == last + 1
+        assert all(x[1] == y[0] and x[1] - x[0] >= cut_tiles for x, y in zip(mine, mine[1:] + [(last + 1,)]))
+    n = a["q"].shape[0]
+    part = torch.full((n * nq * cuts.ways * (d + 4),), float("nan"), device=DEV)
+    ops.attn_prefill_bf16(a["q"], a["k"], vt, off, a["pages"], a["table"], a["ring"], a["row_pos"], a["cu"],
+                          a["cached"], n_tiles, window, a["scale"], a["out"], cuts=cuts, part=part)
+    assert rel_err(a["out"], a["want"]) < KTOL["bfloat16"]
+    whole = torch.empty_like(a["out"])
+    ops.attn_prefill_bf16(a["q"], a["k"], vt, off, a["pages"], a["table"], a["ring"], a["row_pos"], a["cu"],
+                          a["cached"], n_tiles, window, a["scale"], whole)
+    assert rel_err(a["out"], whole.double()) < 1e-2                 # the runs' sums meet in another order
+    cu = a["cu"].tolist()
+    rows_whole = [r for (b, t) in blocks if (b, t) not in cut_blocks
+                  for r in range(cu[b] + t * 128, cu[b] + min(lens_new[b], (t + 1) * 128))]
+    assert torch.equal(a["out"][rows_whole], whole[rows_whole])     # blocks that are not cut keep their bits
+    # the layout belongs to one step; too little room for the sums is refused
+    with pytest.raises(ops.KernelError, match="laid out for"):
+        ops.attn_prefill_bf16(a["q"], a["k"], vt, off, a["pages"], a["table"], a["ring"], a["row_pos"], a["cu"],
+                              a["cached"], n_tiles + 1, window, a["scale"], a["out"], cuts=cuts, part=part)
+    with pytest.raises(ops.KernelError, match="floats for"):
+        ops.attn_prefill_bf16(a["q"], a["k"], vt, off, a["pages"], a["table"], a["ring"], a["row_pos"], a["cu"],
+                              a["cached"], n_tiles, window, a["scale"], a["out"], cuts=cuts, part=part[:128])
+    # a launch with a workgroup for every other compute unit or more is left to the kernel's own order,
+    # and fewer units to spare mean fewer runs (a unit holds two workgroups)
+    assert ops.prefill_cuts(lens_new, lens_cached, window, nq, 2 * n_tiles * nq - 1, DEV) is None
+    fewer = ops.prefill_cuts(lens_new, lens_cached, window, nq, 2 * n_tiles * nq, DEV)
+    assert fewer is None or fewer.ways <= 4
+
+
 @pytest.mark.parametrize("through_lds", [True, False])
 @pytest.mark.parametrize("splits", [1, 3, 8])
 @pytest.mark.parametrize("nq,nkv,d,window", SHAPES)

@@ -42,6 +42,7 @@ __device__ __forceinline__ bf16x8 z8() {
 // are, so tiles are read with aligned 16-byte loads.  The next tile is
 // fetched into registers while the current one is worked on.
 constexpr int PF_BM = 128, PF_BN = 64, PF_VLD = PF_BN + 4;
+constexpr int PF_PART_HEAD = 4;       // floats before O in a half block's partial result: maximum, sum, two of padding
 
 template <int DPAD, bool LEAN>       // LEAN (d == DPAD, 256 % (DPAD / 8) == 0): whole tiles are fetched the short way
 __global__ void __launch_bounds__(256, DPAD <= 128 ? 2 : 1)
@@ -50,7 +51,8 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
                     const bf16* __restrict__ pages, const int* __restrict__ table, int table_stride,
                     int ring_pages, const int* __restrict__ row_pos, const int* __restrict__ cu_seqlens,
                     const int* __restrict__ n_cached, int B, int n_tiles, int nq, int nkv, int d,
-                    int window, float scale, bf16* __restrict__ out) {
+                    int window, float scale, bf16* __restrict__ out, const int4* __restrict__ items,
+                    float* __restrict__ part, int part_ways) {
   constexpr int KB = DPAD / 16, VB = DPAD / 32, KLD = DPAD + 8, CH = DPAD / 8;
   constexpr int PT = DPAD / 32;        // 16-byte chunks of keys, and of values, per thread and tile
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -77,12 +79,29 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
     h = (i % 8) * hpx + idx % hpx;
     t = n_tiles - 1 - idx / hpx;
   }
-  for (; b < B; ++b) {
-    const int tiles = (cu_seqlens[b + 1] - cu_seqlens[b] + PF_BM - 1) / PF_BM;
-    if (t < tiles) break;
-    t -= tiles;
+  // With `items` the host has laid the work out (n_tiles counts its entries, the dearest last): entry
+  // (sequence, block, first tile of keys, one past the last | slot << 24 | (ways - 1) << 27 | 1 << 30), or
+  // (sequence, block, 0, 0) for a whole block.  Else the block's keys are cut into `ways` runs of tiles, one workgroup each, which writes its
+  // sums to place `slot` of the block's rows in `part` for attn_prefill_merge_kernel.  A launch with fewer
+  // workgroups than the device has compute units waits for its longest chain of tiles while units stand
+  // idle, and this is what shortens it.
+  int cut_lo = 0, cut_hi = 0, slot = 0, ways = 0;
+  if (items != nullptr) {
+    const int4 it = items[t];
+    b = it.x;
+    t = it.y;
+    cut_lo = it.z;
+    cut_hi = it.w & 0xffffff;
+    slot = (it.w >> 24) & 7;
+    ways = (it.w >> 30) & 1 ? ((it.w >> 27) & 7) + 1 : 0;
+  } else {
+    for (; b < B; ++b) {
+      const int tiles = (cu_seqlens[b + 1] - cu_seqlens[b] + PF_BM - 1) / PF_BM;
+      if (t < tiles) break;
+      t -= tiles;
+    }
+    if (b == B) return;
   }
-  if (b == B) return;
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64, l32 = lane % 32, half = lane / 32;
   const int kvh = h / (nq / nkv);
   const int row0 = cu_seqlens[b], n_new = cu_seqlens[b + 1] - row0;
@@ -139,7 +158,11 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
   };
   // tiles are fetched in their order: the place in the ring of pages is counted along, and the
   // page of the tile after the next is looked up a tile early, so that no fetch waits for it
-  const int jt_first = j_lo / PF_BN;
+  int jt_first = j_lo / PF_BN, jt_last = p_hi / PF_BN;          // this workgroup's tiles of keys
+  if (ways != 0) {
+    jt_first = max(jt_first, cut_lo);
+    jt_last = min(jt_last, cut_hi - 1);
+  }
   int f_ring = jt_first % ring_pages;
   int page_nxt = ((jt_first + 1) * PF_BN <= cached) ? table[(size_t)b * table_stride + f_ring] : 0;
   auto fetch = [&](int j0) {
@@ -236,13 +259,13 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
     }
   };
 
-  fetch(jt_first * PF_BN);
-  for (int jt = jt_first; jt * PF_BN <= p_hi; ++jt) {
+  if (jt_first <= jt_last) fetch(jt_first * PF_BN);
+  for (int jt = jt_first; jt <= jt_last; ++jt) {
     const int j0 = jt * PF_BN;
     __syncthreads();                  // the previous tile has been worked on
     stash();
     __syncthreads();
-    if ((jt + 1) * PF_BN <= p_hi) fetch((jt + 1) * PF_BN);
+    if (jt < jt_last) fetch((jt + 1) * PF_BN);
     // does any query of this wave see any key of this tile?
     if (pw_lo > p_hi || j0 > pw_hi || (window > 0 && j0 + PF_BN - 1 <= pw_lo - window)) continue;
 
@@ -336,6 +359,26 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
     psum += __shfl_xor(psum, 32, WAVE);
     l += psum;
   }
+  if (ways != 0) {
+    // a run of a block's keys: running maximum, sum and unscaled O of every row, for the merge
+    if (q_ok) {
+      float* pp = part + (((size_t)(row0 + qr) * nq + h) * part_ways + slot) * (size_t)(d + PF_PART_HEAD);
+      if (half == 0) {
+        pp[0] = m;
+        pp[1] = l;
+      }
+#pragma unroll
+      for (int vb = 0; vb < VB; ++vb)
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {                 // four values in a row: 16 bytes a store
+          const int dv = vb * 32 + 8 * g4 + 4 * half;
+          if (dv < d)
+            *reinterpret_cast<f32x4*>(pp + PF_PART_HEAD + dv) =
+                f32x4{o[vb][4 * g4], o[vb][4 * g4 + 1], o[vb][4 * g4 + 2], o[vb][4 * g4 + 3]};
+        }
+    }
+    return;
+  }
   if (q_ok) {
     bf16* op = out + ((size_t)(row0 + qr) * nq + h) * d;
     const float inv = 1.0f / l;
@@ -346,6 +389,44 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
         const int dv = vb * 32 + 8 * (r / 4) + 4 * half + (r % 4);
         if (dv < d) op[dv] = (bf16)(o[vb][r] * inv);
       }
+  }
+}
+
+// The runs of a block whose keys were cut between workgroups (see `items` above) become its rows of the
+// output: common maximum, weighted sums, in the order of the runs.  A workgroup takes PF_MERGE values of
+// one (block, head): blockIdx.x = block * pieces + piece.  blocks: (sequence, block, ways, -) each.
+constexpr int PF_MERGE = 1024, PF_MAX_WAYS = 8;
+
+__global__ void __launch_bounds__(256)
+attn_prefill_merge_kernel(const float* __restrict__ part, int part_ways, const int4* __restrict__ blocks,
+                          const int* __restrict__ cu_seqlens, int pieces, int nq, int d, bf16* __restrict__ out) {
+  const int4 bt = blocks[blockIdx.x / pieces];
+  const int piece = blockIdx.x % pieces, h = blockIdx.y, ways = bt.z;
+  const int row0 = cu_seqlens[bt.x] + bt.y * PF_BM;
+  const int rows = min(PF_BM, cu_seqlens[bt.x + 1] - row0);
+  const size_t stride = (size_t)(d + PF_PART_HEAD);
+#pragma unroll
+  for (int i = 0; i < PF_MERGE / 256; ++i) {
+    const int e = piece * PF_MERGE + i * 256 + threadIdx.x;
+    const int r = e / d, dv = e % d;
+    if (r >= rows) continue;
+    const float* p = part + (((size_t)(row0 + r) * nq + h) * part_ways) * stride;
+    float ms[PF_MAX_WAYS], mm = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < PF_MAX_WAYS; ++w) {
+      ms[w] = (w < ways) ? p[w * stride] : -INFINITY;
+      mm = fmaxf(mm, ms[w]);
+    }
+    float l = 0.f, acc = 0.f;
+#pragma unroll
+    for (int w = 0; w < PF_MAX_WAYS; ++w) {
+      if (w < ways && ms[w] != -INFINITY) {
+        const float f = __expf(ms[w] - mm);
+        l += p[w * stride + 1] * f;
+        acc += p[w * stride + PF_PART_HEAD + dv] * f;
+      }
+    }
+    out[((size_t)(row0 + r) * nq + h) * d + dv] = (bf16)(acc / l);
   }
 }
 
@@ -840,7 +921,8 @@ template <int DPAD>
 static int launch_prefill(const bf16* q, const bf16* k_new, const bf16* vt_new, int vt_cols,
                           const int* tile_off, const bf16* pages, const int* table, int table_stride, int ring_pages, const int* row_pos,
                           const int* cu_seqlens, const int* n_cached, int B, int n_tiles, int nq, int nkv,
-                          int d, int window, float scale, bf16* out, hipStream_t st) {
+                          int d, int window, float scale, bf16* out, const int4* items, const int4* cut_blocks,
+                          int n_cut, float* part, int part_ways, hipStream_t st) {
   const size_t smem = ((size_t)PF_BN * (DPAD + 8) + (size_t)DPAD * PF_VLD) * sizeof(bf16);
   constexpr bool can_lean = 256 % (DPAD / 8) == 0;
   if (smem > 48 * 1024) {
@@ -868,12 +950,20 @@ static int launch_prefill(const bf16* q, const bf16* k_new, const bf16* vt_new, 
   if (can_lean && d == DPAD)
     attn_prefill_kernel<DPAD, can_lean><<<grid, 256, smem, st>>>(q, k_new, vt_new, vt_cols, tile_off, pages, table,
                                                              table_stride, ring_pages, row_pos, cu_seqlens,
-                                                             n_cached, B, n_tiles, nq, nkv, d, window, scale, out);
+                                                             n_cached, B, n_tiles, nq, nkv, d, window, scale, out,
+                                                             items, part, part_ways);
   else
     attn_prefill_kernel<DPAD, false><<<grid, 256, smem, st>>>(q, k_new, vt_new, vt_cols, tile_off, pages, table,
                                                               table_stride, ring_pages, row_pos, cu_seqlens,
-                                                              n_cached, B, n_tiles, nq, nkv, d, window, scale, out);
+                                                              n_cached, B, n_tiles, nq, nkv, d, window, scale, out,
+                                                              items, part, part_ways);
   TL_LAUNCH_CHECK("attn_prefill");
+  if (n_cut > 0) {
+    const int pieces = (PF_BM * d + PF_MERGE - 1) / PF_MERGE;
+    attn_prefill_merge_kernel<<<dim3(n_cut * pieces, nq), 256, 0, st>>>(part, part_ways, cut_blocks, cu_seqlens, pieces,
+                                                                        nq, d, out);
+    TL_LAUNCH_CHECK("attn_prefill_merge");
+  }
   return 0;
 }
 
@@ -950,9 +1040,21 @@ extern "C" int tl_attn_prefill_bf16(const void* q, const void* k_new, const void
                                     const int* tile_off, const void* pages, const int* table, int table_stride,
                                     int ring_pages, const int* row_pos, const int* cu_seqlens,
                                     const int* n_cached, int B, int n_tiles, int nq, int nkv, int d,
-                                    int window, float scale, void* out, hipStream_t st) {
+                                    int window, float scale, void* out, const int* items, const int* cut_blocks,
+                                    int n_cut, float* part, int part_ways, long long part_floats, int n_rows,
+                                    hipStream_t st) {
   TL_REQUIRE(B > 0 && n_tiles > 0 && nq > 0 && nkv > 0 && nq % nkv == 0 && nq <= 65535,
              "attn_prefill: bad sizes B=%d tiles=%d nq=%d nkv=%d", B, n_tiles, nq, nkv);
+  // items (or null): n_tiles entries laid out by the host, see the kernel; cut_blocks: the n_cut blocks
+  // (sequence, block, ways, -) whose keys several entries share; part: room for their sums, part_ways places a row
+  TL_REQUIRE(n_cut >= 0 && (n_cut == 0 || (items != nullptr && cut_blocks != nullptr && part != nullptr && n_rows > 0 &&
+                                          part_ways >= 2 && part_ways <= PF_MAX_WAYS &&
+                                          part_floats >= (long long)n_rows * nq * part_ways * (d + PF_PART_HEAD))),
+             "attn_prefill: %d blocks cut %d ways at most (2 to 8) need the entries, the blocks and %lld floats for "
+             "their sums (%lld given)", n_cut, part_ways, (long long)n_rows * nq * part_ways * (d + PF_PART_HEAD),
+             part_floats);
+  TL_REQUIRE(((uintptr_t)items % 16 == 0) && ((uintptr_t)cut_blocks % 16 == 0) && ((uintptr_t)part % 16 == 0),
+             "attn_prefill: the entries and the room for the sums must be 16-byte aligned");
   TL_REQUIRE(d >= 16 && d <= 256 && d % 16 == 0, "attn_prefill: head size %d is not served "
              "(multiples of 16 up to 256)", d);
   TL_REQUIRE(ring_pages > 0 && table_stride > 0 && window >= 0,
@@ -967,7 +1069,8 @@ extern "C" int tl_attn_prefill_bf16(const void* q, const void* k_new, const void
              vt_cols, nkv, d);
   TL_BY_DPAD(launch_prefill, (const bf16*)q, (const bf16*)k_new, (const bf16*)vt_new, vt_cols, tile_off,
              (const bf16*)pages, table, table_stride, ring_pages, row_pos, cu_seqlens, n_cached, B,
-             n_tiles, nq, nkv, d, window, scale, (bf16*)out, st);
+             n_tiles, nq, nkv, d, window, scale, (bf16*)out, reinterpret_cast<const int4*>(items),
+             reinterpret_cast<const int4*>(cut_blocks), n_cut, part, part_ways, st);
   return 1;
 }
 

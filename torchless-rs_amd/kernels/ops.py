@@ -722,12 +722,70 @@ def aligned_columns(n_cached, n_new):
     return off.tolist(), int(total)
 
 
+PREFILL_BLOCK = 128            # rows of a sequence that one workgroup of the multi-token attention takes
+PREFILL_CUT_TILES = 8          # fewest tiles of 64 keys of a run into which a block's keys are cut
+PREFILL_MAX_WAYS = 8           # most runs of a block
+
+
+class PrefillCuts:
+    """How the host lays out the work of the multi-token attention for a step with fewer workgroups than
+    the device has compute units: `items` int32 [n, 4] on the device, rows (sequence, block, first tile of
+    keys, one past the last | slot << 24 | (ways - 1) << 27 | 1 << 30) with the dearest last for one of the
+    `ways` runs into which a block's keys are cut, (sequence, block, 0, 0) for a whole block; `blocks` int32 [n_cut, 4], the (sequence,
+    block, ways, 0) that are cut; `ways`: the most runs of any block (the places a row has for its sums)."""
+
+    def __init__(self, entries, blocks, n_seqs: int, n_tiles: int, device):
+        self.n_items, self.n_cut, self.n_seqs, self.n_tiles = len(entries), len(blocks), n_seqs, n_tiles
+        self.ways = max(w for _, _, w in blocks)
+        flat = torch.tensor([v for e in entries for v in e] + [v for b in blocks for v in (*b, 0)], dtype=torch.int32)
+        dev = flat.to(device)
+        self.items = dev[:4 * len(entries)].view(-1, 4)
+        self.blocks = dev[4 * len(entries):].view(-1, 4)
+
+
+def prefill_cuts(n_new, len_before, window: Optional[int], nq: int, units: int, device) -> Optional[PrefillCuts]:
+    """The layout for a step whose sequences bring `n_new` rows after `len_before` positions, or None
+    where the kernel's own order serves.  A launch with fewer workgroups (blocks of 128 rows x heads) than
+    half the compute units leaves units idle while its longest chain of key tiles runs: then a block's keys
+    are cut into as many runs as there are units for (`PREFILL_MAX_WAYS` at most, `PREFILL_CUT_TILES` tiles
+    a run at least), each run a workgroup of its own, and a second kernel merges their sums.  (A launch that
+    fills the device gains nothing: one prompt of 2,048 tokens takes 81 us cut in two against 75.)"""
+    blocks = [(b, t) for b, n in enumerate(n_new) for t in range(-(-int(n) // PREFILL_BLOCK))]
+    if not blocks or len(blocks) * nq * 2 > units:
+        return None
+    most = min(PREFILL_MAX_WAYS, 2 * units // (len(blocks) * nq))      # (a compute unit holds two workgroups)
+    entries, cut = [], []
+    for b, t in blocks:
+        first = int(len_before[b])
+        p_lo = first + t * PREFILL_BLOCK
+        p_hi = first + min((t + 1) * PREFILL_BLOCK, int(n_new[b])) - 1
+        j_lo = max(0, p_lo - window + 1) if window else 0
+        jt_first, jt_last = j_lo // PAGE, p_hi // PAGE
+        tiles = jt_last - jt_first + 1
+        ways = min(most, tiles // PREFILL_CUT_TILES)
+        if ways < 2:
+            entries.append((tiles, (b, t, 0, 0)))
+            continue
+        cut.append((b, t, ways))
+        for w in range(ways):
+            lo, hi = jt_first + tiles * w // ways, jt_first + tiles * (w + 1) // ways
+            if hi >= 1 << 24:
+                return None                   # (a tile index beyond the entry's 24 bits)
+            entries.append((hi - lo, (b, t, lo, hi | (w << 24) | ((ways - 1) << 27) | (1 << 30))))
+    if not cut:
+        return None
+    entries.sort(key=lambda e: e[0])
+    return PrefillCuts([e[1] for e in entries], cut, len(n_new), len(blocks), device)
+
+
 def attn_prefill_bf16(q, k_new, vt_new, tile_off, pages, table, ring_pages: int, row_pos, cu_seqlens,
-                      n_cached, n_tiles: int, window: Optional[int], scale: float, out) -> None:
+                      n_cached, n_tiles: int, window: Optional[int], scale: float, out,
+                      cuts: Optional[PrefillCuts] = None, part: Optional[torch.Tensor] = None) -> None:
     """bfloat16 attention for steps with many rows per sequence.  `vt_new`:
     this step's values transposed [nkv, d, cols] at the columns that
     `aligned_columns` gives (`tile_off`).  `n_tiles`: sum over the sequences
-    of ceil(rows / 128)."""
+    of ceil(rows / 128).  `cuts` (`prefill_cuts` of this step) with `part`, float32 scratch of
+    n * nq * cuts.ways * (d + 4) elements: the keys of long blocks go to several workgroups each."""
     n, nq, d = q.shape
     nkv = pages.shape[2]
     B = n_cached.shape[0]
@@ -747,10 +805,26 @@ def attn_prefill_bf16(q, k_new, vt_new, tile_off, pages, table, ring_pages: int,
     _req(out, "attn.out", torch.bfloat16, (n, nq, d))
     if table.dim() != 2 or table.shape[0] != B:
         raise KernelError("attn.table: needs one row per sequence")
+    if cuts is None:
+        _check(lib().tl_attn_prefill_bf16(_p(q), _p(k_new), _p(vt_new), vt_new.shape[2], _p(tile_off), _p(pages),
+                                          _p(table), table.shape[1], ring_pages, _p(row_pos), _p(cu_seqlens),
+                                          _p(n_cached), B, int(n_tiles), nq, nkv, d, int(window or 0),
+                                          ctypes.c_float(scale), _p(out), None, None, 0, None, 0,
+                                          ctypes.c_longlong(0), n, _stream()))
+        return
+    if cuts.n_seqs != B or cuts.n_tiles != int(n_tiles):
+        raise KernelError(f"attn.cuts: laid out for {cuts.n_seqs} sequences and {cuts.n_tiles} blocks, "
+                          f"the step has {B} and {int(n_tiles)}")
+    if part is None:
+        raise KernelError("attn.part: blocks cut in halves need room for their sums")
+    _req(part, "attn.part", torch.float32)
+    _req(cuts.items, "attn.cuts.items", torch.int32, (cuts.n_items, 4))
+    _req(cuts.blocks, "attn.cuts.blocks", torch.int32, (cuts.n_cut, 4))
     _check(lib().tl_attn_prefill_bf16(_p(q), _p(k_new), _p(vt_new), vt_new.shape[2], _p(tile_off), _p(pages),
                                       _p(table), table.shape[1], ring_pages, _p(row_pos), _p(cu_seqlens),
-                                      _p(n_cached), B, int(n_tiles), nq, nkv, d, int(window or 0),
-                                      ctypes.c_float(scale), _p(out), _stream()))
+                                      _p(n_cached), B, cuts.n_items, nq, nkv, d, int(window or 0),
+                                      ctypes.c_float(scale), _p(out), _p(cuts.items), _p(cuts.blocks), cuts.n_cut,
+                                      _p(part), cuts.ways, ctypes.c_longlong(part.numel()), n, _stream()))
 
 
 def attn_decode_bf16(q, pages, table, ring_pages: int, row_pos, window: Optional[int], scale: float,
@@ -849,9 +923,18 @@ def attention(q, k_new, v_new, pages, table, ring_pages: int, ctx, n_cached, win
         part = ctx.workspace.get("attn_part", (n * nq * splits * (d + 2),), torch.float32)
         attn_decode_bf16(q, pages, table, ring_pages, ctx.row_pos, window, scale, splits, part, out)
     elif fast and k_new is not None and vt_new is not None:
-        n_tiles = int(sum(-(-int(x) // 128) for x in ctx.host["n_new"]))
+        n_tiles = int(sum(-(-int(x) // PREFILL_BLOCK) for x in ctx.host["n_new"]))
+        cuts = part = None
+        if n > MID_ROWS:            # (a step of fewer rows may be a captured graph, which lengths must not shape)
+            at = ("prefill_cuts", window, nq)
+            if at not in ctx.host:                               # the same for every layer of the step
+                ctx.host[at] = prefill_cuts(ctx.host["n_new"], ctx.host["len_before"], window, nq,
+                                            compute_units(q.device), q.device)
+            cuts = ctx.host[at]
+            if cuts is not None:
+                part = ctx.workspace.get("attn_prefill_part", (n * nq * cuts.ways * (d + 4),), torch.float32)
         attn_prefill_bf16(q, k_new, vt_new, ctx.tile_off, pages, table, ring_pages, ctx.row_pos,
-                          ctx.cu_seqlens, n_cached, n_tiles, window, scale, out)
+                          ctx.cu_seqlens, n_cached, n_tiles, window, scale, out, cuts=cuts, part=part)
     else:
         attn_plain(q, k_new, v_new, pages, table, ring_pages, ctx.row_seq, ctx.row_pos, ctx.cu_seqlens,
                    n_cached, window, scale, out)
