@@ -626,6 +626,49 @@ def test_steps_of_several_tokens_are_captured_when_their_shape_comes_again(zoo, 
     eng_g.close(); eng_e.close()
 
 
+def test_a_small_step_over_a_long_context_is_not_captured_but_cut_into_runs(tmp_path):
+    """A step of 100 rows may be captured as a graph when its shape comes again, but a graph's launches are
+    those of the step it was captured from: over 1,300 cached positions the attention part prefers to shape
+    its launches by the lengths (the keys of its one block of rows in runs for workgroups of their own,
+    `Part.prefers_eager`), and the step stays eager however often it comes; over 100 cached positions the
+    same step is captured at its third coming.  Both against the plain implementation."""
+    from torchless_rs_amd import write_random_model
+    from torchless_rs_amd.engine import Engine, SeqInput, load_model
+    from torchless_rs_amd.kernels import ops
+    cfg = {"architectures": ["MistralForCausalLM"], "model_type": "mistral", "num_hidden_layers": 2,
+           "hidden_size": 128, "num_attention_heads": 4, "num_key_value_heads": 2, "head_dim": 32,
+           "intermediate_size": 256, "vocab_size": 300, "rope_theta": 10000.0, "sliding_window": None,
+           "rms_norm_eps": 1e-5, "max_position_embeddings": 4096, "tie_word_embeddings": False, "hidden_act": "silu"}
+    mdir = write_random_model(str(tmp_path / "m"), cfg, seed=4, std=0.05, norm_std=0.1, dtype=torch.bfloat16)
+    cfgd, w = read_model_dir(mdir)
+    model = load_model(mdir, "bfloat16")
+    assert model.may_capture(100)
+    units = ops.compute_units("cuda:0")
+    assert ops.prefill_layout([100], [1300], None, 4, units) is not None and ops.prefill_layout([100], [100], None, 4, units) is None
+    assert model.prefers_eager([100], [1300], "cuda:0") and not model.prefers_eager([100], [100], "cuda:0")
+    eng = Engine(model, max_tokens=64 * 70, max_slots=3, use_graphs=True)
+    for cached in (1300, 100):
+        ids = prompts(cfg["vocab_size"], [cached + 100] * 3, seed=80 + cached)
+        got, slots = [], []
+        for p in ids:                                   # the same shape three times, in three slots
+            s = eng.alloc()
+            slots.append(s)
+            head = eng.step([SeqInput(s, p[:cached], list(range(cached)))]).clone()
+            tail = eng.step([SeqInput(s, p[cached:], list(range(100)))]).clone()
+            got.append(torch.cat([head, tail]))
+        several = [g for k, g in eng._graphs.items() if len(k) > 5]
+        if cached == 1300:
+            assert not several                          # never on the way to a graph
+        else:
+            assert several and any(g.graph is not None for g in several)
+        for s in slots:
+            eng.free(s)
+        exact = [plain.forward(w, cfgd, p) for p in ids]
+        held_to_the_format("bfloat16", got, exact, w, cfgd, ids, [[cached] * cached + [100] * 100] * 3, what=cached)
+    eng.cache.check()
+    eng.close()
+
+
 # ---- other storage widths and real layer sizes ------------------------------------------
 
 def test_float32_checkpoint_in_bfloat16_mode(tmp_path):

@@ -283,7 +283,10 @@ class Engine:
             raise StepError("token_rows without device_tokens")
         packed = pack_step(self.cache, batch, self.vocab_size, token_rows)
         growth = [(s.slot, len(s.tokens)) for s in batch]
-        if self.use_graphs and self.model.may_capture(packed.n_rows) and (packed.all_single or self._seen_before(packed)):
+        if (self.use_graphs and self.model.may_capture(packed.n_rows)
+                and (packed.all_single or not self.model.prefers_eager(packed.host["n_new"], packed.host["len_before"],
+                                                                        self.device))
+                and (packed.all_single or self._seen_before(packed))):
             logits = self._graph_step(packed, device_tokens)
         else:
             dev = torch.from_numpy(packed.flat).to(self.device, non_blocking=False)
@@ -334,6 +337,7 @@ class Engine:
         if g.graph is None and g.logits is not None:
             ctx, want_rows, n_want = context_from(packed, g.meta, self.cache, self.model.dtype,
                                                   self.device, g.workspace)
+            ctx.host["fixed_launches"] = True        # replays come with other lengths
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 g.logits = self.model.forward(ctx, self.runs, want_rows, n_want)
@@ -343,5 +347,6 @@ class Engine:
             return g.logits
         ctx, want_rows, n_want = context_from(packed, g.meta, self.cache, self.model.dtype, self.device,
                                               g.workspace)
+        ctx.host["fixed_launches"] = True            # the same launches as the capture that follows
         g.logits = self.model.forward(ctx, self.runs, want_rows, n_want)
         return g.logits

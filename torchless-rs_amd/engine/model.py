@@ -47,6 +47,11 @@ class Model:
         return self.loaded and all(p.may_capture(n_rows)
                                    for p in [self.embedding, self.final_norm, self.head] + self.blocks)
 
+    def prefers_eager(self, n_new, len_before, device) -> bool:
+        """Does any part want to shape its launches by this step's own lengths (see `Part.prefers_eager`)?"""
+        return any(p.prefers_eager(n_new, len_before, device)
+                   for p in [self.embedding, self.final_norm, self.head] + self.blocks)
+
     # ---- weights -----------------------------------------------------------
     def load_weights(self, source, tiled_copies: bool = True) -> None:
         """`source`: anything with names/shape/dtype/tensor (a model folder's

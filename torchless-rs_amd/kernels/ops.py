@@ -743,16 +743,32 @@ class PrefillCuts:
         self.blocks = dev[4 * len(entries):].view(-1, 4)
 
 
-def prefill_cuts(n_new, len_before, window: Optional[int], nq: int, units: int, device) -> Optional[PrefillCuts]:
-    """The layout for a step whose sequences bring `n_new` rows after `len_before` positions, or None
-    where the kernel's own order serves.  A launch with fewer workgroups (blocks of 128 rows x heads) than
-    half the compute units leaves units idle while its longest chain of key tiles runs: then a block's keys
-    are cut into as many runs as there are units for (`PREFILL_MAX_WAYS` at most, `PREFILL_CUT_TILES` tiles
-    a run at least), each run a workgroup of its own, and a second kernel merges their sums.  (A launch that
-    fills the device gains nothing: one prompt of 2,048 tokens takes 81 us cut in two against 75.)"""
-    blocks = [(b, t) for b, n in enumerate(n_new) for t in range(-(-int(n) // PREFILL_BLOCK))]
-    if not blocks or len(blocks) * nq * 2 > units:
+def prefill_layout(n_new, len_before, window: Optional[int], nq: int, units: int):
+    """The host's side of `prefill_cuts`: (entries, cut blocks, number of blocks), or None where the
+    kernel's own order serves.  A launch with fewer workgroups (blocks of 128 rows x heads) than half the
+    compute units leaves units idle while its longest chain of key tiles runs: then a block's keys are cut
+    into as many runs as there are units for (`PREFILL_MAX_WAYS` at most, `PREFILL_CUT_TILES` tiles a run at
+    least), each run a workgroup of its own, and a second kernel merges their sums.  (A launch that fills the
+    device gains nothing: one prompt of 2,048 tokens takes 81 us cut in two against 75.)"""
+    global _last_layout
+    key = (tuple(int(n) for n in n_new), tuple(int(c) for c in len_before), window, nq, units, PREFILL_CUT_TILES)
+    if _last_layout is not None and _last_layout[0] == key:       # every layer of a step asks the same
+        return _last_layout[1]
+    laid = _prefill_layout(key[0], key[1], window, nq, units)
+    _last_layout = (key, laid)
+    return laid
+
+
+_last_layout = None
+
+
+def _prefill_layout(n_new, len_before, window, nq, units):
+    n_blocks = sum(-(-n // PREFILL_BLOCK) for n in n_new)
+    if n_blocks == 0 or n_blocks * nq * 2 > units:
         return None
+    if max(c + n for c, n in zip(len_before, n_new)) <= (2 * PREFILL_CUT_TILES - 1) * PAGE:
+        return None                               # no sequence reaches into the last tile of two runs
+    blocks = [(b, t) for b, n in enumerate(n_new) for t in range(-(-n // PREFILL_BLOCK))]
     most = min(PREFILL_MAX_WAYS, 2 * units // (len(blocks) * nq))      # (a compute unit holds two workgroups)
     entries, cut = [], []
     for b, t in blocks:
@@ -775,7 +791,21 @@ def prefill_cuts(n_new, len_before, window: Optional[int], nq: int, units: int, 
     if not cut:
         return None
     entries.sort(key=lambda e: e[0])
-    return PrefillCuts([e[1] for e in entries], cut, len(n_new), len(blocks), device)
+    return [e[1] for e in entries], cut, len(blocks)
+
+
+def prefill_cuts(n_new, len_before, window: Optional[int], nq: int, units: int, device) -> Optional[PrefillCuts]:
+    """The layout (`prefill_layout`) for a step whose sequences bring `n_new` rows after `len_before`
+    positions, on the device, or None where the kernel's own order serves."""
+    laid = prefill_layout(n_new, len_before, window, nq, units)
+    if laid is None:
+        return None
+    return PrefillCuts(laid[0], laid[1], len(n_new), laid[2], device)
+
+
+def prefill_serves(dtype: torch.dtype, d: int) -> bool:
+    """Does the multi-token attention on the matrix cores serve this dtype and head size?"""
+    return dtype == torch.bfloat16 and d % 16 == 0 and 16 <= d <= 256
 
 
 def attn_prefill_bf16(q, k_new, vt_new, tile_off, pages, table, ring_pages: int, row_pos, cu_seqlens,
@@ -925,7 +955,7 @@ def attention(q, k_new, v_new, pages, table, ring_pages: int, ctx, n_cached, win
     elif fast and k_new is not None and vt_new is not None:
         n_tiles = int(sum(-(-int(x) // PREFILL_BLOCK) for x in ctx.host["n_new"]))
         cuts = part = None
-        if n > MID_ROWS:            # (a step of fewer rows may be a captured graph, which lengths must not shape)
+        if not ctx.host.get("fixed_launches"):   # (a captured graph's launches must not be shaped by lengths)
             at = ("prefill_cuts", window, nq)
             if at not in ctx.host:                               # the same for every layer of the step
                 ctx.host[at] = prefill_cuts(ctx.host["n_new"], ctx.host["len_before"], window, nq,

@@ -68,6 +68,11 @@ class AttentionMixer(Mixer):
     def may_capture(self, n_rows: int) -> bool:
         return self.qkv is not None and self.qkv.own_kernels(n_rows) and self.o.own_kernels(n_rows)
 
+    def prefers_eager(self, n_new, len_before, device) -> bool:
+        # few rows over a long context: the host cuts the keys into runs for workgroups of their own
+        return (self.qkv is not None and ops.prefill_serves(self.qkv.weight.dtype, self.d)
+                and ops.prefill_layout(n_new, len_before, self.window, self.nq, ops.compute_units(device)) is not None)
+
     def weight_specs(self) -> Dict[str, WeightSpec]:
         p, nm = self.prefix, self.names
         if nm["qkv"]:

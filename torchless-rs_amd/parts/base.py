@@ -120,6 +120,13 @@ class Part:
         the BLAS library, whose launches stay out of graphs) answers for that number."""
         return self.graph_safe
 
+    def prefers_eager(self, n_new, len_before, device) -> bool:
+        """Would this part rather shape its launches by the lengths of this very step (sequences that
+        bring `n_new` rows after `len_before` positions) than be replayed from a captured graph, whose
+        launches are those of the step it was captured from?  A step that any part prefers eager is
+        not captured."""
+        return False
+
     def weight_specs(self) -> Dict[str, WeightSpec]:
         return {}
 

@@ -43,6 +43,9 @@ class PreNormBlock(Part):
     def may_capture(self, n_rows: int) -> bool:
         return all(p.may_capture(n_rows) for p in (self.mixer, self.ffn, self.mixer_norm, self.ffn_norm))
 
+    def prefers_eager(self, n_new, len_before, device) -> bool:
+        return any(p.prefers_eager(n_new, len_before, device) for p in (self.mixer, self.ffn, self.mixer_norm, self.ffn_norm))
+
     def entry_norm(self):
         """The norm that reads the stream first, if the part behind it can take a norm cut in
         two (the block before this one may then do the norm's first half)."""
