@@ -547,11 +547,14 @@ def test_attention_prefill_with_long_blocks_cut_into_runs(ops, monkeypatch, nq, 
     with pytest.raises(ops.KernelError, match="floats for"):
         ops.attn_prefill_bf16(a["q"], a["k"], vt, off, a["pages"], a["table"], a["ring"], a["row_pos"], a["cu"],
                               a["cached"], n_tiles, window, a["scale"], a["out"], cuts=cuts, part=part[:128])
-    # a launch with a workgroup for every other compute unit or more is left to the kernel's own order,
-    # and fewer units to spare mean fewer runs (a unit holds two workgroups)
-    assert ops.prefill_cuts(lens_new, lens_cached, window, nq, 2 * n_tiles * nq - 1, DEV) is None
+    # a launch with more workgroups than compute units is left to the kernel's own order; fewer units to
+    # spare mean fewer runs (a unit holds two workgroups), and longer ones once every other unit has a workgroup
+    assert ops.prefill_cuts(lens_new, lens_cached, window, nq, n_tiles * nq - 1, DEV) is None
     fewer = ops.prefill_cuts(lens_new, lens_cached, window, nq, 2 * n_tiles * nq, DEV)
     assert fewer is None or fewer.ways <= 4
+    fuller = ops.prefill_cuts(lens_new, lens_cached, window, nq, n_tiles * nq, DEV)
+    assert fuller is None or (fuller.ways == 2 and all((w & 0xffffff) - lo >= 2 * cut_tiles
+                                                       for _, _, lo, w in fuller.items.cpu().tolist() if w >> 30))
 
 
 @pytest.mark.parametrize("through_lds", [True, False])

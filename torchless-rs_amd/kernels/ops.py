@@ -745,7 +745,7 @@ class PrefillCuts:
 
 def prefill_layout(n_new, len_before, window: Optional[int], nq: int, units: int):
     """The host's side of `prefill_cuts`: (entries, cut blocks, number of blocks), or None where the
-    kernel's own order serves.  A launch with fewer workgroups (blocks of 128 rows x heads) than half the
+    kernel's own order serves.  A launch with fewer workgroups (blocks of 128 rows x heads) than
     compute units leaves units idle while its longest chain of key tiles runs: then a block's keys are cut
     into as many runs as there are units for (`PREFILL_MAX_WAYS` at most, `PREFILL_CUT_TILES` tiles a run at
     least), each run a workgroup of its own, and a second kernel merges their sums.  (A launch that fills the
@@ -764,9 +764,12 @@ _last_layout = None
 
 def _prefill_layout(n_new, len_before, window, nq, units):
     n_blocks = sum(-(-n // PREFILL_BLOCK) for n in n_new)
-    if n_blocks == 0 or n_blocks * nq * 2 > units:
+    if n_blocks == 0 or n_blocks * nq > units:
         return None
-    if max(c + n for c, n in zip(len_before, n_new)) <= (2 * PREFILL_CUT_TILES - 1) * PAGE:
+    # with a workgroup for more than every other unit only chains twice as long are worth the merge
+    # (1,024 tokens alone, 256 workgroups of at most 16 tiles: 43.8 us with the last block cut in two against 40.3)
+    run = PREFILL_CUT_TILES * (1 if n_blocks * nq * 2 <= units else 2)
+    if max(c + n for c, n in zip(len_before, n_new)) <= (2 * run - 1) * PAGE:
         return None                               # no sequence reaches into the last tile of two runs
     blocks = [(b, t) for b, n in enumerate(n_new) for t in range(-(-n // PREFILL_BLOCK))]
     most = min(PREFILL_MAX_WAYS, 2 * units // (len(blocks) * nq))      # (a compute unit holds two workgroups)
@@ -778,7 +781,7 @@ def _prefill_layout(n_new, len_before, window, nq, units):
         j_lo = max(0, p_lo - window + 1) if window else 0
         jt_first, jt_last = j_lo // PAGE, p_hi // PAGE
         tiles = jt_last - jt_first + 1
-        ways = min(most, tiles // PREFILL_CUT_TILES)
+        ways = min(most, tiles // run)
         if ways < 2:
             entries.append((tiles, (b, t, 0, 0)))
             continue
