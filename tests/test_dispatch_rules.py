@@ -61,3 +61,62 @@ def test_rows_choose_the_kernel():
     odd = Linear(torch.zeros(96, 4104, dtype=torch.bfloat16))        # K no multiple of 128: the library from 65 rows on
     assert [odd.mid(torch.zeros(m, 4104, dtype=torch.bfloat16)) for m in (17, 64, 65)] == [True, True, False]
     assert [odd.own_kernels(m) for m in (64, 65)] == [True, False]
+
+
+def test_prefill_layout_cuts_long_blocks_of_small_launches_into_runs():
+    """The host's layout for the multi-token attention of a step with fewer workgroups than compute
+    units: every block's keys are covered once, by one entry or by consecutive runs, no run shorter
+    than the rule says, no more runs than there are units for, the dearest entries last."""
+    import itertools
+
+    def check(n_new, before, window, nq, units):
+        laid = ops.prefill_layout(n_new, before, window, nq, units)
+        blocks = [(b, t) for b, n in enumerate(n_new) for t in range(-(-n // 128))]
+        if laid is None:
+            return None
+        entries, cut, n_blocks = laid
+        assert n_blocks == len(blocks) and len(blocks) * nq <= units
+        run = ops.PREFILL_CUT_TILES * (1 if len(blocks) * nq * 2 <= units else 2)
+        most = min(ops.PREFILL_MAX_WAYS, 2 * units // (len(blocks) * nq))
+        ways_of = {(b, t): w for b, t, w in cut}
+        assert ways_of and all(2 <= w <= most for w in ways_of.values())
+        tiles_of = {}
+        for bt in blocks:
+            b, t = bt
+            lo_pos = before[b] + 128 * t
+            hi_pos = before[b] + min(128 * (t + 1), n_new[b]) - 1
+            first = max(0, lo_pos - window + 1) // 64 if window else 0
+            last = hi_pos // 64
+            tiles_of[bt] = last - first + 1
+            mine = sorted((lo, w & 0xffffff, (w >> 24) & 7, ((w >> 27) & 7) + 1 if w >> 30 else 0)
+                          for eb, et, lo, w in entries if (eb, et) == bt)
+            if bt not in ways_of:
+                assert mine == [(0, 0, 0, 0)] and (last - first + 1) // run < 2
+                continue
+            assert [m[2] for m in mine] == list(range(ways_of[bt])) and {m[3] for m in mine} == {ways_of[bt]}
+            assert mine[0][0] == first and mine[-1][1] == last + 1
+            assert all(x[1] == y[0] for x, y in zip(mine, mine[1:])) and all(m[1] - m[0] >= run for m in mine)
+            assert ways_of[bt] == min(most, (last - first + 1) // run)
+        cost = [(w & 0xffffff) - lo if w >> 30 else tiles_of[(eb, et)] for eb, et, lo, w in entries]
+        assert cost == sorted(cost)                  # workgroups start from the end of the table: the dearest first
+        assert len(entries) == len(blocks) + sum(w - 1 for w in ways_of.values())
+        return laid
+
+    # the cases of the design notes: few rows over a long context are cut, a launch that fills the device is not
+    assert check([200], [8192], None, 32, 256) is not None
+    assert check([256], [32768], None, 32, 256)[1] == [(0, 0, 8), (0, 1, 8)]
+    assert check([512], [4096], None, 32, 256)[1] == [(0, t, 4) for t in range(4)]
+    assert check([600], [35000], None, 32, 256)[1] == [(0, t, 3) for t in range(5)]      # 160 workgroups: three runs each
+    assert check([100], [32768], None, 32, 256) is not None
+    assert ops.prefill_layout([2048], [0], None, 32, 256) is None and ops.prefill_layout([1024], [0], None, 32, 256) is None
+    assert ops.prefill_layout([100], [100], None, 4, 256) is None                           # nothing long
+    assert ops.prefill_layout([128] * 9, [50000] * 9, None, 32, 256) is None                # 288 workgroups
+    assert check([128] * 8, [50000] * 8, None, 32, 256)[1] == [(b, 0, 2) for b in range(8)]
+    # a window bounds the tiles of a block: 4,096 positions are 64 tiles and the block's own two
+    assert check([128], [100000], 4096, 32, 256)[1] == [(0, 0, 8)]
+    assert ops.prefill_layout([128], [100000], 512, 32, 256) is None                        # ten tiles
+    for n_new, before, window, nq, units in itertools.product(
+            ([1], [129], [300, 5], [128, 128, 700], [1500]), ([0], [63], [5000], [70000]), (None, 70, 4096),
+            (1, 4, 32), (8, 256, 1024)):
+        before = (before * len(n_new))[:len(n_new)]
+        check(n_new, before, window, nq, units)
