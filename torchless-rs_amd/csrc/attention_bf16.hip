@@ -79,12 +79,12 @@ attn_prefill_kernel(const bf16* __restrict__ q, const bf16* __restrict__ k_new,
     h = (i % 8) * hpx + idx % hpx;
     t = n_tiles - 1 - idx / hpx;
   }
-  // With `items` the host has laid the work out (n_tiles counts its entries, the dearest last): entry
-  // (sequence, block, first tile of keys, one past the last | slot << 24 | (ways - 1) << 27 | 1 << 30), or
-  // (sequence, block, 0, 0) for a whole block.  Else the block's keys are cut into `ways` runs of tiles, one workgroup each, which writes its
-  // sums to place `slot` of the block's rows in `part` for attn_prefill_merge_kernel.  A launch with fewer
-  // workgroups than the device has compute units waits for its longest chain of tiles while units stand
-  // idle, and this is what shortens it.
+  // With `items` the host has laid the work out (n_tiles counts its entries, the dearest last).  An entry
+  // is (sequence, block, 0, 0) for a whole block, or (sequence, block, first tile of keys, one past the
+  // last | slot << 24 | (ways - 1) << 27 | 1 << 30) for one of the `ways` runs of tiles into which the
+  // block's keys are cut: a workgroup a run, which writes its sums to place `slot` of the block's rows in
+  // `part` for attn_prefill_merge_kernel.  A launch with fewer workgroups than the device has compute units
+  // waits for its longest chain of tiles while units stand idle, and this is what shortens it.
   int cut_lo = 0, cut_hi = 0, slot = 0, ways = 0;
   if (items != nullptr) {
     const int4 it = items[t];
